@@ -1,0 +1,310 @@
+"""ctypes binding of the CPU oracle (TEST INFRASTRUCTURE ONLY).
+
+Only tests, the smoke check and the benchmark's cpu_baseline leg import this module; the
+product package never does.  Functions take and return numpy arrays.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmld_oracle.so")
+
+LAYOUT_I4O4 = 1
+LAYOUT_O4I4 = 2
+LAYOUT_2D_I4O4 = 6
+PREC_F32, PREC_F32F16, PREC_F16 = 0, 1, 2
+SCALE_SCALAR, SCALE_LINEAR, SCALE_BLOCK = 0, 1, 2
+PACKED_UINT8C4, PACKED_INT8C4, PACKED_INT8C16, PACKED_UINT8C16 = 1, 2, 5, 6
+AXIS_O, AXIS_H, AXIS_W, AXIS_I = 0, 1, 2, 3
+
+
+def build(force=False):
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s"],
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+class FcParams(C.Structure):
+    _fields_ = [("m", C.c_int), ("k", C.c_int), ("n", C.c_int), ("precision", C.c_int),
+                ("weight_bits", C.c_int), ("scale_kind", C.c_int), ("groups", C.c_int),
+                ("has_zero_point", C.c_int), ("has_bias", C.c_int), ("use_fma", C.c_int),
+                ("wg_y", C.c_int), ("scalar_scale", C.c_float),
+                ("scalar_zero_point", C.c_float), ("threads", C.c_int)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.mldo_total_elements.restype = C.c_size_t
+        _lib.mldo_custom_total_elements.restype = C.c_size_t
+        _lib.mldo_f32_to_f16.restype = C.c_uint16
+        _lib.mldo_f32_to_f16.argtypes = [C.c_float]
+        _lib.mldo_f16_to_f32.restype = C.c_float
+        _lib.mldo_f16_to_f32.argtypes = [C.c_uint16]
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype):
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def div_up(a, b):
+    return (a + b - 1) // b
+
+
+# ---- fp16 ----
+def f32_to_f16_bits(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().mldo_convert_f32_f16(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
+def f16_bits_to_f32(h):
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().mldo_convert_f16_f32(_p(h), _p(out), C.c_size_t(h.size))
+    return out
+
+
+# ---- tensor layout ----
+def to_slices(x):
+    """[tokens][channels] -> slice-major [ceil(C/4)][tokens][4], zero padded."""
+    x = np.ascontiguousarray(x)
+    t, c = x.shape
+    out = np.empty((div_up(c, 4), t, 4), x.dtype)
+    lib().mldo_bhwc_to_slices(_p(x), t, c, x.dtype.itemsize, _p(out))
+    return out
+
+
+def from_slices(x, channels):
+    x = np.ascontiguousarray(x)
+    s, t, four = x.shape
+    assert four == 4 and s == div_up(channels, 4)
+    out = np.empty((t, channels), x.dtype)
+    lib().mldo_slices_to_bhwc(_p(x), t, channels, x.dtype.itemsize, _p(out))
+    return out
+
+
+# ---- packers.  weights are numpy arrays shaped (O, H, W, I) or (O, I) ----
+def _ohwi(w):
+    w = np.ascontiguousarray(w)
+    if w.ndim == 2:
+        w = w.reshape(w.shape[0], 1, 1, w.shape[1])
+    return w
+
+
+def total_elements(layout, o, h, w, i, group):
+    return lib().mldo_total_elements(layout, o, h, w, i, group)
+
+
+def rearrange_u8(w, layout, group, pad, reshape_path=False):
+    w = _ohwi(_c(w, np.uint8))
+    o, h, ww, i = w.shape
+    out = np.empty(total_elements(layout, o, h, ww, i, group), np.uint8)
+    fn = lib().mldo_rearrange_u8_reshape if reshape_path else lib().mldo_rearrange_u8
+    rc = fn(_p(w), o, h, ww, i, layout, group, C.c_uint8(pad), _p(out))
+    if rc:
+        raise ValueError("unsupported layout")
+    return out
+
+
+def rearrange_i8(w, layout, group):
+    w = _ohwi(_c(w, np.int8))
+    o, h, ww, i = w.shape
+    out = np.empty(total_elements(layout, o, h, ww, i, group), np.int8)
+    if lib().mldo_rearrange_i8(_p(w), o, h, ww, i, layout, group, _p(out)):
+        raise ValueError("unsupported layout")
+    return out
+
+
+def int8_as_uint8(w, layout, group, shift=128, pad=128):
+    w = _ohwi(_c(w, np.int8))
+    o, h, ww, i = w.shape
+    out = np.empty(total_elements(layout, o, h, ww, i, group), np.uint8)
+    if lib().mldo_int8_as_uint8(_p(w), o, h, ww, i, layout, group, shift, C.c_uint(pad), _p(out)):
+        raise ValueError("unsupported layout")
+    return out
+
+
+def int8_as_uint4(w, layout, group, shift=8, pad=8):
+    w = _ohwi(_c(w, np.int8))
+    o, h, ww, i = w.shape
+    out = np.empty(total_elements(layout, o, h, ww, i, group) // 2, np.uint8)
+    if lib().mldo_int8_as_uint4(_p(w), o, h, ww, i, layout, group, shift, C.c_uint(pad), _p(out)):
+        raise ValueError("unsupported layout")
+    return out
+
+
+def uint4_packed(src_packed, shape_ohwi, layout, group, pad=8, swap_dims=False, sum_len=None,
+                 sum_init=None):
+    src = _c(src_packed, np.uint8)
+    o, h, w, i = shape_ohwi
+    out = np.empty(total_elements(layout, o, h, w, i, group) // 2, np.uint8)
+    sum_len = o if sum_len is None else sum_len
+    sums = np.zeros(sum_len, np.int32) if sum_init is None else _c(sum_init, np.int32).copy()
+    rc = lib().mldo_uint4_packed(_p(src), o, h, w, i, layout, group, _p(out), _p(sums),
+                                 C.c_size_t(sum_len), C.c_uint(pad), int(swap_dims))
+    if rc:
+        raise NotImplementedError("Unsupported layout")
+    return out, sums
+
+
+def weights_sum_i(w):
+    w = _ohwi(_c(w, np.int8))
+    o, h, ww, i = w.shape
+    out = np.empty(o, np.int32)
+    lib().mldo_weights_sum_i(_p(w), o, h, ww, i, _p(out))
+    return out
+
+
+def rearrange_custom_i8(w, groups, pad=0):
+    """groups: list of (axis, size), fastest-varying first; size <= 0 = rest of the axis."""
+    w = _ohwi(_c(w, np.int8))
+    o, h, ww, i = w.shape
+    axes = np.array([g[0] for g in groups], np.int32)
+    sizes = np.array([g[1] for g in groups], np.int32)
+    n = lib().mldo_custom_total_elements(o, h, ww, i, _p(axes), _p(sizes), len(groups))
+    out = np.empty(n, np.int8)
+    lib().mldo_rearrange_custom_i8(_p(w), o, h, ww, i, _p(axes), _p(sizes), len(groups),
+                                   C.c_int8(pad), _p(out))
+    return out
+
+
+def scale_to_hoio4(scale_ohi):
+    """(O, I) float scales -> [I groups][ceil(O/4)][4] float, zero padded."""
+    s = _c(scale_ohi, np.float32)
+    o, i = s.shape
+    out = np.empty((div_up(o, 4), 4 * i), np.float32)
+    lib().mldo_scale_to_hoio4(_p(s), o, 1, i, _p(out))
+    # HWC (1, os, 4*i) with channel index i*4+ch -> slice-major [i][os][4]
+    return np.ascontiguousarray(out.reshape(div_up(o, 4), i, 4).transpose(1, 0, 2))
+
+
+# ---- FullyConnected ----
+def fc_kernel(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=SCALE_LINEAR,
+              scale=None, zero_point=None, bias=None, groups=1, use_fma=True, wg_y=1,
+              scalar_scale=1.0, scalar_zero_point=0.0, threads=0):
+    """act_slices / scale / zero_point / bias / result are in the tensor dtype of the
+    precision: float32 for PREC_F32, uint16 (binary16 bits) otherwise."""
+    tdt = np.float32 if precision == PREC_F32 else np.uint16
+    act = _c(act_slices, tdt)
+    assert act.size == div_up(k, 4) * m * 4
+    w = _c(weights, np.uint8)
+    p = FcParams(m, k, n, precision, weight_bits, scale_kind, groups,
+                 int(zero_point is not None or (scale_kind == SCALE_SCALAR and scalar_zero_point != 0.0)),
+                 int(bias is not None), int(use_fma), wg_y, scalar_scale, scalar_zero_point,
+                 threads)
+    sc = None if scale is None else _c(scale, tdt)
+    zp = None if zero_point is None else _c(zero_point, tdt)
+    bi = None if bias is None else _c(bias, tdt)
+    out = np.empty((div_up(n, 4), m, 4), tdt)
+    lib().mldo_fc_kernel(C.byref(p), _p(act), _p(w), _p(sc), _p(zp), _p(bi), _p(out))
+    return out
+
+
+def fc_int8_kernel(act_slices_i8, weights, m, k, n, weight_bits):
+    act = _c(act_slices_i8, np.int8)
+    w = _c(weights, np.uint8)
+    out = np.empty((div_up(n, 4), m, 4), np.int32)
+    lib().mldo_fc_int8_kernel(m, k, n, weight_bits, _p(act), _p(w), _p(out))
+    return out
+
+
+def fc_reference_f32(src, weights, bias=None):
+    src = _c(src, np.float32)
+    w = _c(weights, np.float32)
+    m, k = src.shape
+    n = w.shape[0]
+    b = None if bias is None else _c(bias, np.float32)
+    out = np.empty((m, n), np.float32)
+    lib().mldo_fc_reference_f32(m, k, n, _p(src), _p(w), _p(b), _p(out))
+    return out
+
+
+def fc_reference_i8(src, weights):
+    src = _c(src, np.int8)
+    w = _c(weights, np.int8)
+    m, k = src.shape
+    n = w.shape[0]
+    out = np.empty((m, n), np.int32)
+    lib().mldo_fc_reference_i8(m, k, n, _p(src), _p(w), _p(out))
+    return out
+
+
+def make_weights_from_int8(w, scale, zero_point=None):
+    w = _c(w, np.int8)
+    n, k = w.shape
+    s = _c(scale, np.float32).reshape(-1, 1) if np.ndim(scale) == 1 else _c(scale, np.float32)
+    z = None
+    if zero_point is not None:
+        z = _c(zero_point, np.float32).reshape(s.shape)
+    out = np.empty((n, k), np.float32)
+    lib().mldo_make_weights_from_int8(n, k, _p(w), _p(s), _p(z), s.shape[0], s.shape[1], _p(out))
+    return out
+
+
+# ---- quantization ----
+def quantize(src_slices, tokens, channels, packed_type=PACKED_INT8C4, symmetric=False,
+             calculate_sum=False, batch=1):
+    src = np.ascontiguousarray(src_slices)
+    is_f16 = src.dtype == np.uint16
+    assert is_f16 or src.dtype == np.float32
+    slices = div_up(channels, 4)
+    assert src.size == slices * tokens * 4
+    signed = packed_type in (PACKED_INT8C4, PACKED_INT8C16)
+    cdt = np.int8 if signed else np.uint8
+    if packed_type in (PACKED_INT8C16, PACKED_UINT8C16):
+        codes = np.empty((div_up(slices, 4), tokens, 16), cdt)
+    else:
+        codes = np.empty((slices, tokens, 4), cdt)
+    params = np.empty((tokens, 4), np.float32)
+    lib().mldo_quantize(tokens, channels, batch, int(is_f16), _p(src), packed_type,
+                        int(symmetric), int(calculate_sum), _p(codes), _p(params))
+    return codes, params
+
+
+def dequantize(acc_slices, params, weights_sum, weights_scale, n, k, weights_zero_point=None,
+               bias=None, dst_f16=True):
+    acc = _c(acc_slices, np.int32)
+    ns, tokens, _ = acc.shape
+    pr = _c(params, np.float32)
+
+    def padded(a, dt):
+        a = _c(a, dt).ravel()
+        out = np.zeros(ns * 4, dt)
+        out[:a.size] = a
+        return out
+    ws = padded(weights_sum, np.int32)
+    sc = padded(weights_scale, np.float32)
+    zp = None if weights_zero_point is None else padded(weights_zero_point, np.float32)
+    bdt = np.uint16 if dst_f16 else np.float32
+    bi = None if bias is None else padded(bias, bdt)
+    out = np.empty((ns, tokens, 4), bdt)
+    lib().mldo_dequantize(tokens, n, k, _p(acc), _p(pr), _p(ws), _p(sc), _p(zp), _p(bi),
+                          int(dst_f16), _p(out))
+    return out
+
+
+def dequantize_weights(weights, n, k, weight_bits, scale_bits, scale_kind=SCALE_LINEAR, groups=1,
+                       zero_point_bits=None):
+    w = _c(weights, np.uint8)
+    sc = _c(scale_bits, np.uint16)
+    zp = None if zero_point_bits is None else _c(zero_point_bits, np.uint16)
+    out = np.empty((n, k), np.uint16)
+    lib().mldo_dequantize_weights(n, k, weight_bits, _p(w), scale_kind, groups, _p(sc), _p(zp),
+                                  _p(out))
+    return out
