@@ -1,0 +1,276 @@
+/*
+ * mldhip — MI355X (gfx950) implementation of ML Drift's quantized fully-connected path.
+ *
+ * C-ABI boundary.  Everything here is `extern "C"`, plain pointers and sizes.  Each entry
+ * point names the reference interface it stands in for (paths relative to the reference
+ * checkout, ml_drift/...).
+ *
+ * Conventions
+ *  - Return value: an absl::StatusCode number (0 OK, 3 INVALID_ARGUMENT, 9
+ *    FAILED_PRECONDITION, 11 OUT_OF_RANGE, 12 UNIMPLEMENTED, 13 INTERNAL), the same codes
+ *    the reference's absl::Status carries.  mldhip_last_error() gives the message of the
+ *    last failure on the calling thread.  No exception crosses this boundary.
+ *  - Device pointers are caller-owned (the reference's tensors belong to its
+ *    InferenceContext; external weights "must be valid during life of InferenceContext",
+ *    common/gpu_model.h:83-96).  An op owns only its metadata and a small private
+ *    device workspace allocated at creation.
+ *  - Launches are asynchronous on the caller's hipStream_t (passed as void*).  Handles
+ *    are not thread-safe; creation functions are re-entrant.
+ *  - Weight shapes are OHWI with H = W = 1 for ops; the host packers accept any H, W.
+ *  - Activation / output tensors are buffers in the reference's default physical layout
+ *    PhysicalLayout1D::kDCHWBC4 = [ceil(C/4)][tokens][4] with tokens = (y*W+x)*B+b
+ *    (common/task/tensor_desc.cc:1604-1609, 1857-1860).
+ */
+#ifndef MLDHIP_H_
+#define MLDHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* absl::StatusCode numerics */
+enum {
+  MLDHIP_OK = 0,
+  MLDHIP_INVALID_ARGUMENT = 3,
+  MLDHIP_NOT_FOUND = 5,
+  MLDHIP_FAILED_PRECONDITION = 9,
+  MLDHIP_OUT_OF_RANGE = 11,
+  MLDHIP_UNIMPLEMENTED = 12,
+  MLDHIP_INTERNAL = 13
+};
+
+/* DataType, common/data_type.h:25-48 (same numbers) */
+enum {
+  MLDHIP_FLOAT16 = 1,
+  MLDHIP_FLOAT32 = 2,
+  MLDHIP_UINT8 = 5,
+  MLDHIP_INT8 = 6,
+  MLDHIP_INT32 = 10,
+  MLDHIP_UINT4 = 15
+};
+
+/* PackedType, common/data_type.h:50-60 (same numbers; the ones this path produces) */
+enum {
+  MLDHIP_PACKED_UINT8C4 = 1,
+  MLDHIP_PACKED_INT8C4 = 2,
+  MLDHIP_PACKED_INT8C16 = 5,
+  MLDHIP_PACKED_UINT8C16 = 6
+};
+
+/* WeightsLayout, common/task/weights_layout.h:27-42 (same order) */
+enum {
+  MLDHIP_LAYOUT_UNKNOWN = 0,
+  MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4 = 1,
+  MLDHIP_LAYOUT_OSPATIAL_IOGROUP_O4I4 = 2,
+  MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4 = 6,
+  MLDHIP_LAYOUT_CUSTOM_GROUPS = 7
+};
+
+/* CalculationsPrecision, common/precision.h:24-33 */
+enum { MLDHIP_PRECISION_F32 = 0, MLDHIP_PRECISION_F32_F16 = 1, MLDHIP_PRECISION_F16 = 2 };
+
+/* Axis ids for custom group lists (Axis::kOutputChannels, kHeight, kWidth, kInputChannels) */
+enum { MLDHIP_AXIS_O = 0, MLDHIP_AXIS_H = 1, MLDHIP_AXIS_W = 2, MLDHIP_AXIS_I = 3 };
+
+#define MLDHIP_MAX_CUSTOM_GROUPS 8
+
+/* WeightsDescription, common/task/weights_layout.h:44-93 (the fields this path uses).
+ * For MLDHIP_LAYOUT_CUSTOM_GROUPS the list is fastest-varying first and a size <= 0 means
+ * "the rest of that axis" (common/task/weights_conversion.cc:285-331). */
+typedef struct {
+  int32_t type;              /* MLDHIP_UINT8 / MLDHIP_UINT4 / MLDHIP_INT8 */
+  int32_t layout;            /* MLDHIP_LAYOUT_* */
+  int32_t output_group_size; /* OGroup size, for the OGroup layouts */
+  int32_t n_groups;          /* custom groups only */
+  int32_t group_axis[MLDHIP_MAX_CUSTOM_GROUPS];
+  int32_t group_size[MLDHIP_MAX_CUSTOM_GROUPS];
+} mldhip_weights_desc;
+
+const char* mldhip_last_error(void);
+const char* mldhip_version(void);
+
+/* ------------------------------------------------------------------------------------ */
+/* Weight descriptions and host packers ("weights rearrangement")                         */
+/* ------------------------------------------------------------------------------------ */
+
+/* GetFullyConnectedInt8WeightsDesc / GetFullyConnectedInt4WeightsDesc
+ * (common/kernels/fully_connected.h:185-192, .cc:1218-1246): uint8 / uint4,
+ * kOSpatialIOGroupI4O4 (buffer storage), output_group_size = ceil(o/4). */
+int mldhip_fc_int8_weights_desc(int o, int i, mldhip_weights_desc* desc);
+int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc);
+
+/* The weights layout the int8 x int8 MFMA convolution asks for, the counterpart of the
+ * conv_weights_desc that SelectConvolutionInt8 returns to the builder
+ * (common/gpu_model_builder.cc:1383-1407): signed int8, custom groups {I:16, O:rest, I:rest},
+ * i.e. [ceil(i/16)][o][16]. */
+int mldhip_conv_int8_weights_desc(int o, int i, mldhip_weights_desc* desc);
+
+/* GetTotalElementsCountForLayout (common/task/weights_conversion.cc:1015-1076) and the byte
+ * size of the packed buffer (elements * bits / 8). */
+int mldhip_total_elements(const mldhip_weights_desc* desc, int o, int h, int w, int i,
+                          size_t* elements);
+int mldhip_packed_bytes(const mldhip_weights_desc* desc, int o, int h, int w, int i,
+                        size_t* bytes);
+
+/* RearrangeWeightsInt8AsUint8 / RearrangeWeightsInt8AsUint4
+ * (common/task/weights_conversion.h, .cc:1495-1523): int8-held values + shift, reordered to
+ * desc->layout, padding elements = pad.  The reference calls them with (128, 128u) and
+ * (8, 8u) (weights_conversion.cc:1679-1684). */
+int mldhip_rearrange_int8_as_uint8(const int8_t* weights, int o, int h, int w, int i,
+                                   const mldhip_weights_desc* desc, uint8_t* dst,
+                                   size_t dst_bytes, int shift, unsigned pad);
+int mldhip_rearrange_int8_as_uint4(const int8_t* weights, int o, int h, int w, int i,
+                                   const mldhip_weights_desc* desc, uint8_t* dst,
+                                   size_t dst_bytes, int shift, unsigned pad);
+
+/* RearrangeWeights(Tensor<OHWI,kInt8>) (common/task/weights_conversion.cc:1351-1423):
+ * signed int8, pad 0; layouts I4O4, O4I4, 2D twin and custom groups. */
+int mldhip_rearrange_int8(const int8_t* weights, int o, int h, int w, int i,
+                          const mldhip_weights_desc* desc, int8_t* dst, size_t dst_bytes);
+
+/* RearrangeWeightsUInt4Packed (common/task/weights_conversion.cc:1604-1620): input is
+ * nibble-packed two's-complement OHWI (IHWO when swap_dims), low nibble = even element;
+ * also writes weights_sum_i[o] = sum_i w[o,i].  sum_len may exceed o (padding sums stay
+ * as given beyond o, entries < o are overwritten).  Layouts other than the two I4O4 ones
+ * return MLDHIP_UNIMPLEMENTED like the reference. */
+int mldhip_rearrange_uint4_packed(const uint8_t* weights, int o, int h, int w, int i,
+                                  const mldhip_weights_desc* desc, uint8_t* dst,
+                                  size_t dst_bytes, int32_t* weights_sum_i, size_t sum_len,
+                                  unsigned pad, int swap_dims);
+
+/* GetWeightsAccumulatedInputChannels (common/task/weights_conversion.cc:1584-1602) */
+int mldhip_weights_sum_i(const int8_t* weights, int o, int h, int w, int i, int32_t* sum);
+
+/* ScaleOrZeroPointToTensorDesc (common/task/tensor_desc.cc:2245-2257, 267-292): float
+ * scales OHWI(o,1,1,groups) -> the tensor the kernels read: groups == 1: linear, ceil(o/4)*4
+ * values; else [groups][ceil(o/4)][4]; element type dst_type (FLOAT16 or FLOAT32),
+ * zero padded.  dst_bytes must be groups*ceil(o/4)*4*sizeof(type). */
+int mldhip_scale_to_tensor(const float* scale, int o, int groups, int dst_type, void* dst,
+                           size_t dst_bytes);
+
+/* ------------------------------------------------------------------------------------ */
+/* Operations (node executors)                                                            */
+/* ------------------------------------------------------------------------------------ */
+
+typedef struct mldhip_op mldhip_op;
+
+/* IsFullyConnectedRecommended (common/kernels/fully_connected.cc:998-1011) restated for
+ * this device: returns 1 when `tokens` is small enough for the streaming GEMV kernels,
+ * 0 when the MFMA GEMM kernels are used.  mldhip_fc_create serves both ranges. */
+int mldhip_fc_is_recommended(int precision, int tokens);
+
+/* CreateFullyConnectedExternalWeights (common/kernels/fully_connected.h:155-161,
+ * .cc:1078-1172) and, for larger token counts, the WeightsConverter + float ConvGeneric
+ * pair the builder would emit instead (common/gpu_model_builder.cc:1110-1276), fused into
+ * one MFMA kernel.
+ *
+ * src objects, in the reference's registration order (fully_connected.cc:359-360,
+ * 1160-1170; fully_connected_util.cc:409-487):
+ *   0 "src_tensor"            activations [ceil(i/4)][tokens][4], src_type
+ *   1 "weights"               packed buffer per `weights`
+ *   2 "weights_scale"         present iff scale_o*scale_i > 1
+ *   3 "weights_zero_point"    present iff has_zero_point_tensor
+ *   4 "biases"                present iff has_bias, ceil(o/4)*4 values of dst_type
+ * (absent objects do not take an index).  dst 0 "dst_tensor": [ceil(o/4)][tokens][4].
+ *
+ * src_type INT8 selects the integer-math variant (fully_connected.cc:543-621, 874-903):
+ * no scales, dst_type must be INT32. */
+typedef struct {
+  int32_t precision;  /* MLDHIP_PRECISION_*; F32 <=> fp32 tensors, otherwise fp16 tensors */
+  int32_t src_type;   /* MLDHIP_FLOAT32 / MLDHIP_FLOAT16 / MLDHIP_INT8 */
+  int32_t dst_type;   /* MLDHIP_FLOAT32 / MLDHIP_FLOAT16 / MLDHIP_INT32 */
+  int32_t o, i;       /* ExternalWeights::shape = OHWI(o,1,1,i) */
+  mldhip_weights_desc weights; /* ExternalWeights::desc */
+  int32_t scale_o, scale_i;    /* ExternalWeights::scale_zp_shape (o, i); (1,1) = scalar */
+  float scalar_scale;          /* used when scale_o*scale_i == 1 */
+  int32_t has_zero_point_tensor;
+  int32_t has_scalar_zero_point;
+  float scalar_zero_point;
+  int32_t has_bias;
+  int32_t max_tokens; /* upper bound for mldhip_op_set_shape's b*h*w */
+} mldhip_fc_desc;
+
+int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);
+
+/* CreateQuantization (common/kernels/quantize_and_dequantize.h:57-73, .cc:693-842).
+ * src 0 "src_tensor" [ceil(c/4)][tokens][4] (FLOAT16 or FLOAT32);
+ * dst 0 "dst_tensor": codes, C4 types [ceil(c/4)][tokens][4] bytes, C16 types
+ *       [ceil(c/16)][tokens][16] bytes;
+ * dst 1 "dst_params": fp32 [tokens][4] = (inv_scale, offset, sum, 0), the BHWC(b,h,w,2|3)
+ *       fp32 tensor the builder allocates (common/gpu_model_builder.cc:1285-1289). */
+typedef struct {
+  int32_t src_type;
+  int32_t packed_type; /* MLDHIP_PACKED_* */
+  int32_t channels;
+  int32_t calculate_sum;
+  int32_t symmetric;
+  int32_t max_tokens;
+} mldhip_quant_desc;
+
+int mldhip_quantization_create(const mldhip_quant_desc* desc, mldhip_op** op);
+
+/* GetConvolutionInt8SrcType (common/selectors/convolution_selector.cc:384-400) for this
+ * device: the packed activation type the int8 convolution reads (MLDHIP_PACKED_INT8C16). */
+int mldhip_conv_int8_src_type(void);
+
+/* CreateConvGenericInt8ExternalWeights (common/kernels/conv_generic.cc:4237-4265) for 1x1
+ * kernels with CreateDequantization (common/kernels/quantize_and_dequantize.h:76-81,
+ * .cc:867-964) linked as its epilogue, as the builder wires them
+ * (common/gpu_model_builder.cc:1325-1431).  src objects in node-input order (:1414-1424):
+ *   0 "src_tensor"          codes, src_packed_type
+ *   1 "weights"             per `weights` (mldhip_conv_int8_weights_desc)
+ *   2 "params_tensor"       fp32 [tokens][4] from the quantization op
+ *   3 "weights_sum"         int32, ceil(o/4)*4
+ *   4 "weights_scale"       fp32, ceil(o/4)*4
+ *   5 "weights_zero_point"  fp32, present iff has_zero_point
+ *   6 "biases"              dst_type, present iff has_bias (the builder's separate Add)
+ * dst 0 "dst_tensor" [ceil(o/4)][tokens][4]; dst_type INT32 returns the raw accumulators
+ * (no epilogue; only objects 0 and 1 are bound). */
+typedef struct {
+  int32_t src_packed_type;
+  int32_t dst_type; /* MLDHIP_FLOAT16 / MLDHIP_FLOAT32 / MLDHIP_INT32 */
+  int32_t o, i;
+  mldhip_weights_desc weights;
+  int32_t has_zero_point;
+  int32_t has_bias;
+  int32_t max_tokens;
+} mldhip_conv_int8_desc;
+
+int mldhip_conv_int8_create(const mldhip_conv_int8_desc* desc, mldhip_op** op);
+
+/* Introspection of the object lists, in registration order (GPUOperation::src_tensors_names_,
+ * dst_tensors_names_, common/task/gpu_operation.h:97-274). */
+int mldhip_op_src_count(const mldhip_op* op);
+int mldhip_op_dst_count(const mldhip_op* op);
+const char* mldhip_op_src_name(const mldhip_op* op, int index);
+const char* mldhip_op_dst_name(const mldhip_op* op, int index);
+
+/* ClOperation::SetSrcTensor / SetDstTensor (cl/cl_operation.cc:66-82): bind a device buffer
+ * to the index-th src / dst object.  `bytes` is checked against what the current shape
+ * needs at launch. */
+int mldhip_op_set_src(mldhip_op* op, int index, const void* device_ptr, size_t bytes);
+int mldhip_op_set_dst(mldhip_op* op, int index, void* device_ptr, size_t bytes);
+
+/* Runtime shape of the activation tensor, BHW (channels are fixed at creation); the
+ * counterpart of UpdateParams -> BindArguments + GetGridSize (cl/cl_operation.cc:59-64,
+ * common/kernels/fully_connected.cc:944-979).  b*h*w must be <= max_tokens. */
+int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w);
+
+/* ClOperation::AddToQueue (cl/cl_operation.cc:84-88): enqueue on `stream` (hipStream_t). */
+int mldhip_op_launch(mldhip_op* op, void* stream);
+
+/* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
+ * at the current shape (GPUOperation::flops_/read_size_/write_size_,
+ * common/task/gpu_operation.h:190-195). */
+const char* mldhip_op_kernel_name(const mldhip_op* op);
+int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops);
+
+void mldhip_op_destroy(mldhip_op* op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLDHIP_H_ */

@@ -1,0 +1,636 @@
+// C-ABI layer: argument validation, op objects (the node executors), kernel dispatch.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/mldhip.h"
+#include "kernels.h"
+#include "packer.h"
+
+using namespace mldhip;
+
+namespace {
+
+thread_local std::string g_error;
+
+int Fail(int code, const std::string& msg) {
+  g_error = msg;
+  return code;
+}
+
+int HipFail(hipError_t e, const char* what) {
+  return Fail(MLDHIP_INTERNAL, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+size_t TypeBytes(int type) {
+  switch (type) {
+    case MLDHIP_FLOAT16: return 2;
+    case MLDHIP_FLOAT32: return 4;
+    case MLDHIP_INT32: return 4;
+    case MLDHIP_UINT8:
+    case MLDHIP_INT8: return 1;
+    default: return 0;
+  }
+}
+
+int WeightBits(int type) {
+  if (type == MLDHIP_UINT4) return 4;
+  if (type == MLDHIP_UINT8 || type == MLDHIP_INT8) return 8;
+  return 0;
+}
+
+int CheckShape(int o, int h, int w, int i) {
+  if (o <= 0 || h <= 0 || w <= 0 || i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
+  return MLDHIP_OK;
+}
+
+bool IsOGroupLayout(int layout) {
+  return layout == MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4 || layout == MLDHIP_LAYOUT_OSPATIAL_IOGROUP_O4I4 ||
+         layout == MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4;
+}
+
+int CheckDesc(const mldhip_weights_desc* d) {
+  if (!d) return Fail(MLDHIP_INVALID_ARGUMENT, "null WeightsDescription");
+  if (IsOGroupLayout(d->layout)) {
+    if (d->output_group_size <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "output_group_size must be positive");
+    return MLDHIP_OK;
+  }
+  if (d->layout == MLDHIP_LAYOUT_CUSTOM_GROUPS) {
+    if (d->n_groups <= 0 || d->n_groups > MLDHIP_MAX_CUSTOM_GROUPS)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "custom groups: bad group count");
+    for (int g = 0; g < d->n_groups; ++g)
+      if (d->group_axis[g] < 0 || d->group_axis[g] > 3)
+        return Fail(MLDHIP_INVALID_ARGUMENT, "custom groups: bad axis");
+    return MLDHIP_OK;
+  }
+  return Fail(MLDHIP_UNIMPLEMENTED, "Unsupported layout");
+}
+
+}  // namespace
+
+struct mldhip_op {
+  enum Kind { kFc, kQuant, kConvInt8 } kind = kFc;
+  std::vector<std::string> src_names, dst_names;
+  std::vector<const void*> src_ptr;
+  std::vector<size_t> src_bytes;
+  std::vector<void*> dst_ptr;
+  std::vector<size_t> dst_bytes;
+  int b = 1, h = 1, w = 1;
+  int max_tokens = 1;
+  mldhip_fc_desc fc{};
+  mldhip_quant_desc q{};
+  mldhip_conv_int8_desc cv{};
+  int idx_scale = -1, idx_zp = -1, idx_bias = -1;
+  float* partial = nullptr;
+  size_t partial_floats = 0;
+  int* counters = nullptr;
+  const char* last_kernel = "";
+
+  void AddSrc(const char* name) {
+    src_names.emplace_back(name);
+    src_ptr.push_back(nullptr);
+    src_bytes.push_back(0);
+  }
+  void AddDst(const char* name) {
+    dst_names.emplace_back(name);
+    dst_ptr.push_back(nullptr);
+    dst_bytes.push_back(0);
+  }
+  int Tokens() const { return b * h * w; }
+};
+
+extern "C" {
+
+const char* mldhip_last_error(void) { return g_error.c_str(); }
+const char* mldhip_version(void) { return "mldhip 0.1 (gfx950)"; }
+
+// ---------------------------------------------------------------------------------------
+// weight descriptions and packers
+// ---------------------------------------------------------------------------------------
+
+static int FcDesc(int o, int i, int type, mldhip_weights_desc* desc) {
+  if (!desc) return Fail(MLDHIP_INVALID_ARGUMENT, "null desc");
+  if (o <= 0 || i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
+  std::memset(desc, 0, sizeof(*desc));
+  desc->type = type;
+  desc->layout = MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4;
+  desc->output_group_size = DivUp(o, 4);
+  return MLDHIP_OK;
+}
+
+int mldhip_fc_int8_weights_desc(int o, int i, mldhip_weights_desc* desc) { return FcDesc(o, i, MLDHIP_UINT8, desc); }
+int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc) { return FcDesc(o, i, MLDHIP_UINT4, desc); }
+
+int mldhip_conv_int8_weights_desc(int o, int i, mldhip_weights_desc* desc) {
+  if (!desc) return Fail(MLDHIP_INVALID_ARGUMENT, "null desc");
+  if (o <= 0 || i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
+  std::memset(desc, 0, sizeof(*desc));
+  desc->type = MLDHIP_INT8;
+  desc->layout = MLDHIP_LAYOUT_CUSTOM_GROUPS;
+  desc->output_group_size = 1;
+  desc->n_groups = 3;
+  desc->group_axis[0] = MLDHIP_AXIS_I;
+  desc->group_size[0] = 16;
+  desc->group_axis[1] = MLDHIP_AXIS_O;
+  desc->group_size[1] = 0;
+  desc->group_axis[2] = MLDHIP_AXIS_I;
+  desc->group_size[2] = 0;
+  return MLDHIP_OK;
+}
+
+int mldhip_total_elements(const mldhip_weights_desc* desc, int o, int h, int w, int i, size_t* elements) {
+  if (!elements) return Fail(MLDHIP_INVALID_ARGUMENT, "null output");
+  if (int rc = CheckDesc(desc)) return rc;
+  if (int rc = CheckShape(o, h, w, i)) return rc;
+  const PackShape sh{o, h, w, i};
+  *elements = desc->layout == MLDHIP_LAYOUT_CUSTOM_GROUPS
+                  ? CustomTotalElements(sh, desc->group_axis, desc->group_size, desc->n_groups)
+                  : TotalElements(sh, desc->layout, desc->output_group_size);
+  return MLDHIP_OK;
+}
+
+int mldhip_packed_bytes(const mldhip_weights_desc* desc, int o, int h, int w, int i, size_t* bytes) {
+  size_t elements = 0;
+  if (int rc = mldhip_total_elements(desc, o, h, w, i, &elements)) return rc;
+  const int bits = WeightBits(desc->type);
+  if (!bits) return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type");
+  *bytes = (elements * bits + 7) / 8;
+  return MLDHIP_OK;
+}
+
+static int CheckPackArgs(const void* weights, const mldhip_weights_desc* desc, const void* dst, int o, int h,
+                         int w, int i, size_t dst_bytes, int bits) {
+  if (!weights || !dst) return Fail(MLDHIP_INVALID_ARGUMENT, "null buffer");
+  if (int rc = CheckDesc(desc)) return rc;
+  if (int rc = CheckShape(o, h, w, i)) return rc;
+  size_t elements = 0;
+  if (int rc = mldhip_total_elements(desc, o, h, w, i, &elements)) return rc;
+  if (dst_bytes < (elements * bits + 7) / 8)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "destination span is smaller than the layout needs");
+  return MLDHIP_OK;
+}
+
+int mldhip_rearrange_int8_as_uint8(const int8_t* weights, int o, int h, int w, int i,
+                                   const mldhip_weights_desc* desc, uint8_t* dst, size_t dst_bytes, int shift,
+                                   unsigned pad) {
+  if (int rc = CheckPackArgs(weights, desc, dst, o, h, w, i, dst_bytes, 8)) return rc;
+  if (!IsOGroupLayout(desc->layout)) return Fail(MLDHIP_UNIMPLEMENTED, "Unsupported layout");
+  RearrangeU8(reinterpret_cast<const uint8_t*>(weights), PackShape{o, h, w, i}, desc->layout,
+              desc->output_group_size, (uint8_t)pad, shift, dst);
+  return MLDHIP_OK;
+}
+
+int mldhip_rearrange_int8_as_uint4(const int8_t* weights, int o, int h, int w, int i,
+                                   const mldhip_weights_desc* desc, uint8_t* dst, size_t dst_bytes, int shift,
+                                   unsigned pad) {
+  if (int rc = CheckPackArgs(weights, desc, dst, o, h, w, i, dst_bytes, 4)) return rc;
+  if (!IsOGroupLayout(desc->layout)) return Fail(MLDHIP_UNIMPLEMENTED, "Unsupported layout");
+  RearrangeInt8AsUint4(weights, PackShape{o, h, w, i}, desc->layout, desc->output_group_size, shift, pad, dst);
+  return MLDHIP_OK;
+}
+
+int mldhip_rearrange_int8(const int8_t* weights, int o, int h, int w, int i, const mldhip_weights_desc* desc,
+                          int8_t* dst, size_t dst_bytes) {
+  if (int rc = CheckPackArgs(weights, desc, dst, o, h, w, i, dst_bytes, 8)) return rc;
+  const PackShape sh{o, h, w, i};
+  if (desc->layout == MLDHIP_LAYOUT_CUSTOM_GROUPS) {
+    RearrangeCustomI8(weights, sh, desc->group_axis, desc->group_size, desc->n_groups, 0, dst);
+  } else {
+    RearrangeU8(reinterpret_cast<const uint8_t*>(weights), sh, desc->layout, desc->output_group_size, 0, 0,
+                reinterpret_cast<uint8_t*>(dst));
+  }
+  return MLDHIP_OK;
+}
+
+int mldhip_rearrange_uint4_packed(const uint8_t* weights, int o, int h, int w, int i,
+                                  const mldhip_weights_desc* desc, uint8_t* dst, size_t dst_bytes,
+                                  int32_t* weights_sum_i, size_t sum_len, unsigned pad, int swap_dims) {
+  if (!desc) return Fail(MLDHIP_INVALID_ARGUMENT, "null WeightsDescription");
+  if (desc->layout != MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4 &&
+      desc->layout != MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4)
+    return Fail(MLDHIP_UNIMPLEMENTED, "Unsupported layout");
+  if (int rc = CheckPackArgs(weights, desc, dst, o, h, w, i, dst_bytes, 4)) return rc;
+  if (!weights_sum_i) return Fail(MLDHIP_INVALID_ARGUMENT, "null weights_sum_i");
+  RearrangeUint4Packed(weights, PackShape{o, h, w, i}, desc->layout, desc->output_group_size, dst, weights_sum_i,
+                       sum_len, pad, swap_dims != 0);
+  return MLDHIP_OK;
+}
+
+int mldhip_weights_sum_i(const int8_t* weights, int o, int h, int w, int i, int32_t* sum) {
+  if (!weights || !sum) return Fail(MLDHIP_INVALID_ARGUMENT, "null buffer");
+  if (int rc = CheckShape(o, h, w, i)) return rc;
+  WeightsSumI(weights, PackShape{o, h, w, i}, sum);
+  return MLDHIP_OK;
+}
+
+static uint16_t FloatToHalfBits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  const int32_t exp = (int32_t)((x >> 23) & 0xFF) - 127 + 15;
+  uint32_t man = x & 0x7FFFFFu;
+  if (((x >> 23) & 0xFF) == 0xFF) return (uint16_t)(sign | 0x7C00u | (man ? 0x200u : 0u));
+  if (exp >= 31) return (uint16_t)(sign | 0x7C00u);
+  if (exp <= 0) {
+    if (exp < -10) return (uint16_t)sign;
+    man |= 0x800000u;
+    const int shift = 14 - exp;
+    uint32_t q = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1))) ++q;
+    return (uint16_t)(sign | q);
+  }
+  uint32_t q = ((uint32_t)exp << 10) | (man >> 13);
+  const uint32_t rem = man & 0x1FFFu;
+  if (rem > 0x1000u || (rem == 0x1000u && (q & 1))) ++q;
+  return (uint16_t)(sign | q);
+}
+
+int mldhip_scale_to_tensor(const float* scale, int o, int groups, int dst_type, void* dst, size_t dst_bytes) {
+  if (!scale || !dst) return Fail(MLDHIP_INVALID_ARGUMENT, "null buffer");
+  if (o <= 0 || groups <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad scale shape");
+  if (dst_type != MLDHIP_FLOAT16 && dst_type != MLDHIP_FLOAT32)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "scale tensor type must be FLOAT16 or FLOAT32");
+  const int os = DivUp(o, 4);
+  const size_t count = (size_t)groups * os * 4;
+  if (dst_bytes < count * TypeBytes(dst_type)) return Fail(MLDHIP_INVALID_ARGUMENT, "destination too small");
+  for (int g = 0; g < groups; ++g)
+    for (int oc = 0; oc < os * 4; ++oc) {
+      const float v = oc < o ? scale[(size_t)oc * groups + g] : 0.0f;
+      const size_t idx = (size_t)g * os * 4 + oc;
+      if (dst_type == MLDHIP_FLOAT32)
+        static_cast<float*>(dst)[idx] = v;
+      else
+        static_cast<uint16_t*>(dst)[idx] = FloatToHalfBits(v);
+    }
+  return MLDHIP_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// ops
+// ---------------------------------------------------------------------------------------
+
+int mldhip_fc_is_recommended(int precision, int tokens) {
+  (void)precision;
+  return tokens <= kGemvMaxTokens ? 1 : 0;
+}
+
+static int AllocWorkspace(mldhip_op* op, int n) {
+  if (op->partial && op->counters) return MLDHIP_OK;
+  const int n_pad = DivUp(n, 4) * 4;
+  op->partial_floats = (size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad;
+  hipError_t e = hipMalloc(reinterpret_cast<void**>(&op->partial), op->partial_floats * sizeof(float));
+  if (e != hipSuccess) return HipFail(e, "hipMalloc(workspace)");
+  e = hipMalloc(reinterpret_cast<void**>(&op->counters), kGemvMaxStrips * sizeof(int));
+  if (e != hipSuccess) return HipFail(e, "hipMalloc(counters)");
+  e = hipMemset(op->counters, 0, kGemvMaxStrips * sizeof(int));
+  if (e != hipSuccess) return HipFail(e, "hipMemset(counters)");
+  return MLDHIP_OK;
+}
+
+int mldhip_fc_create(const mldhip_fc_desc* d, mldhip_op** out) {
+  if (!d || !out) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  if (d->o <= 0 || d->i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
+  if (d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "max_tokens must be positive");
+  const mldhip_weights_desc& wd = d->weights;
+  if (wd.type != MLDHIP_UINT8 && wd.type != MLDHIP_UINT4) {
+    if (wd.type == MLDHIP_FLOAT16 || wd.type == MLDHIP_FLOAT32)
+      return Fail(MLDHIP_UNIMPLEMENTED, "float weights are outside the quantized path");
+    return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type.");
+  }
+  if (wd.layout != MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4) {
+    if (wd.layout == MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4)
+      return Fail(MLDHIP_UNIMPLEMENTED, "texture weight layouts are not supported; use the buffer layout");
+    return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout");
+  }
+  if (wd.output_group_size != DivUp(d->o, 4))
+    return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
+  if (d->precision < MLDHIP_PRECISION_F32 || d->precision > MLDHIP_PRECISION_F16)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "bad precision");
+  const bool int8_math = d->src_type == MLDHIP_INT8;
+  if (int8_math) {
+    if (d->dst_type != MLDHIP_INT32) return Fail(MLDHIP_INVALID_ARGUMENT, "int8 source needs an int32 destination");
+    if (d->scale_o * d->scale_i > 1 || d->has_zero_point_tensor || d->has_bias)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "int8-math FullyConnected takes no scale, zero point or bias");
+  } else {
+    const int tensor_type = d->precision == MLDHIP_PRECISION_F32 ? MLDHIP_FLOAT32 : MLDHIP_FLOAT16;
+    if (d->src_type != tensor_type || d->dst_type != tensor_type)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "tensor types do not match the calculations precision");
+    if (d->scale_o < 1 || d->scale_i < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "bad scale_zp_shape");
+    if (d->scale_o != 1 && d->scale_o != d->o)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "scale_zp_shape.o must be 1 or the output channel count");
+    if (d->scale_o == 1 && d->scale_i != 1)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "group-wise scales need one row per output channel");
+    if (d->scale_i > 1 && (d->i % (4 * d->scale_i)) != 0)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "input channels must split into scale groups of whole 4-channel slices");
+    if (d->has_zero_point_tensor && d->scale_o * d->scale_i == 1)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "a zero-point tensor needs a scale tensor of the same shape");
+  }
+  mldhip_op* op = new (std::nothrow) mldhip_op();
+  if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
+  op->kind = mldhip_op::kFc;
+  op->fc = *d;
+  op->max_tokens = d->max_tokens;
+  op->AddSrc("src_tensor");
+  op->AddSrc("weights");
+  if (!int8_math && d->scale_o * d->scale_i > 1) {
+    op->idx_scale = (int)op->src_names.size();
+    op->AddSrc("weights_scale");
+    if (d->has_zero_point_tensor) {
+      op->idx_zp = (int)op->src_names.size();
+      op->AddSrc("weights_zero_point");
+    }
+  }
+  if (d->has_bias) {
+    op->idx_bias = (int)op->src_names.size();
+    op->AddSrc("biases");
+  }
+  op->AddDst("dst_tensor");
+  *out = op;
+  return MLDHIP_OK;
+}
+
+int mldhip_quantization_create(const mldhip_quant_desc* d, mldhip_op** out) {
+  if (!d || !out) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  if (d->src_type != MLDHIP_FLOAT16 && d->src_type != MLDHIP_FLOAT32)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "source must be FLOAT16 or FLOAT32");
+  if (d->packed_type != MLDHIP_PACKED_UINT8C4 && d->packed_type != MLDHIP_PACKED_INT8C4 &&
+      d->packed_type != MLDHIP_PACKED_INT8C16 && d->packed_type != MLDHIP_PACKED_UINT8C16)
+    return Fail(MLDHIP_UNIMPLEMENTED, "packed type not supported");
+  if (d->channels <= 0 || d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad shape");
+  mldhip_op* op = new (std::nothrow) mldhip_op();
+  if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
+  op->kind = mldhip_op::kQuant;
+  op->q = *d;
+  op->max_tokens = d->max_tokens;
+  op->AddSrc("src_tensor");
+  op->AddDst("dst_tensor");
+  op->AddDst("dst_params");
+  *out = op;
+  return MLDHIP_OK;
+}
+
+int mldhip_conv_int8_src_type(void) { return MLDHIP_PACKED_INT8C16; }
+
+int mldhip_conv_int8_create(const mldhip_conv_int8_desc* d, mldhip_op** out) {
+  if (!d || !out) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  if (d->o <= 0 || d->i <= 0 || d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad shape");
+  if (d->src_packed_type != MLDHIP_PACKED_INT8C16)
+    return Fail(MLDHIP_UNIMPLEMENTED, "the int8 convolution reads kInt8C16 activations");
+  mldhip_weights_desc want;
+  mldhip_conv_int8_weights_desc(d->o, d->i, &want);
+  const mldhip_weights_desc& wd = d->weights;
+  bool same = wd.type == want.type && wd.layout == want.layout && wd.n_groups == want.n_groups;
+  for (int g = 0; same && g < want.n_groups; ++g)
+    same = wd.group_axis[g] == want.group_axis[g] && wd.group_size[g] == want.group_size[g];
+  if (!same)
+    return Fail(MLDHIP_INVALID_ARGUMENT,
+                "weights must be in the layout mldhip_conv_int8_weights_desc returns (convert them first)");
+  if (d->dst_type != MLDHIP_FLOAT16 && d->dst_type != MLDHIP_FLOAT32 && d->dst_type != MLDHIP_INT32)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "bad destination type");
+  mldhip_op* op = new (std::nothrow) mldhip_op();
+  if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
+  op->kind = mldhip_op::kConvInt8;
+  op->cv = *d;
+  op->max_tokens = d->max_tokens;
+  op->AddSrc("src_tensor");
+  op->AddSrc("weights");
+  if (d->dst_type != MLDHIP_INT32) {
+    op->AddSrc("params_tensor");
+    op->AddSrc("weights_sum");
+    op->AddSrc("weights_scale");
+    if (d->has_zero_point) {
+      op->idx_zp = (int)op->src_names.size();
+      op->AddSrc("weights_zero_point");
+    }
+    if (d->has_bias) {
+      op->idx_bias = (int)op->src_names.size();
+      op->AddSrc("biases");
+    }
+  }
+  op->AddDst("dst_tensor");
+  *out = op;
+  return MLDHIP_OK;
+}
+
+int mldhip_op_src_count(const mldhip_op* op) { return op ? (int)op->src_names.size() : 0; }
+int mldhip_op_dst_count(const mldhip_op* op) { return op ? (int)op->dst_names.size() : 0; }
+const char* mldhip_op_src_name(const mldhip_op* op, int index) {
+  if (!op || index < 0 || index >= (int)op->src_names.size()) return nullptr;
+  return op->src_names[index].c_str();
+}
+const char* mldhip_op_dst_name(const mldhip_op* op, int index) {
+  if (!op || index < 0 || index >= (int)op->dst_names.size()) return nullptr;
+  return op->dst_names[index].c_str();
+}
+
+int mldhip_op_set_src(mldhip_op* op, int index, const void* device_ptr, size_t bytes) {
+  if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+  if (index < 0 || index >= (int)op->src_ptr.size()) return Fail(MLDHIP_OUT_OF_RANGE, "src index out of range");
+  if (!device_ptr) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  op->src_ptr[index] = device_ptr;
+  op->src_bytes[index] = bytes;
+  return MLDHIP_OK;
+}
+
+int mldhip_op_set_dst(mldhip_op* op, int index, void* device_ptr, size_t bytes) {
+  if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+  if (index < 0 || index >= (int)op->dst_ptr.size()) return Fail(MLDHIP_OUT_OF_RANGE, "dst index out of range");
+  if (!device_ptr) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  op->dst_ptr[index] = device_ptr;
+  op->dst_bytes[index] = bytes;
+  return MLDHIP_OK;
+}
+
+int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w) {
+  if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+  if (b <= 0 || h <= 0 || w <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "shape must be positive");
+  if ((long long)b * h * w > op->max_tokens) return Fail(MLDHIP_OUT_OF_RANGE, "b*h*w exceeds max_tokens");
+  op->b = b;
+  op->h = h;
+  op->w = w;
+  return MLDHIP_OK;
+}
+
+// Sizes (bytes) every object needs at the current shape, in object order.
+static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::vector<size_t>* dst) {
+  const size_t m = (size_t)op->Tokens();
+  src->assign(op->src_ptr.size(), 0);
+  dst->assign(op->dst_ptr.size(), 0);
+  if (op->kind == mldhip_op::kFc) {
+    const mldhip_fc_desc& d = op->fc;
+    const size_t ks = DivUp(d.i, 4), ns = DivUp(d.o, 4);
+    (*src)[0] = ks * m * 4 * TypeBytes(d.src_type);
+    (*src)[1] = ks * ns * 16 * WeightBits(d.weights.type) / 8;
+    const size_t tb = TypeBytes(d.src_type);
+    if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * ns * 4 * tb;
+    if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * ns * 4 * tb;
+    if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
+    (*dst)[0] = ns * m * 4 * TypeBytes(d.dst_type);
+  } else if (op->kind == mldhip_op::kQuant) {
+    const mldhip_quant_desc& d = op->q;
+    const size_t s = DivUp(d.channels, 4);
+    const bool c16 = d.packed_type == MLDHIP_PACKED_INT8C16 || d.packed_type == MLDHIP_PACKED_UINT8C16;
+    (*src)[0] = s * m * 4 * TypeBytes(d.src_type);
+    (*dst)[0] = c16 ? (size_t)DivUp((int)s, 4) * m * 16 : s * m * 4;
+    (*dst)[1] = m * 4 * sizeof(float);
+  } else {
+    const mldhip_conv_int8_desc& d = op->cv;
+    const size_t k16 = DivUp(d.i, 16), ns = DivUp(d.o, 4);
+    (*src)[0] = k16 * m * 16;
+    (*src)[1] = k16 * (size_t)d.o * 16;
+    if (d.dst_type != MLDHIP_INT32) {
+      (*src)[2] = m * 4 * sizeof(float);
+      (*src)[3] = ns * 4 * sizeof(int32_t);
+      (*src)[4] = ns * 4 * sizeof(float);
+      if (op->idx_zp >= 0) (*src)[op->idx_zp] = ns * 4 * sizeof(float);
+      if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
+    }
+    (*dst)[0] = ns * m * 4 * TypeBytes(d.dst_type);
+  }
+}
+
+static int CheckBindings(const mldhip_op* op) {
+  std::vector<size_t> need_src, need_dst;
+  RequiredSizes(op, &need_src, &need_dst);
+  for (size_t i = 0; i < need_src.size(); ++i) {
+    if (!op->src_ptr[i]) return Fail(MLDHIP_FAILED_PRECONDITION, "src object '" + op->src_names[i] + "' is not bound");
+    if (op->src_bytes[i] < need_src[i])
+      return Fail(MLDHIP_INVALID_ARGUMENT, "src object '" + op->src_names[i] + "' is smaller than the shape needs (" +
+                                               std::to_string(op->src_bytes[i]) + " < " + std::to_string(need_src[i]) + ")");
+  }
+  for (size_t i = 0; i < need_dst.size(); ++i) {
+    if (!op->dst_ptr[i]) return Fail(MLDHIP_FAILED_PRECONDITION, "dst object '" + op->dst_names[i] + "' is not bound");
+    if (op->dst_bytes[i] < need_dst[i])
+      return Fail(MLDHIP_INVALID_ARGUMENT, "dst object '" + op->dst_names[i] + "' is smaller than the shape needs (" +
+                                               std::to_string(op->dst_bytes[i]) + " < " + std::to_string(need_dst[i]) + ")");
+  }
+  return MLDHIP_OK;
+}
+
+static int EnvFlag(const char* name) {
+  const char* v = std::getenv(name);
+  return v && v[0] && v[0] != '0';
+}
+
+int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
+  if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+  if (int rc = CheckBindings(op)) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
+  hipError_t e = hipSuccess;
+  if (op->kind == mldhip_op::kFc) {
+    const mldhip_fc_desc& d = op->fc;
+    if (d.src_type == MLDHIP_INT8) {
+      e = LaunchFcInt8Math(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
+                           static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o,
+                           WeightBits(d.weights.type), stream, &op->last_kernel);
+    } else {
+      FcArgs a;
+      a.act = op->src_ptr[0];
+      a.weights = static_cast<const uint8_t*>(op->src_ptr[1]);
+      a.scale = op->idx_scale >= 0 ? op->src_ptr[op->idx_scale] : nullptr;
+      a.zero_point = op->idx_zp >= 0 ? op->src_ptr[op->idx_zp] : nullptr;
+      a.bias = op->idx_bias >= 0 ? op->src_ptr[op->idx_bias] : nullptr;
+      a.dst = op->dst_ptr[0];
+      a.m = op->Tokens();
+      a.k = d.i;
+      a.n = d.o;
+      a.act_f16 = d.src_type == MLDHIP_FLOAT16;
+      a.dst_f16 = d.dst_type == MLDHIP_FLOAT16;
+      a.weight_bits = WeightBits(d.weights.type);
+      a.scale_kind = d.scale_o * d.scale_i == 1 ? kScaleScalar : (d.scale_i == 1 ? kScaleLinear : kScaleBlock);
+      a.groups = d.scale_i;
+      a.scalar_scale = d.scalar_scale;
+      a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
+      a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
+      // split-K workspace of the streaming kernel: allocated once, on the first launch
+      if (a.m <= kGemvMaxTokens && a.weight_bits == 4 && a.act_f16)
+        if (int rc = AllocWorkspace(op, d.o)) return rc;
+      a.partial = op->partial;
+      a.partial_floats = op->partial_floats;
+      a.counters = op->counters;
+      a.n_counters = kGemvMaxStrips;
+      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
+      if (!force_generic && FcW4StreamSupported(a)) {
+        e = LaunchFcW4Stream(a, stream, &op->last_kernel);
+      } else if (!force_generic && FcW4MfmaSupported(a)) {
+        e = LaunchFcW4Mfma(a, stream, &op->last_kernel);
+      } else {
+        e = LaunchFcGeneric(a, stream, &op->last_kernel);
+      }
+    }
+  } else if (op->kind == mldhip_op::kQuant) {
+    const mldhip_quant_desc& d = op->q;
+    QuantArgs a;
+    a.src = op->src_ptr[0];
+    a.codes = op->dst_ptr[0];
+    a.params = static_cast<float*>(op->dst_ptr[1]);
+    a.tokens = op->Tokens();
+    a.channels = d.channels;
+    a.batch = op->b;
+    a.src_f16 = d.src_type == MLDHIP_FLOAT16;
+    a.packed_type = d.packed_type;
+    a.symmetric = d.symmetric != 0;
+    a.calculate_sum = d.calculate_sum != 0;
+    e = LaunchQuantize(a, stream, &op->last_kernel);
+  } else {
+    const mldhip_conv_int8_desc& d = op->cv;
+    ConvInt8Args a;
+    a.codes = static_cast<const int8_t*>(op->src_ptr[0]);
+    a.weights = static_cast<const int8_t*>(op->src_ptr[1]);
+    if (d.dst_type != MLDHIP_INT32) {
+      a.params = static_cast<const float*>(op->src_ptr[2]);
+      a.weights_sum = static_cast<const int32_t*>(op->src_ptr[3]);
+      a.weights_scale = static_cast<const float*>(op->src_ptr[4]);
+      a.weights_zero_point = op->idx_zp >= 0 ? static_cast<const float*>(op->src_ptr[op->idx_zp]) : nullptr;
+      a.bias = op->idx_bias >= 0 ? op->src_ptr[op->idx_bias] : nullptr;
+    }
+    a.dst = op->dst_ptr[0];
+    a.m = op->Tokens();
+    a.k = d.i;
+    a.n = d.o;
+    a.dst_type = d.dst_type;
+    e = LaunchConvInt8(a, stream, &op->last_kernel);
+  }
+  if (e != hipSuccess) return HipFail(e, "kernel launch");
+  return MLDHIP_OK;
+}
+
+const char* mldhip_op_kernel_name(const mldhip_op* op) { return op ? op->last_kernel : ""; }
+
+int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {
+  if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+  std::vector<size_t> need_src, need_dst;
+  RequiredSizes(op, &need_src, &need_dst);
+  uint64_t total = 0;
+  for (size_t v : need_src) total += v;
+  for (size_t v : need_dst) total += v;
+  if (bytes) *bytes = total;
+  if (flops) {
+    const uint64_t m = (uint64_t)op->Tokens();
+    if (op->kind == mldhip_op::kFc)
+      *flops = 2 * m * (uint64_t)op->fc.i * (uint64_t)op->fc.o;
+    else if (op->kind == mldhip_op::kConvInt8)
+      *flops = 2 * m * (uint64_t)op->cv.i * (uint64_t)op->cv.o;
+    else
+      *flops = 5 * m * (uint64_t)op->q.channels;
+  }
+  return MLDHIP_OK;
+}
+
+void mldhip_op_destroy(mldhip_op* op) {
+  if (!op) return;
+  if (op->partial) (void)hipFree(op->partial);
+  if (op->counters) (void)hipFree(op->counters);
+  delete op;
+}
+
+}  // extern "C"

@@ -1,0 +1,84 @@
+// Internal launch interface between the C-ABI layer (api.cpp) and the HIP kernels.
+#ifndef MLDHIP_KERNELS_H_
+#define MLDHIP_KERNELS_H_
+
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mldhip {
+
+inline int DivUp(int a, int b) { return (a + b - 1) / b; }
+
+enum ScaleKind { kScaleScalar = 0, kScaleLinear = 1, kScaleBlock = 2 };
+
+// One FullyConnected launch.  Tensors are slice-major: act [Ks][m][4], dst [Ns][m][4].
+struct FcArgs {
+  const void* act = nullptr;
+  const uint8_t* weights = nullptr;  // I4O4 blocks: [Ks][Ns] x (16 B for uint8, 8 B for uint4)
+  const void* scale = nullptr;       // linear: Ns*4; block: [groups][Ns][4]; tensor type
+  const void* zero_point = nullptr;  // same shape as scale
+  const void* bias = nullptr;        // Ns*4, dst type
+  void* dst = nullptr;
+  int m = 0, k = 0, n = 0;
+  bool act_f16 = true;   // activations / scale / zero-point element type
+  bool dst_f16 = true;   // output / bias element type
+  int weight_bits = 4;
+  int scale_kind = kScaleLinear;
+  int groups = 1;
+  float scalar_scale = 1.0f;
+  bool has_zero_point = false;
+  float scalar_zero_point = 0.0f;
+  // private workspace of the op (split-K partial sums and arrival counters)
+  float* partial = nullptr;
+  size_t partial_floats = 0;
+  int* counters = nullptr;
+  int n_counters = 0;
+};
+
+// Split-K workspace sizing for the streaming GEMV.
+constexpr int kGemvMaxTokens = 4;
+constexpr int kGemvMaxKSplit = 32;
+constexpr int kGemvMaxStrips = 4096;
+
+hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+bool FcW4StreamSupported(const FcArgs& a);
+hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+
+// int8 activations x uint8/uint4 weights -> int32 (no scales).
+hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k,
+                            int n, int weight_bits, hipStream_t stream, const char** kernel_name);
+
+struct QuantArgs {
+  const void* src = nullptr;
+  void* codes = nullptr;
+  float* params = nullptr;
+  int tokens = 0, channels = 0, batch = 1;
+  bool src_f16 = true;
+  int packed_type = 2;
+  bool symmetric = false;
+  bool calculate_sum = false;
+};
+hipError_t LaunchQuantize(const QuantArgs& a, hipStream_t stream, const char** kernel_name);
+
+struct ConvInt8Args {
+  const int8_t* codes = nullptr;    // [ceil(k/16)][m][16]
+  const int8_t* weights = nullptr;  // [ceil(k/16)][n][16]
+  const float* params = nullptr;    // [m][4]
+  const int32_t* weights_sum = nullptr;
+  const float* weights_scale = nullptr;
+  const float* weights_zero_point = nullptr;
+  const void* bias = nullptr;
+  void* dst = nullptr;
+  int m = 0, k = 0, n = 0;
+  int dst_type = 1;  // MLDHIP_FLOAT16 / FLOAT32 / INT32
+};
+hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char** kernel_name);
+
+// Multi-token FullyConnected with int4 weights on the MFMA units (fp16 tensors).
+bool FcW4MfmaSupported(const FcArgs& a);
+hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+
+}  // namespace mldhip
+
+#endif  // MLDHIP_KERNELS_H_

@@ -1,0 +1,130 @@
+"""CPU-side checks of the product library: it loads, exports every symbol include/mldhip.h
+declares, validates arguments like the reference factories do, and lists src/dst objects in
+the reference's registration order.  No kernel is launched here."""
+import os
+import re
+
+import pytest
+
+import mldhip as M
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mldhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mldhip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = M.lib()
+    names = declared_symbols()
+    assert len(names) >= 25
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(M.SYMBOLS) == names
+    assert b"gfx950" in lib.mldhip_version()
+
+
+def test_fc_weights_desc_matches_reference_factories():
+    # common/kernels/fully_connected.cc:1218-1246
+    d = M.fc_int4_weights_desc(14336, 4096)
+    assert (d.type, d.layout, d.output_group_size) == (M.UINT4, M.LAYOUT_I4O4, 3584)
+    d = M.fc_int8_weights_desc(533, 171)
+    assert (d.type, d.layout, d.output_group_size) == (M.UINT8, M.LAYOUT_I4O4, 134)
+    assert M.packed_bytes(M.fc_int4_weights_desc(14336, 4096), 14336, 1, 1, 4096) == 29360128
+    assert M.packed_bytes(M.fc_int8_weights_desc(2048, 2048), 2048, 1, 1, 2048) == 4194304
+
+
+def test_fc_object_order():
+    # fully_connected.cc:359-360, 1160-1170; fully_connected_util.cc:409-487
+    wd = M.fc_int4_weights_desc(64, 64)
+    op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, wd, scale_shape=(64, 2),
+                     has_zero_point_tensor=True, has_bias=True, max_tokens=4)
+    assert op.src_names == ["src_tensor", "weights", "weights_scale", "weights_zero_point", "biases"]
+    assert op.dst_names == ["dst_tensor"]
+    op = M.fc_create(M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 64, 64, M.fc_int8_weights_desc(64, 64),
+                     scalar_scale=0.5, has_bias=True)
+    assert op.src_names == ["src_tensor", "weights", "biases"]
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 64, 64, M.fc_int8_weights_desc(64, 64))
+    assert op.src_names == ["src_tensor", "weights"]
+
+
+def test_quantization_and_conv_object_order():
+    # quantize_and_dequantize.cc:754-756; gpu_model_builder.cc:1414-1424
+    q = M.quantization_create(M.FLOAT16, M.PACKED_INT8C16, 2048, max_tokens=8)
+    assert q.src_names == ["src_tensor"] and q.dst_names == ["dst_tensor", "dst_params"]
+    wd = M.conv_int8_weights_desc(128, 64)
+    c = M.conv_int8_create(M.FLOAT16, 128, 64, wd, has_zero_point=True, has_bias=True)
+    assert c.src_names == ["src_tensor", "weights", "params_tensor", "weights_sum", "weights_scale",
+                           "weights_zero_point", "biases"]
+    c = M.conv_int8_create(M.INT32, 128, 64, wd)
+    assert c.src_names == ["src_tensor", "weights"]
+    assert M.lib().mldhip_conv_int8_src_type() == M.PACKED_INT8C16
+
+
+def expect_error(code, fn, *a, **k):
+    with pytest.raises(M.MldhipError) as e:
+        fn(*a, **k)
+    assert e.value.code == code, e.value
+    return e.value.message
+
+
+def test_fc_create_rejects_what_the_reference_rejects():
+    wd = M.fc_int4_weights_desc(64, 64)
+    bad_group = M.make_desc(M.UINT4, M.LAYOUT_I4O4, 3)
+    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_group)
+    assert "output_group_size" in msg  # fully_connected.cc:1107-1110
+    bad_layout = M.make_desc(M.UINT4, M.LAYOUT_O4I4, 16)
+    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_layout)
+    assert "layout" in msg  # fully_connected.cc:1111-1115
+    bad_type = M.make_desc(M.INT32, M.LAYOUT_I4O4, 16)
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_type)
+    # precision / tensor type mismatch (fully_connected.cc:1098-1102 for the weights; same rule for tensors)
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32, M.FLOAT16, M.FLOAT16, 64, 64, wd)
+    # texture layouts and float weights are declared out of scope
+    tex = M.make_desc(M.UINT4, M.LAYOUT_2D_I4O4, 16)
+    expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, tex)
+    flt = M.make_desc(M.FLOAT16, M.LAYOUT_I4O4, 16)
+    expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, flt)
+    # scale groups must split K into whole slices
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, wd,
+                 scale_shape=(64, 3))
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.INT8, M.FLOAT16, 64, 64, wd)
+
+
+def test_op_binding_errors():
+    wd = M.fc_int4_weights_desc(64, 64)
+    op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, wd, scale_shape=(64, 1),
+                     max_tokens=2)
+    expect_error(M.OUT_OF_RANGE, op.set_shape, 1, 1, 3)
+    expect_error(M.INVALID_ARGUMENT, op.set_shape, 0, 1, 1)
+    expect_error(M.OUT_OF_RANGE, op.set_src_raw, 7, 4096, 16)
+    expect_error(M.INVALID_ARGUMENT, op.set_src_raw, 0, 0, 16)
+    msg = expect_error(M.FAILED_PRECONDITION, op.launch)  # nothing bound: refused before any GPU call
+    assert "src_tensor" in msg
+    # too-small buffers are refused at launch, before any GPU call
+    op.set_src_raw(0, 4096, 16)
+    op.set_src_raw(1, 4096, 10)
+    op.set_src_raw(2, 4096, 10)
+    op.set_dst_raw(0, 4096, 10)
+    msg = expect_error(M.INVALID_ARGUMENT, op.launch)
+    assert "smaller" in msg
+
+
+def test_conv_int8_requires_its_layout():
+    fc_layout = M.fc_int8_weights_desc(128, 64)
+    msg = expect_error(M.INVALID_ARGUMENT, M.conv_int8_create, M.FLOAT16, 128, 64, fc_layout)
+    assert "convert" in msg
+    wd = M.conv_int8_weights_desc(128, 64)
+    expect_error(M.UNIMPLEMENTED, M.conv_int8_create, M.FLOAT16, 128, 64, wd,
+                 src_packed_type=M.PACKED_INT8C4)
+
+
+def test_unsupported_pack_layout_is_unimplemented():
+    import numpy as np
+    d = M.make_desc(M.UINT4, M.LAYOUT_O4I4, 1)
+    with pytest.raises(M.MldhipError) as e:  # weights_conversion.cc:1617
+        M.rearrange_uint4_packed(np.zeros(8, np.uint8), (4, 1, 1, 4), d)
+    assert e.value.code == M.UNIMPLEMENTED and "Unsupported layout" in e.value.message

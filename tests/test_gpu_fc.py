@@ -1,0 +1,214 @@
+"""GPU parity of the FullyConnected kernels, through the C-ABI, against the CPU oracle.
+
+Bars: int32 results bit-exact; fp16-output paths max|err| <= 2e-2 * RMS(reference output)
+(the tolerance the north star states); fp32 paths eps_f32 * (K+1), the reference tests'
+own rule (common/task/testing_util.cc:328-331)."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mldhip as M
+import workloads as W
+
+FP16_TOL = 2e-2
+
+
+def torch_cuda():
+    import torch
+    assert torch.cuda.is_available()
+    return torch
+
+
+def oracle_fc(o, case, precision=None, use_kernel=True, wg_y=1):
+    """Oracle output [m][n] float32 for a workloads case."""
+    m, k, n, bits, groups = case["m"], case["k"], case["n"], case["weight_bits"], case["groups"]
+    f16 = case["tensor_dtype"] == np.float16
+    if precision is None:
+        precision = o.PREC_F32F16 if f16 else o.PREC_F32
+    ns = (n + 3) // 4
+    packed = (o.int8_as_uint4 if bits == 4 else o.int8_as_uint8)(case["w"], o.LAYOUT_I4O4, ns)
+    conv = (lambda a: o.f32_to_f16_bits(a)) if f16 else (lambda a: np.asarray(a, np.float32))
+    act = conv(o.to_slices(case["act"]))
+    if groups == 1:
+        sc = np.zeros(ns * 4, np.float32); sc[:n] = case["scale"][:, 0]
+        kind = o.SCALE_LINEAR
+        zp = None
+        if case["zero_point"] is not None:
+            zp = np.zeros(ns * 4, np.float32); zp[:n] = case["zero_point"][:, 0]
+    else:
+        sc = o.scale_to_hoio4(case["scale"]); kind = o.SCALE_BLOCK
+        zp = None if case["zero_point"] is None else o.scale_to_hoio4(case["zero_point"])
+    bias = None
+    if case["bias"] is not None:
+        bias = np.zeros(ns * 4, np.float32); bias[:n] = case["bias"]
+        bias = conv(bias)
+    out = o.fc_kernel(act, packed, m, k, n, precision, bits, kind, conv(sc),
+                      None if zp is None else conv(zp), bias, groups, True, wg_y)
+    out = o.f16_bits_to_f32(out) if f16 else out
+    return o.from_slices(out, n)
+
+
+def textbook(case):
+    ref = case["act"].astype(np.float64) @ W.dequantized_weights(case).T
+    if case["bias"] is not None:
+        ref = ref + case["bias"]
+    return ref
+
+
+def check_fp(got, ref, case, label=""):
+    err = np.abs(got.astype(np.float64) - ref).max()
+    rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
+    if case["tensor_dtype"] == np.float16:
+        assert err <= FP16_TOL * rms, (label, err, rms)
+    else:
+        tol = 1.1920929e-7 * (case["k"] + 1) * max(1.0, np.abs(ref).max())
+        assert err <= tol, (label, err, tol)
+    return err / rms
+
+
+def run_case(oracle, case, expect_kernel=None, env=None):
+    torch_cuda()
+    old = {}
+    for key, val in (env or {}).items():
+        old[key] = os.environ.get(key)
+        os.environ[key] = val
+    try:
+        print("case", {k: case[k] for k in ("m", "k", "n", "weight_bits", "groups")}, env, flush=True)
+        dev = W.FcDevice(case)
+        dev.run()
+        got = dev.result()
+        if expect_kernel:
+            assert dev.op.kernel_name == expect_kernel, dev.op.kernel_name
+        # run twice: the split-K counters must have been reset by the first launch
+        dev.run()
+        assert np.array_equal(got, dev.result())
+    finally:
+        for key, val in old.items():
+            if val is None:
+                os.environ.pop(key, None)
+            else:
+                os.environ[key] = val
+    ref_tb = textbook(case)
+    check_fp(got, ref_tb, case, "textbook")
+    if case["m"] * case["k"] * case["n"] <= 1 << 27:
+        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+    return got
+
+
+def test_config1_int8_fp32(oracle):
+    case = W.make_fc_case(**W.CONFIGS["c1"])
+    run_case(oracle, case, "fc_generic_kernel")
+
+
+def test_config2_int4_decode(oracle):
+    case = W.make_fc_case(**W.CONFIGS["c2"])
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
+@pytest.mark.parametrize("lpr", ["16", "32", "64"])
+@pytest.mark.parametrize("ksplit", ["1", "3", "16"])
+def test_stream_kernel_shapes(oracle, lpr, ksplit):
+    case = W.make_fc_case(seed=3, m=1, k=1024, n=1536, weight_bits=4, tensor_dtype=np.float16)
+    run_case(oracle, case, "fc_w4_stream_kernel", {"MLDHIP_GEMV_LPR": lpr, "MLDHIP_GEMV_KSPLIT": ksplit})
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("groups", [1, 64])
+def test_stream_kernel_tokens_and_groups(oracle, m, groups):
+    case = W.make_fc_case(seed=5 + m, m=m, k=2048, n=2048, weight_bits=4, tensor_dtype=np.float16,
+                          groups=groups, with_bias=True)
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
+@pytest.mark.parametrize("name,k,n", W.C5_LAYER)
+def test_config5_decode_layer_shapes(oracle, name, k, n):
+    case = W.make_fc_case(seed=7, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=k // 32)
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
+def test_stream_kernel_ragged(oracle):
+    # K not a multiple of 32 (partial chunk), N = 8*odd (partial strip)
+    case = W.make_fc_case(seed=11, m=2, k=1000, n=1032, weight_bits=4, tensor_dtype=np.float16)
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("kind", ["linear", "block", "block_zp"])
+def test_generic_kernel_reference_test_shapes(oracle, bits, dtype, kind):
+    """Shapes of the reference's big tests: K=171 or 11*4*7, N=533, tokens 1/4/15."""
+    k = 171 if kind == "linear" else 11 * 4 * 7
+    groups = 1 if kind == "linear" else 7
+    for m in (1, 4, 15):
+        case = W.make_fc_case(seed=13 + m, m=m, k=k, n=533, weight_bits=bits, tensor_dtype=dtype,
+                              groups=groups, with_bias=True, with_zero_point=kind == "block_zp",
+                              act_uniform=True)
+        # (N=533 gives an even slice count, so the symmetric fp16 int4 cases take the streaming kernel)
+        streamable = bits == 4 and dtype == np.float16 and kind == "linear" and m <= 4
+        run_case(oracle, case, "fc_w4_stream_kernel" if streamable else "fc_generic_kernel")
+
+
+def test_known_answers_on_gpu():
+    """Literal cases of common/kernels/tests/fully_connected_test_util.cc:49-249, 1541-1614."""
+    torch = torch_cuda()
+    # scalar scale 0.5 + bias -> {20.5, 15.5}
+    case = dict(m=1, k=4, n=2, weight_bits=8, tensor_dtype=np.float32, groups=1,
+                act=np.array([[0, 1, 2, 3]], np.float32),
+                w=np.array([[2, 4, 6, 8], [10, 12, -14, 16]], np.int8),
+                scale=np.ones((2, 1), np.float32), bias=np.array([0.5, -0.5], np.float32), zero_point=None)
+    dev = W.FcDevice(case, scalar_scale=0.5)
+    dev.run()
+    assert np.allclose(dev.result(), [[20.5, 15.5]], atol=1e-6)
+    # block-wise -> {91.0, 26.8}
+    case = dict(m=1, k=8, n=2, weight_bits=8, tensor_dtype=np.float32, groups=2,
+                act=np.arange(8, dtype=np.float32)[None],
+                w=np.array([[1, 1, 1, 1, 2, 2, 2, 2], [3, 3, 3, 3, 4, 4, 4, 4]], np.int8),
+                scale=np.array([[0.5, 2.0], [1.0, 0.1]], np.float32), bias=np.zeros(2, np.float32),
+                zero_point=None)
+    dev = W.FcDevice(case); dev.run()
+    assert np.allclose(dev.result(), [[91.0, 26.8]], atol=1e-5)
+    # block-wise with zero points -> {509.0, -121.4}
+    case.update(act=np.arange(1, 9, dtype=np.float32)[None],
+                w=np.array([[1, 2, 3, 4, 5, 6, 7, 8], [-8, -7, -6, -5, -4, -3, -2, -1]], np.int8),
+                scale=np.array([[0.5, 2.0], [1.5, 0.1]], np.float32),
+                zero_point=np.array([[2, -3], [1, 4]], np.float32))
+    dev = W.FcDevice(case); dev.run()
+    assert np.allclose(dev.result(), [[509.0, -121.4]], atol=1e-4)
+    # int4 block-wise all ones -> 8.0
+    for dtype, eps in ((np.float32, 1e-6), (np.float16, 1e-2)):
+        case = dict(m=1, k=16, n=4, weight_bits=4, tensor_dtype=dtype, groups=2,
+                    act=np.ones((1, 16), np.float32), w=np.ones((4, 16), np.int8),
+                    scale=np.full((4, 2), 0.5, np.float32), bias=np.zeros(4, np.float32), zero_point=None)
+        dev = W.FcDevice(case); dev.run()
+        assert np.allclose(dev.result(), np.full((1, 4), 8.0), atol=eps)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,k,n", [(1, 112, 152), (5, 171, 533), (1, 2048, 2048), (16, 4096, 1024)])
+def test_int8_math_bit_exact(oracle, bits, m, k, n):
+    """int8 activations x packed weights -> int32, exact (fully_connected_test_util.cc:1446-1448)."""
+    torch = torch_cuda()
+    rng = np.random.default_rng(k + n + bits)
+    lo, hi = (-8, 8) if bits == 4 else (-128, 128)
+    w = rng.integers(lo, hi, size=(n, k), dtype=np.int8)
+    src = rng.integers(-128, 128, size=(m, k), dtype=np.int8)
+    desc = M.fc_int4_weights_desc(n, k) if bits == 4 else M.fc_int8_weights_desc(n, k)
+    packed = (M.rearrange_int8_as_uint4 if bits == 4 else M.rearrange_int8_as_uint8)(w, desc)
+    act = torch.from_numpy(W.to_slices(src)).cuda()
+    wt = torch.from_numpy(packed).cuda()
+    out = torch.zeros(((n + 3) // 4, m, 4), dtype=torch.int32, device="cuda")
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=m)
+    op.bind([act, wt], [out])
+    op.set_shape(1, 1, m)
+    print("int8 math", bits, m, k, n, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    got = W.from_slices(out.cpu().numpy(), n)
+    ref = oracle.fc_reference_i8(src, w)
+    assert np.array_equal(got, ref)
+    if m * k * n <= 1 << 24:
+        mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed, m, k, n, bits), n)
+        assert np.array_equal(got, mimic)
