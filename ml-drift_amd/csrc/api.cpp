@@ -88,7 +88,6 @@ struct mldhip_op {
   int idx_scale = -1, idx_zp = -1, idx_bias = -1;
   float* partial = nullptr;
   size_t partial_floats = 0;
-  int* counters = nullptr;
   const char* last_kernel = "";
 
   void AddSrc(const char* name) {
@@ -281,15 +280,11 @@ int mldhip_fc_is_recommended(int precision, int tokens) {
 }
 
 static int AllocWorkspace(mldhip_op* op, int n) {
-  if (op->partial && op->counters) return MLDHIP_OK;
+  if (op->partial) return MLDHIP_OK;
   const int n_pad = DivUp(n, 4) * 4;
   op->partial_floats = (size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad;
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&op->partial), op->partial_floats * sizeof(float));
   if (e != hipSuccess) return HipFail(e, "hipMalloc(workspace)");
-  e = hipMalloc(reinterpret_cast<void**>(&op->counters), kGemvMaxStrips * sizeof(int));
-  if (e != hipSuccess) return HipFail(e, "hipMalloc(counters)");
-  e = hipMemset(op->counters, 0, kGemvMaxStrips * sizeof(int));
-  if (e != hipSuccess) return HipFail(e, "hipMemset(counters)");
   return MLDHIP_OK;
 }
 
@@ -556,8 +551,6 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         if (int rc = AllocWorkspace(op, d.o)) return rc;
       a.partial = op->partial;
       a.partial_floats = op->partial_floats;
-      a.counters = op->counters;
-      a.n_counters = kGemvMaxStrips;
       const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
       if (!force_generic && FcW4StreamSupported(a)) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);
@@ -629,7 +622,6 @@ int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {
 void mldhip_op_destroy(mldhip_op* op) {
   if (!op) return;
   if (op->partial) (void)hipFree(op->partial);
-  if (op->counters) (void)hipFree(op->counters);
   delete op;
 }
 

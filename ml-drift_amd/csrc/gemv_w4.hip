@@ -1,0 +1,365 @@
+// Streaming int4 GEMV for gfx950 (decode: 1..4 tokens, fp16 tensors, symmetric weights,
+// per-channel scales or group-wise scales whose groups are multiples of 32 input channels).
+//
+// Packed buffer (the reference's I4O4 layout): row ks (4 input channels) holds Ns blocks of
+// 8 bytes; one 16-byte load covers two neighbouring blocks = 8 output channels x 4 input
+// channels.  In word h (0/1) of a block, nibble j (j = 0..3) is (input 2h, output j) and
+// nibble 4+j is (input 2h+1, output j).  Masking a word with 0x000F000F after a shift by 4j
+// therefore leaves the pair (input 2h, input 2h+1) of output j in the two 16-bit halves:
+// the operand shape of v_dot2_f32_f16 against the activation pair.  OR-ing 0x6400 turns a
+// half into the fp16 number 1024+u; a nibble sitting in bits 4..7 of a half is read in place
+// by OR-ing 0x5400, which gives 64+u (the mantissa's unit there is 1/16).  The constant
+// offsets (1024+8 and 64+8) are not subtracted per weight: sum_k a_k (c + u_k - 8 - c) =
+// sum_k a_k (c + u_k) - (c + 8) sum_k a_k, so the kernel accumulates the biased products and
+// removes (c+8) * sum(a) once per chunk.
+//
+// Thread layout: LPR lanes cover one contiguous row segment (LPR x 16 B), 64/LPR rows per
+// wave, WAVES waves per work-group.  A thread owns whole chunks of 8 consecutive K-slices
+// (32 input channels, one scale group when group-wise), issues its 8 weight loads back to
+// back and prefetches the next chunk while it computes.  Launch shapes are chosen so that a
+// thread usually owns exactly one chunk: then every load of the problem is in flight at
+// once, which is what a ~4 us kernel needs to approach HBM speed.
+// K is reduced across the rows of a wave with lane shuffles, across waves through LDS, and
+// (only when the strip count is too small to fill the chip) across work-groups through a
+// partial-sum workspace that a second small kernel adds up in a fixed order.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "kernels.h"
+
+namespace mldhip {
+namespace {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Reinterprets a 32-bit word as two halfs.  Taking the word by value matters: applying
+// __builtin_bit_cast directly to a vector element reads element 0 whatever the index.
+__device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
+
+struct StreamParams {
+  const u32x4* weights;
+  const __half* act;
+  const __half* scale;
+  const __half* bias;
+  __half* dst;
+  float* partial;
+  int m, ks, ns, n_pad;  // n_pad = ns * 4
+  int row_u4;            // uint4 per packed row = ns / 2
+  int chunks;            // ceil(ks / 8)
+  int chunks_per_split;
+  int ksplit;
+  int group_chunks;  // chunks per scale group (grouped only)
+  int groups;
+};
+
+__device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const __half* bias, size_t bi) {
+  __half h = __float2half_rn(r);
+  if (bias) h = __hadd(h, bias[bi]);
+  dst[i] = h;
+}
+
+template <int M>
+__device__ __forceinline__ void LoadChunk(const StreamParams& p, int c, int pcol, u32x4 w[8],
+                                          u32x2 a[8][M]) {
+  const int ks0 = c * 8;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int ks = ks0 + j;
+    if (ks < p.ks) {
+      w[j] = __builtin_nontemporal_load(p.weights + (size_t)ks * p.row_u4 + pcol);
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+        a[j][m] = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ks * M + m) * 4);
+    } else {
+      // u = 8 everywhere: a zero weight
+      w[j] = u32x4{0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
+#pragma unroll
+      for (int m = 0; m < M; ++m) a[j][m] = u32x2{0u, 0u};
+    }
+  }
+}
+
+// t[m][o] += sum over the chunk of a * (c_o + u), c_o = 1024 for even o, 64 for odd o;
+// asum[m] += sum over the chunk of a.
+template <int M>
+__device__ __forceinline__ void ComputeChunk(const u32x4 w[8], const u32x2 a[8][M], float t[M][8],
+                                             float asum[M]) {
+  const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    half2_t a01[M], a23[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      a01[m] = AsHalf2(a[j][m][0]);
+      a23[m] = AsHalf2(a[j][m][1]);
+      asum[m] = __builtin_amdgcn_fdot2(a01[m], ones, asum[m], false);
+      asum[m] = __builtin_amdgcn_fdot2(a23[m], ones, asum[m], false);
+    }
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {  // word h: inputs (2(h&1), 2(h&1)+1), outputs 4*(h>>1) .. +3
+      const uint32_t lo = w[j][h];
+      const uint32_t hi = lo >> 8;
+      const half2_t q0 = AsHalf2((lo & 0x000F000Fu) | 0x64006400u);
+      const half2_t q1 = AsHalf2((lo & 0x00F000F0u) | 0x54005400u);
+      const half2_t q2 = AsHalf2((hi & 0x000F000Fu) | 0x64006400u);
+      const half2_t q3 = AsHalf2((hi & 0x00F000F0u) | 0x54005400u);
+      const int ob = 4 * (h >> 1);
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const half2_t av = (h & 1) ? a23[m] : a01[m];
+        t[m][ob + 0] = __builtin_amdgcn_fdot2(q0, av, t[m][ob + 0], false);
+        t[m][ob + 1] = __builtin_amdgcn_fdot2(q1, av, t[m][ob + 1], false);
+        t[m][ob + 2] = __builtin_amdgcn_fdot2(q2, av, t[m][ob + 2], false);
+        t[m][ob + 3] = __builtin_amdgcn_fdot2(q3, av, t[m][ob + 3], false);
+      }
+    }
+  }
+}
+
+template <int LPR, int WAVES, int M, bool GROUPED>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
+  constexpr int RPW = 64 / LPR;        // rows per wave
+  constexpr int STRIP = LPR * 8;       // output channels per work-group
+  __shared__ float red[WAVES][M][STRIP];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane % LPR;
+  const int row = wave * RPW + lane / LPR;
+  const int pcol_raw = blockIdx.x * LPR + col;  // uint4 column = output channels 8*pcol .. +7
+  const bool col_ok = pcol_raw < p.row_u4;
+  const int pcol = col_ok ? pcol_raw : p.row_u4 - 1;  // clamp: loads stay in range, result unused
+  const int ky = blockIdx.y;
+  const int c_begin = ky * p.chunks_per_split;
+  const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
+
+  float acc[M][8];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+#pragma unroll
+    for (int o = 0; o < 8; ++o) acc[m][o] = 0.0f;
+
+  int c = c_begin + row;
+  if (c < c_end) {
+    u32x4 w[8];
+    u32x2 a[8][M];
+    LoadChunk<M>(p, c, pcol, w, a);
+    while (true) {
+      const int cn = c + ROWS;
+      const bool more = cn < c_end;
+      u32x4 wn[8];
+      u32x2 an[8][M];
+      if (more) LoadChunk<M>(p, cn, pcol, wn, an);
+      u32x4 sv;
+      if (GROUPED) {
+        int g = c / p.group_chunks;
+        if (g >= p.groups) g = p.groups - 1;
+        sv = *reinterpret_cast<const u32x4*>(p.scale + ((size_t)g * p.ns + 2 * pcol) * 4);
+      }
+      float t[M][8], asum[M];
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        asum[m] = 0.0f;
+#pragma unroll
+        for (int o = 0; o < 8; ++o) t[m][o] = 0.0f;
+      }
+      ComputeChunk<M>(w, a, t, asum);
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+          const float centered = fmaf((o & 1) ? -72.0f : -1032.0f, asum[m], t[m][o]);
+          if (GROUPED) {
+            const half2_t sp = AsHalf2(sv[o >> 1]);
+            acc[m][o] = fmaf((float)sp[o & 1], centered, acc[m][o]);
+          } else {
+            acc[m][o] += centered;
+          }
+        }
+      if (!more) break;
+      c = cn;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        w[j] = wn[j];
+#pragma unroll
+        for (int m = 0; m < M; ++m) a[j][m] = an[j][m];
+      }
+    }
+  }
+
+  // rows of one wave: lanes that differ only in bits >= log2(LPR)
+#pragma unroll
+  for (int off = LPR; off < 64; off <<= 1)
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int o = 0; o < 8; ++o) acc[m][o] += __shfl_xor(acc[m][o], off, 64);
+  if (lane < LPR) {
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int o = 0; o < 8; ++o) red[wave][m][col * 8 + o] = acc[m][o];
+  }
+  __syncthreads();
+
+  const int n0 = blockIdx.x * STRIP;
+  for (int idx = tid; idx < M * STRIP; idx += THREADS) {
+    const int m = idx / STRIP, nl = idx % STRIP;
+    const int n = n0 + nl;
+    if (n >= p.n_pad) continue;
+    float v = 0.0f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][m][nl];
+    if (p.ksplit == 1) {
+      if (!GROUPED) v *= __half2float(p.scale[n]);
+      StoreHalf(p.dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, p.bias, (size_t)n);
+    } else {
+      p.partial[((size_t)ky * M + m) * p.n_pad + n] = v;
+    }
+  }
+}
+
+// Adds the split-K partial sums in split order and writes the output.
+template <bool GROUPED>
+__global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.m * p.n_pad) return;
+  const int m = idx / p.n_pad, n = idx % p.n_pad;
+  float v = 0.0f;
+  for (int s = 0; s < p.ksplit; ++s) v += p.partial[((size_t)s * p.m + m) * p.n_pad + n];
+  if (!GROUPED) v *= __half2float(p.scale[n]);
+  StoreHalf(p.dst, ((size_t)(n >> 2) * p.m + m) * 4 + (n & 3), v, p.bias, (size_t)n);
+}
+
+template <int LPR, int WAVES, int M>
+hipError_t LaunchCfg(const StreamParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  if (grouped)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  else
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false>), grid, dim3(WAVES * 64), 0, stream, p);
+  return hipGetLastError();
+}
+
+template <int LPR, int WAVES>
+hipError_t LaunchCfgM(const StreamParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  switch (p.m) {
+    case 1: return LaunchCfg<LPR, WAVES, 1>(p, grouped, grid, stream);
+    case 2: return LaunchCfg<LPR, WAVES, 2>(p, grouped, grid, stream);
+    case 3: return LaunchCfg<LPR, WAVES, 3>(p, grouped, grid, stream);
+    case 4: return LaunchCfg<LPR, WAVES, 4>(p, grouped, grid, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <int LPR>
+hipError_t LaunchCfgW(const StreamParams& p, int waves, bool grouped, dim3 grid, hipStream_t stream) {
+  switch (waves) {
+    case 4: return LaunchCfgM<LPR, 4>(p, grouped, grid, stream);
+    case 8: return LaunchCfgM<LPR, 8>(p, grouped, grid, stream);
+    default: return LaunchCfgM<LPR, 16>(p, grouped, grid, stream);
+  }
+}
+
+int EnvInt(const char* name, int fallback) {
+  const char* v = std::getenv(name);
+  return v ? std::atoi(v) : fallback;
+}
+
+}  // namespace
+
+bool FcW4StreamSupported(const FcArgs& a) {
+  if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
+  if (a.m < 1 || a.m > kGemvMaxTokens) return false;
+  if (a.has_zero_point) return false;
+  const int ks = DivUp(a.k, 4), ns = DivUp(a.n, 4);
+  if (ns % 2 != 0) return false;  // 16-byte loads need an even number of 8-byte blocks per row
+  if (a.scale_kind == kScaleScalar) return false;
+  if (a.scale_kind == kScaleBlock) {
+    if (a.groups <= 0 || ks % a.groups != 0) return false;
+    if ((ks / a.groups) % 8 != 0) return false;  // a chunk of 8 K-slices must not straddle groups
+  }
+  return a.partial != nullptr;
+}
+
+hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+  StreamParams p;
+  p.weights = reinterpret_cast<const u32x4*>(a.weights);
+  p.act = static_cast<const __half*>(a.act);
+  p.scale = static_cast<const __half*>(a.scale);
+  p.bias = static_cast<const __half*>(a.bias);
+  p.dst = static_cast<__half*>(a.dst);
+  p.partial = a.partial;
+  p.m = a.m;
+  p.ks = DivUp(a.k, 4);
+  p.ns = DivUp(a.n, 4);
+  p.n_pad = p.ns * 4;
+  p.row_u4 = p.ns / 2;
+  p.chunks = DivUp(p.ks, 8);
+  const bool grouped = a.scale_kind == kScaleBlock;
+  p.groups = grouped ? a.groups : 1;
+  p.group_chunks = grouped ? (p.ks / a.groups) / 8 : p.chunks;
+
+  // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the
+  // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous
+  // bytes) keep K inside one work-group for wide layers; when the layer is too narrow for
+  // that, K is split across work-groups and a second kernel adds the partials.
+  int lpr = 8, waves = 16;
+  {
+    // rows needed to cover K in one work-group step
+    const int strips8 = DivUp(p.row_u4, 8);
+    if (strips8 >= 192) {
+      lpr = 8;
+    } else if (DivUp(p.row_u4, 16) >= 192) {
+      lpr = 16;
+    } else {
+      lpr = 8;
+    }
+  }
+  lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
+  if (lpr != 8 && lpr != 16) lpr = 8;
+  waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
+  if (waves != 4 && waves != 8 && waves != 16) waves = 16;
+  const int strips = DivUp(p.row_u4, lpr);
+  int rows = waves * 64 / lpr;
+  // shrink the work-group while it would leave rows without a chunk
+  while (waves > 4 && rows / 2 >= p.chunks) {
+    waves /= 2;
+    rows /= 2;
+  }
+  int ksplit = 1;
+  if (strips < 128) {
+    ksplit = DivUp(256, strips);
+    const int max_split = DivUp(p.chunks, rows);
+    if (ksplit > max_split) ksplit = max_split;
+  }
+  ksplit = EnvInt("MLDHIP_GEMV_KSPLIT", ksplit);
+  if (ksplit > kGemvMaxKSplit) ksplit = kGemvMaxKSplit;
+  if (ksplit < 1) ksplit = 1;
+  while (ksplit > 1 && (size_t)ksplit * p.m * p.n_pad > a.partial_floats) --ksplit;
+  // every thread row gets the same number of chunks
+  p.chunks_per_split = DivUp(DivUp(p.chunks, ksplit), rows) * rows;
+  p.ksplit = DivUp(p.chunks, p.chunks_per_split);
+  dim3 grid(strips, p.ksplit);
+  if (kernel_name) *kernel_name = "fc_w4_stream_kernel";
+  hipError_t e;
+  if (lpr == 8)
+    e = LaunchCfgW<8>(p, waves, grouped, grid, stream);
+  else
+    e = LaunchCfgW<16>(p, waves, grouped, grid, stream);
+  if (e != hipSuccess || p.ksplit == 1) return e;
+  const int total = p.m * p.n_pad;
+  if (grouped)
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace mldhip

@@ -29,17 +29,14 @@ struct FcArgs {
   float scalar_scale = 1.0f;
   bool has_zero_point = false;
   float scalar_zero_point = 0.0f;
-  // private workspace of the op (split-K partial sums and arrival counters)
+  // private workspace of the op (split-K partial sums)
   float* partial = nullptr;
   size_t partial_floats = 0;
-  int* counters = nullptr;
-  int n_counters = 0;
 };
 
 // Split-K workspace sizing for the streaming GEMV.
 constexpr int kGemvMaxTokens = 4;
 constexpr int kGemvMaxKSplit = 32;
-constexpr int kGemvMaxStrips = 4096;
 
 hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 bool FcW4StreamSupported(const FcArgs& a);
