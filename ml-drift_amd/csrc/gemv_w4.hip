@@ -40,6 +40,14 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // __builtin_bit_cast directly to a vector element reads element 0 whatever the index.
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 
+// (x & mask) | magic in one instruction.  The three-operand form reads at most one scalar
+// register, so the mask stays scalar and the exponent pattern lives in a vector register.
+__device__ __forceinline__ uint32_t AndOr(uint32_t x, uint32_t mask, uint32_t magic) {
+  uint32_t d;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "s"(mask), "v"(magic));
+  return d;
+}
+
 struct StreamParams {
   const u32x4* weights;
   const __half* act;
@@ -54,6 +62,9 @@ struct StreamParams {
   int ksplit;
   int group_chunks;  // chunks per scale group (grouped only)
   int groups;
+  // nibble masks and fp16 exponent patterns, passed as run-time values so that the compiler
+  // keeps them in registers and forms single v_and_or_b32 instructions
+  uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
 };
 
 __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const __half* bias, size_t bi) {
@@ -86,8 +97,8 @@ __device__ __forceinline__ void LoadChunk(const StreamParams& p, int c, int pcol
 // t[m][o] += sum over the chunk of a * (c_o + u), c_o = 1024 for even o, 64 for odd o;
 // asum[m] += sum over the chunk of a.
 template <int M>
-__device__ __forceinline__ void ComputeChunk(const u32x4 w[8], const u32x2 a[8][M], float t[M][8],
-                                             float asum[M]) {
+__device__ __forceinline__ void ComputeChunk(const StreamParams& p, const u32x4 w[8], const u32x2 a[8][M],
+                                             float t[M][8], float asum[M]) {
   const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -103,10 +114,10 @@ __device__ __forceinline__ void ComputeChunk(const u32x4 w[8], const u32x2 a[8][
     for (int h = 0; h < 4; ++h) {  // word h: inputs (2(h&1), 2(h&1)+1), outputs 4*(h>>1) .. +3
       const uint32_t lo = w[j][h];
       const uint32_t hi = lo >> 8;
-      const half2_t q0 = AsHalf2((lo & 0x000F000Fu) | 0x64006400u);
-      const half2_t q1 = AsHalf2((lo & 0x00F000F0u) | 0x54005400u);
-      const half2_t q2 = AsHalf2((hi & 0x000F000Fu) | 0x64006400u);
-      const half2_t q3 = AsHalf2((hi & 0x00F000F0u) | 0x54005400u);
+      const half2_t q0 = AsHalf2(AndOr(lo, p.mask_lo, p.magic_lo));
+      const half2_t q1 = AsHalf2(AndOr(lo, p.mask_hi, p.magic_hi));
+      const half2_t q2 = AsHalf2(AndOr(hi, p.mask_lo, p.magic_lo));
+      const half2_t q3 = AsHalf2(AndOr(hi, p.mask_hi, p.magic_hi));
       const int ob = 4 * (h >> 1);
 #pragma unroll
       for (int m = 0; m < M; ++m) {
@@ -126,7 +137,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
   constexpr int RPW = 64 / LPR;        // rows per wave
   constexpr int STRIP = LPR * 8;       // output channels per work-group
-  __shared__ float red[WAVES][M][STRIP];
+  __shared__ float red[ROWS][M][STRIP];
+  __shared__ float red2[(THREADS / STRIP > 0 ? THREADS / STRIP : 1)][M][STRIP];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -170,7 +182,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
 #pragma unroll
         for (int o = 0; o < 8; ++o) t[m][o] = 0.0f;
       }
-      ComputeChunk<M>(w, a, t, asum);
+      ComputeChunk<M>(p, w, a, t, asum);
 #pragma unroll
       for (int m = 0; m < M; ++m)
 #pragma unroll
@@ -194,29 +206,38 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
     }
   }
 
-  // rows of one wave: lanes that differ only in bits >= log2(LPR)
+  // K reduction inside the work-group, through LDS only: every thread stores its 8*M sums,
+  // PARTS threads per output add ROWS/PARTS rows each, then one thread per output adds the
+  // PARTS results.
+  constexpr int PARTS = THREADS / STRIP >= 1 ? (THREADS / STRIP > ROWS ? ROWS : THREADS / STRIP) : 1;
+  constexpr int RPP = ROWS / PARTS;  // rows per part
 #pragma unroll
-  for (int off = LPR; off < 64; off <<= 1)
-#pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-      for (int o = 0; o < 8; ++o) acc[m][o] += __shfl_xor(acc[m][o], off, 64);
-  if (lane < LPR) {
-#pragma unroll
-    for (int m = 0; m < M; ++m)
-#pragma unroll
-      for (int o = 0; o < 8; ++o) red[wave][m][col * 8 + o] = acc[m][o];
+  for (int m = 0; m < M; ++m) {
+    float4* dst4 = reinterpret_cast<float4*>(&red[row][m][col * 8]);
+    dst4[0] = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+    dst4[1] = make_float4(acc[m][4], acc[m][5], acc[m][6], acc[m][7]);
   }
   __syncthreads();
-
+  const int nl = tid % STRIP;
+  const int part = tid / STRIP;
+  if (part < PARTS) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float v = 0.0f;
+#pragma unroll
+      for (int r = 0; r < RPP; ++r) v += red[part * RPP + r][m][nl];
+      red2[part][m][nl] = v;
+    }
+  }
+  __syncthreads();
   const int n0 = blockIdx.x * STRIP;
   for (int idx = tid; idx < M * STRIP; idx += THREADS) {
-    const int m = idx / STRIP, nl = idx % STRIP;
-    const int n = n0 + nl;
+    const int m = idx / STRIP, ol = idx % STRIP;
+    const int n = n0 + ol;
     if (n >= p.n_pad) continue;
     float v = 0.0f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][m][nl];
+    for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
     if (p.ksplit == 1) {
       if (!GROUPED) v *= __half2float(p.scale[n]);
       StoreHalf(p.dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, p.bias, (size_t)n);
@@ -305,6 +326,10 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   const bool grouped = a.scale_kind == kScaleBlock;
   p.groups = grouped ? a.groups : 1;
   p.group_chunks = grouped ? (p.ks / a.groups) / 8 : p.chunks;
+  p.mask_lo = 0x000F000Fu;
+  p.mask_hi = 0x00F000F0u;
+  p.magic_lo = 0x64006400u;
+  p.magic_hi = 0x54005400u;
 
   // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the
   // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous

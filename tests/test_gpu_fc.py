@@ -118,6 +118,15 @@ def test_stream_kernel_shapes(oracle, lpr, waves, ksplit):
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("groups", [1, 32])
+def test_stream_kernel_variants_ragged(oracle, m, groups):
+    # N = 8*129: the last 4-column block of the strip is partly outside the matrix
+    case = W.make_fc_case(seed=17 + m, m=m, k=1024, n=1032, weight_bits=4, tensor_dtype=np.float16,
+                          groups=groups, with_bias=True)
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
 @pytest.mark.parametrize("groups", [1, 64])
 def test_stream_kernel_tokens_and_groups(oracle, m, groups):
     case = W.make_fc_case(seed=5 + m, m=m, k=2048, n=2048, weight_bits=4, tensor_dtype=np.float16,
