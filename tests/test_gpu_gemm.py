@@ -1,0 +1,162 @@
+"""GPU parity of the prefill-side MFMA kernels, through the C-ABI.
+
+int4 GEMM (fp16 out): max|err| <= 2e-2 * RMS(reference output) against the textbook reference
+over dequantised weights and, at sizes the oracle finishes quickly, against the restatement
+of the reference's generated kernel.
+int8 x int8: int32 accumulators bit-exact against the closed-form integer product; the
+rescaled fp16 output is compared with the oracle's epilogue applied to the same accumulators."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mldhip as M
+import workloads as W
+from test_gpu_fc import check_fp, oracle_fc, textbook
+
+FP16_TOL = 2e-2
+
+
+def run_w4(case):
+    print("w4 gemm", {k: case[k] for k in ("m", "k", "n", "groups")}, flush=True)
+    dev = W.FcDevice(case)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_mfma_gemm_kernel", dev.op.kernel_name
+    dev.run()
+    assert np.array_equal(got, dev.result())
+    return got
+
+
+@pytest.mark.parametrize("m,k,n,groups", [(16, 256, 128, 8), (5, 64, 8, 1), (128, 2048, 2048, 64),
+                                          (77, 352, 200, 11), (130, 96, 260, 1), (64, 4096, 256, 128),
+                                          (300, 1024, 1024, 8)])
+def test_w4_gemm_shapes(oracle, m, k, n, groups):
+    case = W.make_fc_case(seed=m + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=(m % 2 == 1))
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    if m * k * n <= 1 << 26:
+        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+
+
+def test_config3_prefill_gemm(oracle):
+    case = W.make_fc_case(**W.CONFIGS["c3"])
+    got = run_w4(case)
+    rel = check_fp(got, textbook(case), case, "textbook")
+    print("c3 max|err|/rms = %.3e" % rel)
+    # a slab of outputs against the restatement of the generated kernel
+    sub = dict(case, n=64, w=case["w"][:64], scale=case["scale"][:64])
+    ref = oracle_fc(oracle, sub).astype(np.float64)
+    rms = np.sqrt(np.mean(ref ** 2))
+    assert np.abs(got[:, :64] - ref).max() <= FP16_TOL * rms
+
+
+def test_config5_prefill_shapes(oracle):
+    for name, k, n in W.C5_LAYER:
+        case = W.make_fc_case(seed=9, m=128, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=k // 32)
+        got = run_w4(case)
+        check_fp(got, textbook(case), case, name)
+
+
+def make_int8_case(seed, m, k, n, with_zp=False, with_bias=False):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    w = rng.integers(-127, 128, size=(n, k), dtype=np.int8)
+    ws = (np.abs(rng.normal(0, 0.02, size=n)) / 127).astype(np.float32)
+    wzp = rng.integers(-4, 5, size=n).astype(np.float32) if with_zp else None
+    bias = (rng.uniform(-1, 1, size=n) * 0.1).astype(np.float16) if with_bias else None
+    return dict(m=m, k=k, n=n, x=x, w=w, ws=ws, wzp=wzp, bias=bias)
+
+
+def pad4(a, dtype):
+    a = np.asarray(a, dtype).ravel()
+    out = np.zeros((a.size + 3) // 4 * 4, dtype)
+    out[:a.size] = a
+    return out
+
+
+def run_int8_pipeline(oracle, c, symmetric):
+    """quantize (GPU) -> int8 MFMA conv (GPU): returns codes, params, int32 acc, fp16 out."""
+    import torch
+    m, k, n = c["m"], c["k"], c["n"]
+    print("int8 pipeline", m, k, n, symmetric, flush=True)
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.from_numpy(W.to_slices(c["x"])).cuda()
+    k16 = (k + 15) // 16
+    codes = torch.zeros((k16, m, 16), dtype=torch.int8, device="cuda")
+    params = torch.zeros((m, 4), dtype=torch.float32, device="cuda")
+    q = M.quantization_create(M.FLOAT16, M.PACKED_INT8C16, k, calculate_sum=True, symmetric=symmetric, max_tokens=m)
+    q.bind([src], [codes, params])
+    q.set_shape(1, 1, m)
+    q.launch(stream)
+    wd = M.conv_int8_weights_desc(n, k)
+    wt = torch.from_numpy(M.rearrange_int8(c["w"], wd)).cuda()
+    ns = (n + 3) // 4
+    acc = torch.zeros((ns, m, 4), dtype=torch.int32, device="cuda")
+    conv_raw = M.conv_int8_create(M.INT32, n, k, wd, max_tokens=m)
+    conv_raw.bind([codes, wt], [acc])
+    conv_raw.set_shape(1, 1, m)
+    conv_raw.launch(stream)
+    wsum = torch.from_numpy(pad4(M.weights_sum_i(c["w"]), np.int32)).cuda()
+    wscale = torch.from_numpy(pad4(c["ws"], np.float32)).cuda()
+    srcs = [codes, wt, params, wsum, wscale]
+    if c["wzp"] is not None:
+        srcs.append(torch.from_numpy(pad4(c["wzp"], np.float32)).cuda())
+    if c["bias"] is not None:
+        srcs.append(torch.from_numpy(pad4(c["bias"], np.float16)).cuda())
+    out = torch.zeros((ns, m, 4), dtype=torch.float16, device="cuda")
+    conv = M.conv_int8_create(M.FLOAT16, n, k, wd, has_zero_point=c["wzp"] is not None,
+                              has_bias=c["bias"] is not None, max_tokens=m)
+    conv.bind(srcs, [out])
+    conv.set_shape(1, 1, m)
+    conv.launch(stream)
+    torch.cuda.synchronize()
+    assert conv.kernel_name == "conv_int8_mfma_kernel"
+    return codes.cpu().numpy(), params.cpu().numpy(), acc.cpu().numpy(), out.cpu().numpy()
+
+
+def check_int8(oracle, c, symmetric):
+    o = oracle
+    m, k, n = c["m"], c["k"], c["n"]
+    codes, params, acc, out = run_int8_pipeline(o, c, symmetric)
+    # activation codes and params: bit-exact
+    src_bits = o.f32_to_f16_bits(W.to_slices(c["x"]).astype(np.float32))
+    rcodes, rparams = o.quantize(src_bits, m, k, o.PACKED_INT8C16, symmetric, True)
+    assert np.array_equal(codes, rcodes)
+    assert np.array_equal(params.view(np.uint32), rparams.view(np.uint32))
+    # int32 accumulators: exact integer product
+    q = rcodes.transpose(1, 0, 2).reshape(m, -1)[:, :k]
+    ref_acc = q.astype(np.int64) @ c["w"].astype(np.int64).T
+    assert np.array_equal(W.from_slices(acc, n).astype(np.int64), ref_acc)
+    if m * k * n <= 1 << 24:
+        assert np.array_equal(ref_acc, o.fc_reference_i8(q, c["w"]))
+    # rescaled output: the oracle's epilogue on the same accumulators
+    ref_out = o.dequantize(W.to_slices(ref_acc.astype(np.int32)), rparams, o.weights_sum_i(c["w"]), c["ws"], n, k,
+                           weights_zero_point=c["wzp"],
+                           bias=None if c["bias"] is None else c["bias"].view(np.uint16), dst_f16=True)
+    ref_f = W.from_slices(o.f16_bits_to_f32(ref_out), n)
+    got_f = W.from_slices(out.astype(np.float32), n)
+    rms = np.sqrt(np.mean(ref_f.astype(np.float64) ** 2))
+    assert np.abs(got_f - ref_f).max() <= FP16_TOL * rms
+    mismatch = np.count_nonzero(out.view(np.uint16).ravel()[: ref_out.size] != ref_out.ravel())
+    print("fp16 outputs differing from the oracle bit pattern: %d of %d" % (mismatch, ref_out.size))
+    # and against the float product of the de-quantised operands (what the epilogue stands for)
+    a_deq = q.astype(np.float64) * rparams[:, 0:1] + rparams[:, 1:2]
+    w_deq = c["w"].astype(np.float64) * c["ws"][:, None] + (0 if c["wzp"] is None else c["wzp"][:, None])
+    exact = a_deq @ w_deq.T + (0 if c["bias"] is None else c["bias"].astype(np.float64))
+    assert np.abs(got_f - exact).max() <= FP16_TOL * np.sqrt(np.mean(exact ** 2))
+    return mismatch
+
+
+@pytest.mark.parametrize("m,k,n", [(32, 64, 32), (7, 48, 20), (128, 512, 384), (200, 1000, 300), (300, 2048, 512)])
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_int8_conv_shapes(oracle, m, k, n, symmetric):
+    c = make_int8_case(m + n, m, k, n, with_zp=(m % 2 == 1), with_bias=(n % 3 == 0))
+    check_int8(oracle, c, symmetric)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_config4_int8_gemm(oracle, symmetric):
+    c = make_int8_case(0, 2048, 2048, 8192)
+    check_int8(oracle, c, symmetric)
