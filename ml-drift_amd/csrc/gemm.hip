@@ -60,6 +60,9 @@ struct GemmParams {
   const int32_t* wsum;
   const float* wscale;
   const float* wzp;
+  // byte sizes of the A (weights), B (activations / codes) and scale buffers
+  uint32_t a_bytes, b_bytes, s_bytes;
+  int group_size;  // input channels per scale group (fp16 path)
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -94,7 +97,7 @@ __device__ __forceinline__ float Rescale(int acc, float ws, int wsum, float src_
 }
 #pragma clang fp contract(fast)
 
-template <bool W4, int FN, int FM>
+template <bool W4, int FN, int FM, int D>  // D: register stages, even
 __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
   constexpr int BN = 2 * FN * 32;
   constexpr int BM = 2 * FM * 32;
@@ -116,11 +119,26 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
   constexpr int B_ITEMS = W4 ? (KG * 2) * BM : KG * BM;
   constexpr int NA = (A_ITEMS + kThreads - 1) / kThreads;
   constexpr int NB = (B_ITEMS + kThreads - 1) / kThreads;
-  u32x4 ra[NA];  // fp16 path: {blk0.x, blk0.y, blk1.x, blk1.y}
-  u32x2 rs[NA];  // fp16 path: the 4 scales of the item's slice
-  u32x4 rb[NB];  // fp16 path uses .xy only
+  // D register stages: tile t is fetched D K-steps before it is multiplied, so D-1 tiles of
+  // global loads are in flight while the MFMAs of the current tile run.
+  u32x4 ra_[D][NA];  // fp16 path: {blk0.x, blk0.y, blk1.x, blk1.y}
+  u32x2 rs_[D][NA];  // fp16 path: the 4 scales of the item's slice
+  u32x4 rb_[D][W4 ? 1 : NB];
+  u32x2 rb2_[D][W4 ? NB : 1];  // fp16 path: 8-byte activation items
 
-  auto load_tiles = [&](int kt) {
+  // All tile loads are raw buffer loads: out-of-range items get an offset beyond the buffer and
+  // read as zero, so the loop body stays free of branches and the loads of several stages stay
+  // in flight (a zero activation or a zero scale makes the padded product vanish).
+  constexpr uint32_t kOob = 0x7FFFFFF0u;
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void*>(W4 ? static_cast<const void*>(p.w4) : static_cast<const void*>(p.wi8)), 0, p.a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void*>(W4 ? static_cast<const void*>(p.act) : static_cast<const void*>(p.codes)), 0, p.b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_s =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
+
+  auto load_tiles = [&](int kt, u32x4 (&ra)[NA], u32x2 (&rs)[NA], u32x4 (&rb)[W4 ? 1 : NB],
+                        u32x2 (&rb2)[W4 ? NB : 1]) {
     if (W4) {
 #pragma unroll
       for (int q = 0; q < NA; ++q) {
@@ -128,25 +146,15 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
         const int g = it / (BN / 4), nsl = it % (BN / 4);
         const int nsi = n0 / 4 + nsl;
         const int ksa = (kt * KG + g) * 2;
-        u32x4 v = {0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-        u32x2 sc = {0u, 0u};
-        if (it < A_ITEMS && nsi < p.ns) {
-          if (ksa < p.ks) {
-            const u32x2 b0 = *reinterpret_cast<const u32x2*>(p.w4 + ((size_t)ksa * p.ns + nsi) * 8);
-            v[0] = b0[0];
-            v[1] = b0[1];
-          }
-          if (ksa + 1 < p.ks) {
-            const u32x2 b1 = *reinterpret_cast<const u32x2*>(p.w4 + ((size_t)(ksa + 1) * p.ns + nsi) * 8);
-            v[2] = b1[0];
-            v[3] = b1[1];
-          }
-          int grp = kt / p.steps_per_group;
-          if (grp >= p.groups) grp = p.groups - 1;
-          sc = *reinterpret_cast<const u32x2*>(p.scale + ((size_t)grp * p.ns + nsi) * 4);
-        }
-        ra[q] = v;
-        rs[q] = sc;
+        const bool ok = it < A_ITEMS && nsi < p.ns;
+        const uint32_t off0 = ok ? (uint32_t)(ksa * p.ns + nsi) * 8u : kOob;
+        const uint32_t off1 = ok ? off0 + (uint32_t)p.ns * 8u : kOob;
+        const u32x2 b0 = __builtin_amdgcn_raw_buffer_load_b64(rsrc_a, off0, 0, 0);
+        const u32x2 b1 = __builtin_amdgcn_raw_buffer_load_b64(rsrc_a, off1, 0, 0);
+        ra[q] = u32x4{b0[0], b0[1], b1[0], b1[1]};
+        int grp = kt / p.steps_per_group;
+        grp = grp < p.groups ? grp : p.groups - 1;
+        rs[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, ok ? (uint32_t)(grp * p.ns + nsi) * 8u : kOob, 0, 0);
       }
 #pragma unroll
       for (int q = 0; q < NB; ++q) {
@@ -154,10 +162,8 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
         const int ksl = it / BM, ml = it % BM;
         const int ksi = kt * KG * 2 + ksl;
         const int mi = m0 + ml;
-        u32x2 v = {0u, 0u};
-        if (it < B_ITEMS && ksi < p.ks && mi < p.m)
-          v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksi * p.m + mi) * 4);
-        rb[q] = u32x4{v[0], v[1], 0u, 0u};
+        const bool ok = it < B_ITEMS && mi < p.m;
+        rb2[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, ok ? (uint32_t)(ksi * p.m + mi) * 8u : kOob, 0, 0);
       }
     } else {
 #pragma unroll
@@ -165,23 +171,22 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
         const int it = tid + q * kThreads;
         const int g = it / BN, r = it % BN;
         const int kg = kt * KG + g;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (it < A_ITEMS && kg < p.k16 && n0 + r < p.n) v = p.wi8[(size_t)kg * p.n + n0 + r];
-        ra[q] = v;
+        const bool ok = it < A_ITEMS && n0 + r < p.n;
+        ra[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? (uint32_t)(kg * p.n + n0 + r) * 16u : kOob, 0, 0);
       }
 #pragma unroll
       for (int q = 0; q < NB; ++q) {
         const int it = tid + q * kThreads;
         const int g = it / BM, r = it % BM;
         const int kg = kt * KG + g;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (it < B_ITEMS && kg < p.k16 && m0 + r < p.m) v = p.codes[(size_t)kg * p.m + m0 + r];
-        rb[q] = v;
+        const bool ok = it < B_ITEMS && m0 + r < p.m;
+        rb[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? (uint32_t)(kg * p.m + m0 + r) * 16u : kOob, 0, 0);
       }
     }
   };
 
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int buf, u32x4 (&ra)[NA], u32x2 (&rs)[NA], u32x4 (&rb)[W4 ? 1 : NB],
+                         u32x2 (&rb2)[W4 ? NB : 1]) {
     if (W4) {
       const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
       const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
         if (it >= B_ITEMS) continue;
         const int ksl = it / BM, ml = it % BM;
         u32x2* dst2 = reinterpret_cast<u32x2*>(&sB[buf][ksl >> 1][ml]) + (ksl & 1);
-        *dst2 = u32x2{rb[q][0], rb[q][1]};
+        *dst2 = rb2[q];
       }
     } else {
 #pragma unroll
@@ -244,34 +249,46 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
           acci[fn][fm][v] = 0;
       }
 
-  load_tiles(0);
-  store_tiles(0);
+  // prologue: tiles 0 .. D-1 into the register stages, tile 0 on into LDS.  The loop below
+  // has no conditions: it runs a multiple of D steps, tiles beyond K read as zeros (buffer
+  // range check) and add nothing.
+#pragma unroll
+  for (int d = 0; d < D; ++d) load_tiles(d, ra_[d], rs_[d], rb_[d], rb2_[d]);
+  store_tiles(0, ra_[0], rs_[0], rb_[0], rb2_[0]);
   __syncthreads();
-  for (int kt = 0; kt < p.k_steps; ++kt) {
-    const int buf = kt & 1;
-    const bool more = kt + 1 < p.k_steps;
-    if (more) load_tiles(kt + 1);
+  const int k_steps_padded = (p.k_steps + D - 1) / D * D;
+  for (int kt0 = 0; kt0 < k_steps_padded; kt0 += D) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      u32x4 a[FN], b[FM];
+    for (int d = 0; d < D; ++d) {
+      const int kt = kt0 + d;
+      const int buf = d & 1;  // D is even, so the LDS buffer of a stage is fixed
+      // stage d held tile kt (already in LDS): refill it with tile kt + D
+      load_tiles(kt + D, ra_[d], rs_[d], rb_[d], rb2_[d]);
 #pragma unroll
-      for (int fn = 0; fn < FN; ++fn) a[fn] = sA[buf][2 * s + g2][(wn * FN + fn) * 32 + r32];
+      for (int s = 0; s < 2; ++s) {
+        u32x4 a[FN], b[FM];
 #pragma unroll
-      for (int fm = 0; fm < FM; ++fm) b[fm] = sB[buf][2 * s + g2][(wm * FM + fm) * 32 + r32];
+        for (int fn = 0; fn < FN; ++fn) a[fn] = sA[buf][2 * s + g2][(wn * FN + fn) * 32 + r32];
 #pragma unroll
-      for (int fn = 0; fn < FN; ++fn)
+        for (int fm = 0; fm < FM; ++fm) b[fm] = sB[buf][2 * s + g2][(wm * FM + fm) * 32 + r32];
 #pragma unroll
-        for (int fm = 0; fm < FM; ++fm) {
-          if (W4)
-            accf[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(half8_t, a[fn]), __builtin_bit_cast(half8_t, b[fm]), accf[fn][fm], 0, 0, 0);
-          else
-            acci[fn][fm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                __builtin_bit_cast(int4v_t, a[fn]), __builtin_bit_cast(int4v_t, b[fm]), acci[fn][fm], 0, 0, 0);
-        }
+        for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm) {
+            if (W4)
+              accf[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(half8_t, a[fn]), __builtin_bit_cast(half8_t, b[fm]), accf[fn][fm], 0, 0, 0);
+            else
+              acci[fn][fm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                  __builtin_bit_cast(int4v_t, a[fn]), __builtin_bit_cast(int4v_t, b[fm]), acci[fn][fm], 0, 0, 0);
+          }
+      }
+      {
+        const int dn = (d + 1) % D;
+        store_tiles(buf ^ 1, ra_[dn], rs_[dn], rb_[dn], rb2_[dn]);
+      }
+      __syncthreads();
     }
-    if (more) store_tiles(buf ^ 1);
-    __syncthreads();
   }
 
   // ---- epilogue ---------------------------------------------------------------------------
@@ -337,6 +354,176 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// int4 prefill GEMM without LDS in the main loop.
+//
+// Work-group = 4 waves on one output tile of 128 channels x (FM*32) tokens; the waves split K
+// four ways and add their fp32 tiles through LDS at the end (fixed order).  Inside a wave every
+// MFMA operand comes straight from global memory in the layout the instruction wants:
+//  - A (weights): the 32 "rows" of MFMA number t are the output channels 4*i + t, i = lane % 32,
+//    so a lane's two 8-byte blocks (K-slices 2q, 2q+1 of slice i; 8 input channels x 4 output
+//    channels) dequantize to exactly its A operands for t = 0..3.  No transposition, and each
+//    weight is dequantized once per wave: fp16 round((u-8)*s) with two packed ops per pair.
+//  - B (activations): column j = token; a lane's 8 halfs are the two 8-byte slices
+//    [2q][token][4], [2q+1][token][4] of the slice-major tensor.
+// In the 32x32 result, register v of lane j holds row 8*(v/4) + 4*(lane/32) + v%4 = slice i, so
+// the 4 MFMAs t = 0..3 together hold one whole 4-channel output slice per (v, token): one
+// 8-byte store.  Loads are raw buffer loads (out-of-range reads as zero), U steps ahead.
+// ------------------------------------------------------------------------------------------
+template <int FM, int U>
+__global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams p) {
+  constexpr int BN = 128;
+  constexpr int BM = FM * 32;
+  constexpr int kTileFloats = 4 * FM * 16 * 64;  // one wave's accumulators
+  __shared__ float red[2][kTileFloats];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int i32 = lane & 31, g2 = lane >> 5;
+  const int n0 = blockIdx.x * BN;
+  const int m0 = blockIdx.y * BM;
+  const int nsi = n0 / 4 + i32;
+  const bool n_ok = nsi < p.ns;
+
+  constexpr uint32_t kOob = 0x7FFFFFF0u;
+  const __amdgpu_buffer_rsrc_t rsrc_w =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w4), 0, p.a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_x =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, p.b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_s =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
+
+  // this wave's range of 16-channel steps
+  const int steps_total = (p.k + 15) / 16;
+  const int per_wave = ((steps_total + 3) / 4 + U - 1) / U * U;  // multiple of U
+  const int t_begin = wave * per_wave;
+
+  uint32_t tok_off[FM];  // byte offset of this lane's token inside one K-slice row, or out of range
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) {
+    const int mi = m0 + fm * 32 + i32;
+    tok_off[fm] = mi < p.m ? (uint32_t)mi * 8u : kOob;
+  }
+  const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
+  const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
+
+  u32x2 rw[U][2], rsc[U], rx[U][FM][2];
+  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2 (&x)[FM][2]) {
+    // steps beyond this wave's share read nothing: the limit is the next wave's first step
+    const bool live = t < t_begin + per_wave;
+    const uint32_t ksa = (uint32_t)(t * 2 + g2) * 2u;
+    const bool w_ok = live && n_ok;
+    const uint32_t wo = w_ok ? ksa * row_w + (uint32_t)nsi * 8u : kOob;
+    w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, wo, 0, 0);
+    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_ok ? wo + row_w : kOob, 0, 0);
+    int grp = (t * 16) / p.group_size;
+    grp = grp < p.groups ? grp : p.groups - 1;
+    sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, n_ok ? (uint32_t)(grp * p.ns + nsi) * 8u : kOob, 0, 0);
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+      const bool x_ok = live && tok_off[fm] != kOob;
+      const uint32_t xo = x_ok ? ksa * row_x + tok_off[fm] : kOob;
+      x[fm][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, xo, 0, 0);
+      x[fm][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, x_ok ? xo + row_x : kOob, 0, 0);
+    }
+  };
+
+  float16_t acc[4][FM];
+#pragma unroll
+  for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t4][fm][v] = 0.0f;
+
+  const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+  const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+
+#pragma unroll
+  for (int u = 0; u < U; ++u) load_step(t_begin + u, rw[u], rsc[u], rx[u]);
+  for (int tt = 0; tt < per_wave; tt += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int t = t_begin + tt + u;
+      // consume stage u
+      const u32x4 blk = {rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
+      const u32x2 sc = rsc[u];
+      u32x4 bop[FM];
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) bop[fm] = u32x4{rx[u][fm][0][0], rx[u][fm][0][1], rx[u][fm][1][0], rx[u][fm][1][1]};
+      // refill stage u with step t + U
+      load_step(t + U, rw[u], rsc[u], rx[u]);
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) {
+        const uint32_t sw = sc[t4 >> 1];
+        const uint32_t s16 = (t4 & 1) ? (sw >> 16) : (sw & 0xFFFFu);
+        const half2_t s2 = AsHalf2(s16 | (s16 << 16));
+        u32x4 aop;
+#pragma unroll
+        for (int wd = 0; wd < 4; ++wd) {
+          const uint32_t x = (t4 & 2) ? (blk[wd] >> 8) : blk[wd];
+          const uint32_t bits = (t4 & 1) ? AndOr(x, p.mask_hi, p.magic_hi) : AndOr(x, p.mask_lo, p.magic_lo);
+          aop[wd] = AsU32((AsHalf2(bits) + ((t4 & 1) ? off_hi : off_lo)) * s2);
+        }
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+          acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
+                                                               __builtin_bit_cast(half8_t, bop[fm]), acc[t4][fm], 0, 0, 0);
+      }
+    }
+  }
+
+  // K-split reduction: waves 2,3 -> LDS, waves 0,1 add; wave 1 -> LDS, wave 0 adds.
+  auto spill = [&](float* dst) {
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[((t4 * FM + fm) * 16 + v) * 64 + lane] = acc[t4][fm][v];
+  };
+  auto absorb = [&](const float* src) {
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t4][fm][v] += src[((t4 * FM + fm) * 16 + v) * 64 + lane];
+  };
+  if (wave >= 2) spill(red[wave - 2]);
+  __syncthreads();
+  if (wave < 2) absorb(red[wave]);
+  __syncthreads();
+  if (wave == 1) spill(red[0]);
+  __syncthreads();
+  if (wave != 0) return;
+  absorb(red[0]);
+
+  const __half* bias = static_cast<const __half*>(p.bias);
+  __half* dst = static_cast<__half*>(p.dst);
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) {
+    const int mi = m0 + fm * 32 + i32;
+    if (mi >= p.m) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
+      if (slice >= p.ns) continue;
+      __half h[4];
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) {
+        h[t4] = __float2half_rn(acc[t4][fm][v]);
+        if (bias) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
+      }
+      u32x2 o;
+      o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+      o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+      *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+    }
+  }
+}
+
 template <bool W4>
 hipError_t LaunchGemm(const GemmParams& p, hipStream_t stream) {
   // Tile choice: the largest work-group tile that still gives every CU a work-group;
@@ -345,16 +532,16 @@ hipError_t LaunchGemm(const GemmParams& p, hipStream_t stream) {
   auto groups = [&](int bn, int bm) { return (long)DivUp(p.n, bn) * DivUp(p.m, bm); };
   const long want = 200;
   if (groups(256, 256) >= want) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 4>), dim3(DivUp(p.n, 256), DivUp(p.m, 256)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 4, 2>), dim3(DivUp(p.n, 256), DivUp(p.m, 256)), dim3(kThreads), 0,
                        stream, p);
   } else if (groups(256, 128) >= want) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 2>), dim3(DivUp(p.n, 256), DivUp(p.m, 128)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 2, (W4 ? 6 : 4)>), dim3(DivUp(p.n, 256), DivUp(p.m, 128)), dim3(kThreads), 0,
                        stream, p);
   } else if (groups(128, 128) >= want || p.m > 64) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 2>), dim3(DivUp(p.n, 128), DivUp(p.m, 128)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 2, (W4 ? 8 : 6)>), dim3(DivUp(p.n, 128), DivUp(p.m, 128)), dim3(kThreads), 0,
                        stream, p);
   } else {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 1>), dim3(DivUp(p.n, 128), DivUp(p.m, 64)), dim3(kThreads), 0,
+    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 1, (W4 ? 8 : 6)>), dim3(DivUp(p.n, 128), DivUp(p.m, 64)), dim3(kThreads), 0,
                        stream, p);
   }
   return hipGetLastError();
@@ -366,9 +553,12 @@ bool FcW4MfmaSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
   if (a.has_zero_point || a.scale_kind == kScaleScalar) return false;
   if (a.m <= kGemvMaxTokens) return false;
+  // 32-bit buffer offsets
+  if ((size_t)DivUp(a.k, 4) * DivUp(a.n, 4) * 8 >= 0x7FFFFFF0u || (size_t)DivUp(a.k, 4) * a.m * 8 >= 0x7FFFFFF0u)
+    return false;
   if (a.scale_kind == kScaleBlock) {
-    // a K-step of 32 input channels must not straddle scale groups
-    if (a.groups <= 0 || a.k % a.groups != 0 || (a.k / a.groups) % 32 != 0) return false;
+    // an MFMA step of 16 input channels must not straddle scale groups
+    if (a.groups <= 0 || a.k % a.groups != 0 || (a.k / a.groups) % 16 != 0) return false;
   }
   return true;
 }
@@ -393,8 +583,21 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   p.mask_hi = 0x00F000F0u;
   p.magic_lo = 0x64006400u;
   p.magic_hi = 0x54005400u;
+  p.a_bytes = (uint32_t)((size_t)p.ks * p.ns * 8);
+  p.b_bytes = (uint32_t)((size_t)p.ks * p.m * 8);
+  p.s_bytes = (uint32_t)((size_t)p.groups * p.ns * 8);
+  p.group_size = a.scale_kind == kScaleBlock ? a.k / a.groups : a.k;
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
-  return LaunchGemm<true>(p, stream);
+  // token tile: 64 when that still yields a work-group per CU or M is large, else 32
+  const long tiles64 = (long)DivUp(a.n, 128) * DivUp(a.m, 64);
+  if (a.m > 32 && (tiles64 >= 128 || a.m > 64)) {
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4>), dim3(DivUp(a.n, 128), DivUp(a.m, 64)), dim3(kThreads), 0,
+                       stream, p);
+  } else {
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4>), dim3(DivUp(a.n, 128), DivUp(a.m, 32)), dim3(kThreads), 0,
+                       stream, p);
+  }
+  return hipGetLastError();
 }
 
 hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char** kernel_name) {
@@ -414,6 +617,10 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
   p.wsum = a.weights_sum;
   p.wscale = a.weights_scale;
   p.wzp = a.weights_zero_point;
+  if ((size_t)p.k16 * p.n * 16 >= 0x7FFFFFF0u || (size_t)p.k16 * p.m * 16 >= 0x7FFFFFF0u) return hipErrorInvalidValue;
+  p.a_bytes = (uint32_t)((size_t)p.k16 * p.n * 16);
+  p.b_bytes = (uint32_t)((size_t)p.k16 * p.m * 16);
+  p.s_bytes = 0;
   if (kernel_name) *kernel_name = "conv_int8_mfma_kernel";
   return LaunchGemm<false>(p, stream);
 }
