@@ -20,6 +20,8 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "../../include/mldhip.h"
 #include "kernels.h"
 
@@ -62,7 +64,9 @@ struct GemmParams {
   const float* wzp;
   // byte sizes of the A (weights), B (activations / codes) and scale buffers
   uint32_t a_bytes, b_bytes, s_bytes;
-  int group_size;  // input channels per scale group (fp16 path)
+  int group_size;   // input channels per scale group (fp16 path)
+  int group_shift;  // log2(group_size / 16) when that is a power of two, else -1
+  int debug;
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -370,8 +374,8 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
 // the 4 MFMAs t = 0..3 together hold one whole 4-channel output slice per (v, token): one
 // 8-byte store.  Loads are raw buffer loads (out-of-range reads as zero), U steps ahead.
 // ------------------------------------------------------------------------------------------
-template <int FM, int U>
-__global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams p) {
+template <int FM, int U, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
   constexpr int kTileFloats = 4 * FM * 16 * 64;  // one wave's accumulators
@@ -381,8 +385,17 @@ __global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams 
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int i32 = lane & 31, g2 = lane >> 5;
-  const int n0 = blockIdx.x * BN;
-  const int m0 = blockIdx.y * BM;
+  // XCD-aware tile order.  Work-groups go round-robin to the 8 XCDs (id % 8), each with its own
+  // L2.  Tiles are numbered token-tile-major and XCD x takes the contiguous range
+  // [x*per_xcd, (x+1)*per_xcd): the work-groups that share an L2 then share a few activation
+  // tiles (the big fp16 operand), and every weight tile streams through that L2 once.
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const int tiles_m = (p.m + BM - 1) / BM;
+  const int per_xcd = (tiles_n * tiles_m + 7) / 8;
+  const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= tiles_n * tiles_m) return;
+  const int n0 = (tile % tiles_n) * BN;
+  const int m0 = (tile / tiles_n) * BM;
   const int nsi = n0 / 4 + i32;
   const bool n_ok = nsi < p.ns;
 
@@ -396,7 +409,7 @@ __global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams 
 
   // this wave's range of 16-channel steps
   const int steps_total = (p.k + 15) / 16;
-  const int per_wave = ((steps_total + 3) / 4 + U - 1) / U * U;  // multiple of U
+  const int per_wave = ((steps_total + WAVES - 1) / WAVES + U - 1) / U * U;  // multiple of U
   const int t_begin = wave * per_wave;
 
   uint32_t tok_off[FM];  // byte offset of this lane's token inside one K-slice row, or out of range
@@ -417,7 +430,8 @@ __global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams 
     const uint32_t wo = w_ok ? ksa * row_w + (uint32_t)nsi * 8u : kOob;
     w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, wo, 0, 0);
     w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_ok ? wo + row_w : kOob, 0, 0);
-    int grp = (t * 16) / p.group_size;
+    // scale group of this step: a shift when the group holds a power-of-two number of steps
+    int grp = p.group_shift >= 0 ? (t >> p.group_shift) : (t * 16) / p.group_size;
     grp = grp < p.groups ? grp : p.groups - 1;
     sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, n_ok ? (uint32_t)(grp * p.ns + nsi) * 8u : kOob, 0, 0);
 #pragma unroll
@@ -453,7 +467,7 @@ __global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams 
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) bop[fm] = u32x4{rx[u][fm][0][0], rx[u][fm][0][1], rx[u][fm][1][0], rx[u][fm][1][1]};
       // refill stage u with step t + U
-      load_step(t + U, rw[u], rsc[u], rx[u]);
+      if (!p.debug) load_step(t + U, rw[u], rsc[u], rx[u]);
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) {
         const uint32_t sw = sc[t4 >> 1];
@@ -491,14 +505,20 @@ __global__ __launch_bounds__(kThreads) void fc_w4_mfma_direct_kernel(GemmParams 
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t4][fm][v] += src[((t4 * FM + fm) * 16 + v) * 64 + lane];
   };
-  if (wave >= 2) spill(red[wave - 2]);
-  __syncthreads();
-  if (wave < 2) absorb(red[wave]);
-  __syncthreads();
-  if (wave == 1) spill(red[0]);
-  __syncthreads();
+  // pairwise tree over the waves with two LDS regions: in each round two waves spill and two
+  // absorb, in a fixed order
+#pragma unroll
+  for (int half = WAVES / 2; half >= 1; half /= 2) {
+    // waves [half, 2*half) add into waves [0, half), two at a time
+#pragma unroll
+    for (int base = 0; base < half; base += 2) {
+      if (wave >= half + base && wave < half + base + 2 && wave < 2 * half) spill(red[wave - half - base]);
+      __syncthreads();
+      if (wave >= base && wave < base + 2 && wave < half) absorb(red[wave - base]);
+      __syncthreads();
+    }
+  }
   if (wave != 0) return;
-  absorb(red[0]);
 
   const __half* bias = static_cast<const __half*>(p.bias);
   __half* dst = static_cast<__half*>(p.dst);
@@ -587,15 +607,38 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   p.b_bytes = (uint32_t)((size_t)p.ks * p.m * 8);
   p.s_bytes = (uint32_t)((size_t)p.groups * p.ns * 8);
   p.group_size = a.scale_kind == kScaleBlock ? a.k / a.groups : a.k;
+  p.group_shift = -1;
+  p.debug = std::getenv("MLDHIP_DEBUG") ? std::atoi(std::getenv("MLDHIP_DEBUG")) : 0;
+  if (a.scale_kind != kScaleBlock) {
+    p.group_shift = 30;  // one group
+  } else {
+    const int spg = p.group_size / 16;
+    for (int sh = 0; sh < 30; ++sh)
+      if ((1 << sh) == spg) p.group_shift = sh;
+  }
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
   // token tile: 64 when that still yields a work-group per CU or M is large, else 32
   const long tiles64 = (long)DivUp(a.n, 128) * DivUp(a.m, 64);
-  if (a.m > 32 && (tiles64 >= 128 || a.m > 64)) {
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4>), dim3(DivUp(a.n, 128), DivUp(a.m, 64)), dim3(kThreads), 0,
-                       stream, p);
+  int fm = (a.m > 32 && (tiles64 >= 128 || a.m > 64)) ? 2 : 1;
+  int u = 4;
+  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e);
+  if (const char* e = std::getenv("MLDHIP_GEMM_U")) u = std::atoi(e);
+  const int tiles = DivUp(a.n, 128) * DivUp(a.m, fm * 32);
+  const dim3 grid(DivUp(tiles, 8) * 8);
+  int waves = 8;
+  if (const char* e = std::getenv("MLDHIP_GEMM_WAVES")) waves = std::atoi(e);
+  if (fm == 2) {
+    if (waves == 8)
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 2, 8>), grid, dim3(512), 0, stream, p);
+    else if (u == 8)
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 8, 4>), grid, dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4, 4>), grid, dim3(256), 0, stream, p);
   } else {
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4>), dim3(DivUp(a.n, 128), DivUp(a.m, 32)), dim3(kThreads), 0,
-                       stream, p);
+    if (waves == 8)
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4, 8>), grid, dim3(512), 0, stream, p);
+    else
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4, 4>), grid, dim3(256), 0, stream, p);
   }
   return hipGetLastError();
 }
