@@ -158,8 +158,11 @@ def test_generic_kernel_reference_test_shapes(oracle, bits, dtype, kind):
                               groups=groups, with_bias=True, with_zero_point=kind == "block_zp",
                               act_uniform=True)
         # (N=533 gives an even slice count, so the symmetric fp16 int4 cases take the streaming kernel)
-        streamable = bits == 4 and dtype == np.float16 and kind == "linear" and m <= 4
-        run_case(oracle, case, "fc_w4_stream_kernel" if streamable else "fc_generic_kernel")
+        fast = bits == 4 and dtype == np.float16 and kind == "linear"
+        expect = "fc_generic_kernel"
+        if fast:  # symmetric fp16 int4: streaming GEMV up to 4 tokens, MFMA GEMM beyond
+            expect = "fc_w4_stream_kernel" if m <= 4 else "fc_w4_mfma_gemm_kernel"
+        run_case(oracle, case, expect)
 
 
 def test_known_answers_on_gpu():
