@@ -38,6 +38,9 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
+    p.add_argument("--traffic-probe", action="store_true",
+                   help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a 256 MiB device copy (the known-size "
+                        "reference dispatch) followed by 64 launches over the weight ring, then exit")
     return p.parse_args()
 
 
@@ -117,6 +120,17 @@ def main():
             sys.exit(1)
         kernel = ops[0].kernel_name
 
+        if args.traffic_probe:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(7)
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            for i in range(64):
+                ops[i % args.ring].launch(s)
+            stream.synchronize()
+            print(json.dumps({"traffic_probe": "done", "copy_bytes": 256 << 20, "kernel": kernel}))
+            return
+
         for i in range(max(args.warmup, args.ring)):  # every op allocates its workspace on first use
             ops[i % args.ring].launch(s)
         stream.synchronize()
@@ -153,13 +167,14 @@ def main():
     launch_us = ev_ms * 1e3 / args.steps
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
 
+    # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
+    # scaled by a known-size copy); null when no summary is there
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_fc_w4_stream_c2.json")
+    tpath = os.path.join(ROOT, "profiles", "fc_w4_stream_c2.md")
     if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        except Exception:
-            traffic = None
+        import re
+        mt = re.search(r"^hbm_bytes_per_launch = (\d+)", open(tpath).read(), re.M)
+        traffic = int(mt.group(1)) if mt else None
 
     out = {
         "metric": "int4_decode_gemv_hbm_bandwidth",
