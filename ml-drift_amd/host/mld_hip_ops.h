@@ -1,0 +1,221 @@
+// C++ host-side mirror of the reference's operator interface for the quantized
+// fully-connected path, on top of the C-ABI (include/mldhip.h).
+//
+// Names, argument meaning and error behaviour follow the reference so that a builder /
+// backend written against ML Drift's types maps one to one:
+//   WeightsDescription, OHWI, BHWC            common/task/weights_layout.h, common/shape.h
+//   ExternalWeights                            common/task/gpu_operation.h:354-363
+//   CreateFullyConnectedExternalWeights        common/kernels/fully_connected.h:155-161
+//   CreateQuantization                         common/kernels/quantize_and_dequantize.h:68-73
+//   ClOperation::{SetSrcTensor, SetDstTensor, UpdateParams, AddToQueue}   cl/cl_operation.h:44-129
+//   GpuModelBuilder::FullyConnectedInt4/8ExternalWeights (dispatcher)     common/gpu_model_builder.cc:1548-1725
+// Status is a small stand-in for absl::Status carrying the same code numbers.
+#ifndef MLD_HIP_OPS_H_
+#define MLD_HIP_OPS_H_
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../include/mldhip.h"
+
+namespace mld_hip {
+
+struct Status {
+  int code = MLDHIP_OK;
+  std::string message;
+  bool ok() const { return code == MLDHIP_OK; }
+  static Status FromCode(int c) { return c == MLDHIP_OK ? Status{} : Status{c, mldhip_last_error()}; }
+};
+
+struct OHWI {
+  int o = 0, h = 1, w = 1, i = 0;
+};
+struct BHWC {
+  int b = 1, h = 1, w = 1, c = 0;
+};
+enum class CalculationsPrecision { kF32 = 0, kF32F16 = 1, kF16 = 2 };
+enum class DataType { kFloat16 = 1, kFloat32 = 2, kUint8 = 5, kInt8 = 6, kInt32 = 10, kUint4 = 15 };
+enum class PackedType { kUint8C4 = 1, kInt8C4 = 2, kInt8C16 = 5, kUint8C16 = 6 };
+
+using WeightsDescription = mldhip_weights_desc;
+
+inline WeightsDescription GetFullyConnectedInt8WeightsDesc(const OHWI& shape) {
+  WeightsDescription d;
+  mldhip_fc_int8_weights_desc(shape.o, shape.i, &d);
+  return d;
+}
+inline WeightsDescription GetFullyConnectedInt4WeightsDesc(const OHWI& shape) {
+  WeightsDescription d;
+  mldhip_fc_int4_weights_desc(shape.o, shape.i, &d);
+  return d;
+}
+inline WeightsDescription GetConvolutionInt8WeightsDesc(const OHWI& shape) {
+  WeightsDescription d;
+  mldhip_conv_int8_weights_desc(shape.o, shape.i, &d);
+  return d;
+}
+inline size_t GetTotalElementsCountForLayout(const WeightsDescription& d, const OHWI& s) {
+  size_t n = 0;
+  mldhip_total_elements(&d, s.o, s.h, s.w, s.i, &n);
+  return n;
+}
+
+// Host packers, same names as common/task/weights_conversion.h.
+inline Status RearrangeWeightsInt8AsUint8(const int8_t* w, const OHWI& s, const WeightsDescription& d,
+                                          std::vector<uint8_t>* dst, int shift = 128, unsigned pad = 128u) {
+  dst->resize(GetTotalElementsCountForLayout(d, s));
+  return Status::FromCode(
+      mldhip_rearrange_int8_as_uint8(w, s.o, s.h, s.w, s.i, &d, dst->data(), dst->size(), shift, pad));
+}
+inline Status RearrangeWeightsInt8AsUint4(const int8_t* w, const OHWI& s, const WeightsDescription& d,
+                                          std::vector<uint8_t>* dst, int shift = 8, unsigned pad = 8u) {
+  dst->resize(GetTotalElementsCountForLayout(d, s) / 2);
+  return Status::FromCode(
+      mldhip_rearrange_int8_as_uint4(w, s.o, s.h, s.w, s.i, &d, dst->data(), dst->size(), shift, pad));
+}
+inline Status RearrangeWeightsUInt4Packed(const uint8_t* w, const OHWI& s, const WeightsDescription& d,
+                                          std::vector<uint8_t>* dst, std::vector<int32_t>* weights_sum_i,
+                                          unsigned pad = 8u, bool swap_dims = false) {
+  dst->resize(GetTotalElementsCountForLayout(d, s) / 2);
+  if (weights_sum_i->size() < (size_t)s.o) weights_sum_i->resize(s.o);
+  return Status::FromCode(mldhip_rearrange_uint4_packed(w, s.o, s.h, s.w, s.i, &d, dst->data(), dst->size(),
+                                                        weights_sum_i->data(), weights_sum_i->size(), pad, swap_dims));
+}
+
+// Shape/type of the quantized weights of one layer; device buffers are the caller's
+// (ExternalWeights holds non-owning descriptors in the reference as well).
+struct ExternalWeights {
+  WeightsDescription desc{};
+  OHWI shape;
+  OHWI scale_zp_shape{1, 1, 1, 1};  // (o,1,1,groups); (1,1,1,1) = scalar
+  bool has_scale_tensor = false;
+  bool has_zero_point_tensor = false;
+  float scalar_scale = 1.0f;
+  bool has_scalar_zero_point = false;
+  float scalar_zero_point = 0.0f;
+};
+
+// A node executor: what ClOperation is to a GPUOperation in the reference.
+class HipOperation {
+ public:
+  HipOperation() = default;
+  explicit HipOperation(mldhip_op* op) : op_(op, &mldhip_op_destroy) {}
+  HipOperation(HipOperation&&) = default;  // move-only, like GPUOperation
+  HipOperation& operator=(HipOperation&&) = default;
+
+  std::vector<std::string> GetSrcTensorsNames() const {
+    std::vector<std::string> r;
+    for (int i = 0; i < mldhip_op_src_count(op_.get()); ++i) r.emplace_back(mldhip_op_src_name(op_.get(), i));
+    return r;
+  }
+  std::vector<std::string> GetDstTensorsNames() const {
+    std::vector<std::string> r;
+    for (int i = 0; i < mldhip_op_dst_count(op_.get()); ++i) r.emplace_back(mldhip_op_dst_name(op_.get(), i));
+    return r;
+  }
+  Status SetSrcTensor(int index, const void* device_ptr, size_t bytes) {
+    return Status::FromCode(mldhip_op_set_src(op_.get(), index, device_ptr, bytes));
+  }
+  Status SetDstTensor(int index, void* device_ptr, size_t bytes) {
+    return Status::FromCode(mldhip_op_set_dst(op_.get(), index, device_ptr, bytes));
+  }
+  // UpdateParams: re-evaluates everything that depends on the runtime tensor shape.
+  Status UpdateParams(const BHWC& src_shape) {
+    return Status::FromCode(mldhip_op_set_shape(op_.get(), src_shape.b, src_shape.h, src_shape.w));
+  }
+  Status AddToQueue(void* hip_stream) { return Status::FromCode(mldhip_op_launch(op_.get(), hip_stream)); }
+  const char* kernel_name() const { return mldhip_op_kernel_name(op_.get()); }
+  bool valid() const { return op_ != nullptr; }
+
+ private:
+  std::unique_ptr<mldhip_op, void (*)(mldhip_op*)> op_{nullptr, &mldhip_op_destroy};
+};
+
+inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precision, DataType src_type,
+                                                  DataType dst_type, const ExternalWeights& weights, bool has_bias,
+                                                  int max_tokens, HipOperation* result) {
+  mldhip_fc_desc d{};
+  d.precision = (int)precision;
+  d.src_type = (int)src_type;
+  d.dst_type = (int)dst_type;
+  d.o = weights.shape.o;
+  d.i = weights.shape.i;
+  d.weights = weights.desc;
+  d.scale_o = weights.has_scale_tensor ? weights.scale_zp_shape.o : 1;
+  d.scale_i = weights.has_scale_tensor ? weights.scale_zp_shape.i : 1;
+  d.scalar_scale = weights.scalar_scale;
+  d.has_zero_point_tensor = weights.has_zero_point_tensor;
+  d.has_scalar_zero_point = weights.has_scalar_zero_point;
+  d.scalar_zero_point = weights.scalar_zero_point;
+  d.has_bias = has_bias;
+  d.max_tokens = max_tokens;
+  mldhip_op* op = nullptr;
+  const int rc = mldhip_fc_create(&d, &op);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  *result = HipOperation(op);
+  return {};
+}
+
+inline Status CreateQuantization(DataType src_type, PackedType dst_type, const BHWC& shape, bool calculate_sum,
+                                 bool symmetric, HipOperation* result) {
+  mldhip_quant_desc d{(int)src_type, (int)dst_type, shape.c, calculate_sum, symmetric, shape.b * shape.h * shape.w};
+  mldhip_op* op = nullptr;
+  const int rc = mldhip_quantization_create(&d, &op);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  *result = HipOperation(op);
+  return {};
+}
+
+inline Status CreateConvInt8WithDequantization(DataType dst_type, const OHWI& weights_shape,
+                                               const WeightsDescription& weights_desc, bool has_zero_point,
+                                               bool has_bias, int max_tokens, HipOperation* result) {
+  mldhip_conv_int8_desc d{};
+  d.src_packed_type = mldhip_conv_int8_src_type();
+  d.dst_type = (int)dst_type;
+  d.o = weights_shape.o;
+  d.i = weights_shape.i;
+  d.weights = weights_desc;
+  d.has_zero_point = has_zero_point;
+  d.has_bias = has_bias;
+  d.max_tokens = max_tokens;
+  mldhip_op* op = nullptr;
+  const int rc = mldhip_conv_int8_create(&d, &op);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  *result = HipOperation(op);
+  return {};
+}
+
+// One graph node: operation + the ids of its inputs/outputs in the caller's tensor table,
+// in the reference's order (common/gpu_model.h:38-60).
+struct GpuNode {
+  HipOperation gpu_operation;
+  std::vector<int> inputs;
+  std::vector<int> outputs;
+  std::string name;
+};
+
+// The route the builder takes for a quantized FullyConnected
+// (GpuModelBuilder::FullyConnectedInt4/8ExternalWeights, common/gpu_model_builder.cc:1548-1725),
+// restated for this device:
+//   kFullyConnected   one FC node over the packed FC weights (any token count: streaming GEMV
+//                     for a few tokens, fused dequantize+MFMA GEMM beyond; the reference would
+//                     emit WeightsConverter + float ConvGeneric there)
+//   kQuantizedInt8    Quantize -> int8 conv (+ Dequantization), available for per-channel int8
+//                     weights with weights_sum_i when 8-bit convolutions are not disallowed
+enum class FcRoute { kFullyConnected, kQuantizedInt8 };
+
+inline FcRoute SelectFullyConnectedRoute(const ExternalWeights& w, int tokens, bool has_weights_sum_i,
+                                         bool disallow_8bit_convs) {
+  const bool grouped = w.scale_zp_shape.i != 1;
+  const bool int8_weights = w.desc.type == MLDHIP_UINT8 || w.desc.type == MLDHIP_INT8;
+  if (mldhip_fc_is_recommended((int)CalculationsPrecision::kF32F16, tokens)) return FcRoute::kFullyConnected;
+  if (!grouped && int8_weights && has_weights_sum_i && !disallow_8bit_convs) return FcRoute::kQuantizedInt8;
+  return FcRoute::kFullyConnected;
+}
+
+}  // namespace mld_hip
+
+#endif  // MLD_HIP_OPS_H_

@@ -1,0 +1,77 @@
+// Host-only check of the C++ adapter: builds ops through the reference-shaped factories,
+// checks object order, validation codes and the packer against a literal golden vector.
+#include <cstdio>
+#include <cstring>
+
+#include "../ml-drift_amd/host/mld_hip_ops.h"
+
+using namespace mld_hip;
+
+#define EXPECT(cond)                                              \
+  do {                                                            \
+    if (!(cond)) {                                                \
+      std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); \
+      return 1;                                                   \
+    }                                                             \
+  } while (0)
+
+int main() {
+  // common/task/weights_conversion_test.cc:50-91
+  OHWI shape{4, 1, 1, 4};
+  std::vector<uint8_t> src;
+  for (int i = 0; i < 8; ++i) src.push_back((uint8_t)(((2 * i + 1) << 4) | (2 * i)));
+  WeightsDescription d{};
+  d.type = MLDHIP_UINT8;
+  d.layout = MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4;
+  d.output_group_size = 1;
+  std::vector<uint8_t> packed;
+  std::vector<int32_t> sums;
+  EXPECT(RearrangeWeightsUInt4Packed(src.data(), shape, d, &packed, &sums).ok());
+  const int order[16] = {0, 4, 8, 12, 1, 5, 9, 13, 2, 6, 10, 14, 3, 7, 11, 15};
+  for (int i = 0; i < 8; ++i) EXPECT(packed[i] == (uint8_t)((order[2 * i] | (order[2 * i + 1] << 4)) ^ 0x88));
+  EXPECT(sums[0] == 6 && sums[1] == 22 && sums[2] == -26 && sums[3] == -10);
+  d.layout = MLDHIP_LAYOUT_OSPATIAL_IOGROUP_O4I4;
+  Status st = RearrangeWeightsUInt4Packed(src.data(), shape, d, &packed, &sums);
+  EXPECT(st.code == MLDHIP_UNIMPLEMENTED && st.message == "Unsupported layout");
+
+  ExternalWeights w;
+  w.shape = OHWI{14336, 1, 1, 4096};
+  w.desc = GetFullyConnectedInt4WeightsDesc(w.shape);
+  w.scale_zp_shape = OHWI{14336, 1, 1, 1};
+  w.has_scale_tensor = true;
+  HipOperation fc;
+  EXPECT(CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
+                                             /*has_bias=*/true, 4, &fc)
+             .ok());
+  auto names = fc.GetSrcTensorsNames();
+  EXPECT(names.size() == 4 && names[0] == "src_tensor" && names[1] == "weights" && names[2] == "weights_scale" &&
+         names[3] == "biases");
+  EXPECT(fc.UpdateParams(BHWC{1, 1, 5, 4096}).code == MLDHIP_OUT_OF_RANGE);
+  EXPECT(fc.AddToQueue(nullptr).code == MLDHIP_FAILED_PRECONDITION);  // nothing bound: refused before any GPU call
+
+  w.desc.output_group_size = 7;
+  HipOperation bad;
+  st = CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
+                                           false, 1, &bad);
+  EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !bad.valid());
+
+  HipOperation q;
+  EXPECT(CreateQuantization(DataType::kFloat16, PackedType::kInt8C16, BHWC{1, 1, 2048, 2048}, false, true, &q).ok());
+  EXPECT(q.GetDstTensorsNames().size() == 2 && q.GetDstTensorsNames()[1] == "dst_params");
+
+  ExternalWeights w8;
+  w8.shape = OHWI{8192, 1, 1, 2048};
+  w8.desc = GetFullyConnectedInt8WeightsDesc(w8.shape);
+  w8.scale_zp_shape = OHWI{8192, 1, 1, 1};
+  EXPECT(SelectFullyConnectedRoute(w8, 1, true, false) == FcRoute::kFullyConnected);
+  EXPECT(SelectFullyConnectedRoute(w8, 2048, true, false) == FcRoute::kQuantizedInt8);
+  EXPECT(SelectFullyConnectedRoute(w8, 2048, true, true) == FcRoute::kFullyConnected);
+  EXPECT(SelectFullyConnectedRoute(w, 512, false, false) == FcRoute::kFullyConnected);
+  HipOperation conv;
+  EXPECT(CreateConvInt8WithDequantization(DataType::kFloat16, w8.shape, GetConvolutionInt8WeightsDesc(w8.shape), false,
+                                          false, 2048, &conv)
+             .ok());
+  EXPECT(conv.GetSrcTensorsNames().size() == 5 && conv.GetSrcTensorsNames()[2] == "params_tensor");
+  std::printf("host adapter ok\n");
+  return 0;
+}
