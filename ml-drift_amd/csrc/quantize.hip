@@ -4,10 +4,6 @@
 // multiply-add), round half up through floor(x*scale + zp + 0.5) or truncation of
 // (x-min)*scale + 0.5.
 //
-// Work-group = 32 tokens x 8 reduction lanes.  Tokens are the contiguous axis of the
-// slice-major tensor, so the 32 token lanes of a wave read 32 x 8 B (fp16) contiguous bytes
-// per slice.  Each thread owns groups of 4 consecutive slices (16 channels), which is one
-// 16-byte store of codes in the C16 layout.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -27,8 +23,8 @@ __device__ __forceinline__ float Add(float a, float b) { return a + b; }
 __device__ __forceinline__ float Sub(float a, float b) { return a - b; }
 __device__ __forceinline__ float Div(float a, float b) { return a / b; }
 
-constexpr int kTok = 32;
-constexpr int kRed = 8;
+// Groups of 16 channels per thread that stay in registers between the two passes.
+constexpr int kMaxWaves = 16;
 
 struct QuantParams {
   const void* src;
@@ -38,8 +34,18 @@ struct QuantParams {
   int is_signed, c16, symmetric, calculate_sum;
 };
 
-__device__ __forceinline__ void Load4(const __half* src, size_t idx, float v[4]) {
-  const uint2 raw = *reinterpret_cast<const uint2*>(src + idx);
+template <typename SrcT>
+struct Raw;
+template <>
+struct Raw<__half> {
+  using type = uint2;
+};
+template <>
+struct Raw<float> {
+  using type = float4;
+};
+
+__device__ __forceinline__ void Unpack(const uint2& raw, float v[4]) {
   const __half2 lo = *reinterpret_cast<const __half2*>(&raw.x);
   const __half2 hi = *reinterpret_cast<const __half2*>(&raw.y);
   v[0] = __low2float(lo);
@@ -47,8 +53,7 @@ __device__ __forceinline__ void Load4(const __half* src, size_t idx, float v[4])
   v[2] = __low2float(hi);
   v[3] = __high2float(hi);
 }
-__device__ __forceinline__ void Load4(const float* src, size_t idx, float v[4]) {
-  const float4 raw = *reinterpret_cast<const float4*>(src + idx);
+__device__ __forceinline__ void Unpack(const float4& raw, float v[4]) {
   v[0] = raw.x;
   v[1] = raw.y;
   v[2] = raw.z;
@@ -63,133 +68,228 @@ __device__ __forceinline__ float RangeInSrcType(const float*, float mx, float mn
   return Sub(mx, mn);
 }
 
-template <typename SrcT>
-__global__ __launch_bounds__(kTok* kRed) void quantize_kernel(QuantParams p) {
-  __shared__ float s_a[kRed][kTok];
-  __shared__ float s_b[kRed][kTok];
-  __shared__ int s_sum[kRed][kTok];
+template <bool SYM>
+struct Quantizer {
+  float scale, min_value;
+  // The unsigned code of x as an integral float; the caller saturates it to [0, 255] while
+  // packing.  Asymmetric: truncation of a value >= 0.5, i.e. floor; a NaN (constant row:
+  // 0 * inf) becomes code 0.
+  __device__ __forceinline__ float Value(float x) const {
+    if (SYM) return floorf(Add(Mul(x, scale), 128.5f));
+    const float f = floorf(Add(Mul(Sub(x, min_value), scale), 0.5f));
+    return f != f ? 0.0f : f;
+  }
+};
+
+// Work-group = TT tokens x (blockDim.x / TT) reduction lanes.  Tokens are the contiguous axis
+// of the slice-major tensor, so the TT token lanes read TT x 8 B (fp16) contiguous bytes per
+// slice.  Each thread owns groups of 4 consecutive slices (16 channels, one 16-byte store of
+// codes in the C16 layout); the first CACHE groups of a thread stay in registers between the
+// min/max pass and the encoding pass, so a row of up to 16 * CACHE * lanes channels is read
+// from memory once.
+template <typename SrcT, int TT, bool SYM, int CACHE>
+__global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
+  using RawT = typename Raw<SrcT>::type;
+  __shared__ float s_a[kMaxWaves][TT];
+  __shared__ float s_b[kMaxWaves][TT];
+  __shared__ int s_sum[kMaxWaves][TT];
   const SrcT* src = static_cast<const SrcT*>(p.src);
-  const int lt = threadIdx.x % kTok;
-  const int lr = threadIdx.x / kTok;
-  const int tok_raw = blockIdx.x * kTok + lt;
+  const RawT* src4 = static_cast<const RawT*>(p.src);
+  const int red = blockDim.x / TT;
+  const int lt = threadIdx.x % TT;
+  const int lr = threadIdx.x / TT;
+  const int wave = threadIdx.x / 64;
+  const int waves = blockDim.x / 64;
+  const int tok_raw = blockIdx.x * TT + lt;
   const bool tok_ok = tok_raw < p.tokens;
   const int tok = tok_ok ? tok_raw : p.tokens - 1;
   const int s16_count = (p.slices + 3) / 4;
   constexpr bool kHalf = sizeof(SrcT) == 2;
 
+  // Loads of the cached groups; slices past the end re-read the last one and are masked below.
+  RawT cache[CACHE][4];
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) {
+    const int g = lr + i * red;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = min(g * 4 + j, p.slices - 1);
+      cache[i][j] = src4[(size_t)s * p.tokens + tok];
+    }
+  }
+
   // pass 1: abs-max, or min/max seeded with element (batch b, y 0, x 0, channel 0)
   float r0, r1;
-  if (p.symmetric) {
+  if (SYM) {
     r0 = 0.0f;
     r1 = 0.0f;
   } else {
     const int b = p.batch > 0 ? tok % p.batch : 0;
     float seed[4];
-    Load4(src, (size_t)b * 4, seed);
+    Unpack(src4[b], seed);
     r0 = seed[0];
     r1 = seed[0];
   }
-  for (int g = lr; g < s16_count; g += kRed) {
+  // Channels past the end are replaced by the running value, which leaves it unchanged.
+  auto reduce4 = [&](const RawT& raw, int s) {
+    float v[4];
+    Unpack(raw, v);
+    const int nvalid = p.channels - s * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      if (SYM) {
+        r0 = fmaxf(r0, c < nvalid ? fabsf(v[c]) : 0.0f);
+      } else {
+        r0 = fminf(r0, c < nvalid ? v[c] : r0);
+        r1 = fmaxf(r1, c < nvalid ? v[c] : r1);
+      }
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) {
+    const int g = lr + i * red;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) reduce4(cache[i][j], g * 4 + j);
+  }
+  for (int g = lr + CACHE * red; g < s16_count; g += red) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = g * 4 + j;
-      if (s >= p.slices) break;
-      float v[4];
-      Load4(src, ((size_t)s * p.tokens + tok) * 4, v);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        if (s * 4 + c < p.channels) {
-          if (p.symmetric) {
-            r0 = fmaxf(r0, fabsf(v[c]));
-          } else {
-            r0 = fminf(r0, v[c]);
-            r1 = fmaxf(r1, v[c]);
-          }
-        }
-      }
+      if (s < p.slices) reduce4(src4[(size_t)s * p.tokens + tok], s);
     }
   }
-  s_a[lr][lt] = r0;
-  s_b[lr][lt] = r1;
-  __syncthreads();
+  // lanes of a wave that share a token, then the waves of the work-group
 #pragma unroll
-  for (int r = 0; r < kRed; ++r) {
-    if (p.symmetric) {
-      r0 = fmaxf(r0, s_a[r][lt]);
+  for (int off = TT; off < 64; off *= 2) {
+    if (SYM) {
+      r0 = fmaxf(r0, __shfl_xor(r0, off));
     } else {
-      r0 = fminf(r0, s_a[r][lt]);
-      r1 = fmaxf(r1, s_b[r][lt]);
+      r0 = fminf(r0, __shfl_xor(r0, off));
+      r1 = fmaxf(r1, __shfl_xor(r1, off));
+    }
+  }
+  if (threadIdx.x % 64 < TT) {
+    s_a[wave][lt] = r0;
+    if (!SYM) s_b[wave][lt] = r1;
+  }
+  __syncthreads();
+  for (int w = 0; w < waves; ++w) {
+    if (SYM) {
+      r0 = fmaxf(r0, s_a[w][lt]);
+    } else {
+      r0 = fminf(r0, s_a[w][lt]);
+      r1 = fmaxf(r1, s_b[w][lt]);
     }
   }
 
-  float inv_scale = 0.0f, scale = 0.0f, offset = 0.0f, min_value = 0.0f;
-  if (p.symmetric) {
+  float inv_scale = 0.0f, offset = 0.0f;
+  Quantizer<SYM> qz;
+  qz.scale = 0.0f;
+  qz.min_value = 0.0f;
+  const uint32_t sign_flip = p.is_signed ? 0x80808080u : 0u;  // u8 code - 128 as int8
+  const int code_shift = p.is_signed ? 128 : 0;
+  if (SYM) {
     const float abs_max = r0;
     if (abs_max > 0.0f) {
       const float min_scale = kHalf ? 6.103515625e-05f : 1.0e-30f;
       inv_scale = fmaxf(min_scale, Div(abs_max, 127.0f));
       if (!p.is_signed && kHalf) inv_scale = fminf(inv_scale, Div(65504.0f, 128.0f));
-      scale = Div(1.0f, inv_scale);
+      qz.scale = Div(1.0f, inv_scale);
       if (!p.is_signed) offset = Mul(-inv_scale, 128.0f);
     }
   } else {
-    min_value = r0;
+    qz.min_value = r0;
     const float src_range = RangeInSrcType(src, r1, r0);
-    offset = min_value;
-    scale = Div(255.0f, src_range);
+    offset = qz.min_value;
+    qz.scale = Div(255.0f, src_range);
     inv_scale = Div(src_range, 255.0f);
     if (p.is_signed) offset = Add(offset, Mul(src_range, Div(128.0f, 255.0f)));
   }
 
   // pass 2: codes
-  int sum = 0;
-  const int code_shift = p.is_signed ? 128 : 0;
-  for (int g = lr; g < s16_count; g += kRed) {
-    uint32_t packed[4] = {0u, 0u, 0u, 0u};
+  uint32_t sum = 0;
+  auto encode4 = [&](const RawT& raw, int s) -> uint32_t {
+    float v[4];
+    Unpack(raw, v);
+    const int nvalid = max(0, min(4, p.channels - s * 4));
+    uint32_t word = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) word = __builtin_amdgcn_cvt_pk_u8_f32(qz.Value(v[c]), c, word);
+    const uint32_t valid = nvalid >= 4 ? 0xFFFFFFFFu : (1u << (8 * nvalid)) - 1u;
+    sum = __builtin_amdgcn_udot4(word & valid, 0x01010101u, sum, false) - code_shift * nvalid;
+    return word ^ sign_flip;
+  };
+  auto store_group = [&](int g, const uint32_t packed[4]) {
+    if (!tok_ok) return;
+    if (p.c16) {
+      *reinterpret_cast<uint4*>(p.codes + ((size_t)g * p.tokens + tok) * 16) =
+          make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int s = g * 4 + j;
+        if (s < p.slices)
+          *reinterpret_cast<uint32_t*>(p.codes + ((size_t)s * p.tokens + tok) * 4) = packed[j];
+      }
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) {
+    const int g = lr + i * red;
+    if (g < s16_count) {
+      uint32_t packed[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int s = g * 4 + j;
+        const uint32_t word = encode4(cache[i][j], s);
+        packed[j] = s < p.slices ? word : 0u;
+      }
+      store_group(g, packed);
+    }
+  }
+  for (int g = lr + CACHE * red; g < s16_count; g += red) {
+    uint32_t packed[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = g * 4 + j;
-      if (s >= p.slices) break;
-      float v[4];
-      Load4(src, ((size_t)s * p.tokens + tok) * 4, v);
-      uint32_t word = 0;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        int q;
-        if (p.symmetric) {
-          float f = Mul(v[c], scale);
-          f = Add(f, 128.5f);
-          f = floorf(f);
-          f = fminf(255.0f, fmaxf(0.0f, f));
-          q = (int)f;
-        } else {
-          float f = Mul(Sub(v[c], min_value), scale);
-          f = Add(f, 0.5f);
-          q = (f != f) ? 0 : (int)f;  // NaN (constant row: 0 * inf) converts to 0
-          q = max(0, min(255, q));
-        }
-        q -= code_shift;
-        if (s * 4 + c < p.channels) sum += q;
-        word |= (uint32_t)(q & 0xFF) << (8 * c);
-      }
-      packed[j] = word;
-      if (!p.c16 && tok_ok)
-        *reinterpret_cast<uint32_t*>(p.codes + ((size_t)s * p.tokens + tok) * 4) = word;
+      packed[j] = s < p.slices ? encode4(src4[(size_t)s * p.tokens + tok], s) : 0u;
     }
-    if (p.c16 && tok_ok)
-      *reinterpret_cast<uint4*>(p.codes + ((size_t)g * p.tokens + tok) * 16) =
-          make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    store_group(g, packed);
   }
   if (p.calculate_sum) {
-    s_sum[lr][lt] = sum;
-    __syncthreads();
-    sum = 0;
+    int total = (int)sum;
 #pragma unroll
-    for (int r = 0; r < kRed; ++r) sum += s_sum[r][lt];
+    for (int off = TT; off < 64; off *= 2) total += __shfl_xor(total, off);
+    if (threadIdx.x % 64 < TT) s_sum[wave][lt] = total;
+    __syncthreads();
+    total = 0;
+    for (int w = 0; w < waves; ++w) total += s_sum[w][lt];
+    sum = (uint32_t)total;
   }
   if (lr == 0 && tok_ok)
     *reinterpret_cast<float4*>(p.params + (size_t)tok * 4) =
-        make_float4(inv_scale, offset, p.calculate_sum ? (float)sum : 0.0f, 0.0f);
+        make_float4(inv_scale, offset, p.calculate_sum ? (float)(int)sum : 0.0f, 0.0f);
+}
+
+template <int TT, int CACHE>
+void Launch2(bool f16, bool sym, dim3 grid, dim3 block, hipStream_t stream, const QuantParams& p) {
+  if (f16 && sym)
+    hipLaunchKernelGGL((quantize_kernel<__half, TT, true, CACHE>), grid, block, 0, stream, p);
+  else if (f16)
+    hipLaunchKernelGGL((quantize_kernel<__half, TT, false, CACHE>), grid, block, 0, stream, p);
+  else if (sym)
+    hipLaunchKernelGGL((quantize_kernel<float, TT, true, CACHE>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((quantize_kernel<float, TT, false, CACHE>), grid, block, 0, stream, p);
+}
+// One register-cached group per thread when that covers the row, four otherwise.
+template <int TT>
+void Launch(bool f16, bool sym, dim3 grid, dim3 block, hipStream_t stream, const QuantParams& p) {
+  const int red = (int)block.x / TT;
+  if (DivUp(p.slices, 4) <= red)
+    Launch2<TT, 1>(f16, sym, grid, block, stream, p);
+  else
+    Launch2<TT, 4>(f16, sym, grid, block, stream, p);
 }
 
 }  // namespace
@@ -208,12 +308,19 @@ hipError_t LaunchQuantize(const QuantArgs& a, hipStream_t stream, const char** k
   p.symmetric = a.symmetric;
   p.calculate_sum = a.calculate_sum;
   if (kernel_name) *kernel_name = "quantize_kernel";
-  dim3 grid(DivUp(a.tokens, kTok));
-  dim3 block(kTok * kRed);
-  if (a.src_f16)
-    hipLaunchKernelGGL(quantize_kernel<__half>, grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL(quantize_kernel<float>, grid, block, 0, stream, p);
+  // Few channel groups: wide token tiles (32 tokens x >= 2 lanes); otherwise 8 tokens per
+  // work-group and as many reduction lanes as there are groups, up to 128.
+  const int groups16 = DivUp(p.slices, 4);
+  int red = 1;
+  while (red < groups16 && red < 128) red *= 2;
+  if (red <= 8) {
+    red = red < 2 ? 2 : red;
+    dim3 grid(DivUp(a.tokens, 32)), block(32 * red);
+    Launch<32>(a.src_f16, a.symmetric, grid, block, stream, p);
+  } else {
+    dim3 grid(DivUp(a.tokens, 8)), block(8 * red);
+    Launch<8>(a.src_f16, a.symmetric, grid, block, stream, p);
+  }
   return hipGetLastError();
 }
 
