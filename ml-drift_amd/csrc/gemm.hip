@@ -65,8 +65,7 @@ struct GemmParams {
   // byte sizes of the A (weights), B (activations / codes) and scale buffers
   uint32_t a_bytes, b_bytes, s_bytes;
   int group_size;   // input channels per scale group (fp16 path)
-  int group_shift;  // log2(group_size / 16) when that is a power of two, else -1
-  int debug;
+  int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -374,12 +373,16 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
 // the 4 MFMAs t = 0..3 together hold one whole 4-channel output slice per (v, token): one
 // 8-byte store.  Loads are raw buffer loads (out-of-range reads as zero), U steps ahead.
 // ------------------------------------------------------------------------------------------
+// Work-group barrier that waits for this wave's LDS traffic only: global stores issued before
+// it stay in flight.
+__device__ __forceinline__ void LdsBarrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int FM, int U, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
-  constexpr int kTileFloats = 4 * FM * 16 * 64;  // one wave's accumulators
-  __shared__ float red[2][kTileFloats];
+  static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "the reduction handles WAVES registers per phase");
+  __shared__ float4 red[WAVES][WAVES][64];  // [copy][register within the phase][lane]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -399,47 +402,58 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int nsi = n0 / 4 + i32;
   const bool n_ok = nsi < p.ns;
 
+  // This wave's range of 16-channel steps.  The buffer descriptors of the weights and the
+  // activations end where the wave's share of K ends, so the prefetches that run past it (and
+  // past K itself) read zeros without a test in the loop; a lane without an output slice or
+  // a token gets an offset beyond every buffer.
+  const int steps_total = (p.k + 15) / 16;
+  const int per_wave = ((steps_total + WAVES - 1) / WAVES + U - 1) / U * U;  // multiple of U
+  const int t_begin = __builtin_amdgcn_readfirstlane(wave * per_wave);
+  const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
+  const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
+  const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
+  const uint32_t w_end = min((uint64_t)p.a_bytes, (uint64_t)k_slices_end * row_w);
+  const uint32_t x_end = min((uint64_t)p.b_bytes, (uint64_t)k_slices_end * row_x);
+
   constexpr uint32_t kOob = 0x7FFFFFF0u;
   const __amdgpu_buffer_rsrc_t rsrc_w =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w4), 0, p.a_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w4), 0, w_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_x =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, p.b_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, x_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_s =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
 
-  // this wave's range of 16-channel steps
-  const int steps_total = (p.k + 15) / 16;
-  const int per_wave = ((steps_total + WAVES - 1) / WAVES + U - 1) / U * U;  // multiple of U
-  const int t_begin = wave * per_wave;
-
-  uint32_t tok_off[FM];  // byte offset of this lane's token inside one K-slice row, or out of range
+  // Per-lane byte offsets of the next step to fetch; each fetch advances them by one step.
+  // Only the per-lane offset takes part in the range check of a buffer load, so the whole
+  // address lives there.
+  const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
+  uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * 8u : kOob;
+  uint32_t vw1 = n_ok ? vw0 + row_w : kOob;
+  const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
+  uint32_t vx[FM][2];
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
     const int mi = m0 + fm * 32 + i32;
-    tok_off[fm] = mi < p.m ? (uint32_t)mi * 8u : kOob;
+    vx[fm][0] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
+    vx[fm][1] = mi < p.m ? vx[fm][0] + row_x : kOob;
   }
-  const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
-  const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
+  const uint32_t group_bytes = row_w;  // one scale group: [Ns][4] halfs
 
   u32x2 rw[U][2], rsc[U], rx[U][FM][2];
   auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2 (&x)[FM][2]) {
-    // steps beyond this wave's share read nothing: the limit is the next wave's first step
-    const bool live = t < t_begin + per_wave;
-    const uint32_t ksa = (uint32_t)(t * 2 + g2) * 2u;
-    const bool w_ok = live && n_ok;
-    const uint32_t wo = w_ok ? ksa * row_w + (uint32_t)nsi * 8u : kOob;
-    w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, wo, 0, 0);
-    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, w_ok ? wo + row_w : kOob, 0, 0);
-    // scale group of this step: a shift when the group holds a power-of-two number of steps
-    int grp = p.group_shift >= 0 ? (t >> p.group_shift) : (t * 16) / p.group_size;
-    grp = grp < p.groups ? grp : p.groups - 1;
-    sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, n_ok ? (uint32_t)(grp * p.ns + nsi) * 8u : kOob, 0, 0);
+    w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
+    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw1, 0, 0);
+    vw0 += step_w;
+    vw1 += step_w;
+    // scale group of this step (groups hold a power-of-two number of steps); a group past the
+    // last one reads zeros
+    sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
-      const bool x_ok = live && tok_off[fm] != kOob;
-      const uint32_t xo = x_ok ? ksa * row_x + tok_off[fm] : kOob;
-      x[fm][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, xo, 0, 0);
-      x[fm][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, x_ok ? xo + row_x : kOob, 0, 0);
+      x[fm][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[fm][0], 0, 0);
+      x[fm][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[fm][1], 0, 0);
+      vx[fm][0] += step_x;
+      vx[fm][1] += step_x;
     }
   };
 
@@ -454,92 +468,87 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
 
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int u = 0; u < U; ++u) load_step(t_begin + u, rw[u], rsc[u], rx[u]);
+  for (int u = 0; u < U; ++u) {
+    load_step(t_begin + u, rw[u], rsc[u], rx[u]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   for (int tt = 0; tt < per_wave; tt += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int t = t_begin + tt + u;
       // consume stage u
       const u32x4 blk = {rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
-      const u32x2 sc = rsc[u];
-      u32x4 bop[FM];
-#pragma unroll
-      for (int fm = 0; fm < FM; ++fm) bop[fm] = u32x4{rx[u][fm][0][0], rx[u][fm][0][1], rx[u][fm][1][0], rx[u][fm][1][1]};
-      // refill stage u with step t + U
-      if (!p.debug) load_step(t + U, rw[u], rsc[u], rx[u]);
+      const u32x4 blk8 = {blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
+      const half2_t sc01 = AsHalf2(rsc[u][0]), sc23 = AsHalf2(rsc[u][1]);
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) {
-        const uint32_t sw = sc[t4 >> 1];
-        const uint32_t s16 = (t4 & 1) ? (sw >> 16) : (sw & 0xFFFFu);
-        const half2_t s2 = AsHalf2(s16 | (s16 << 16));
+        const half2_t sp = (t4 & 2) ? sc23 : sc01;
+        const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
         u32x4 aop;
 #pragma unroll
         for (int wd = 0; wd < 4; ++wd) {
-          const uint32_t x = (t4 & 2) ? (blk[wd] >> 8) : blk[wd];
+          const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
           const uint32_t bits = (t4 & 1) ? AndOr(x, p.mask_hi, p.magic_hi) : AndOr(x, p.mask_lo, p.magic_lo);
           aop[wd] = AsU32((AsHalf2(bits) + ((t4 & 1) ? off_hi : off_lo)) * s2);
         }
 #pragma unroll
-        for (int fm = 0; fm < FM; ++fm)
+        for (int fm = 0; fm < FM; ++fm) {
+          const u32x4 bop = {rx[u][fm][0][0], rx[u][fm][0][1], rx[u][fm][1][0], rx[u][fm][1][1]};
           acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
-                                                               __builtin_bit_cast(half8_t, bop[fm]), acc[t4][fm], 0, 0, 0);
+                                                               __builtin_bit_cast(half8_t, bop), acc[t4][fm], 0, 0, 0);
+        }
       }
+      // refill stage u with step t + U; the fences keep the loads of a stage together and in
+      // program order, so that waiting for one stage leaves the younger ones in flight
+      __builtin_amdgcn_sched_barrier(0);
+      load_step(t + U, rw[u], rsc[u], rx[u]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
-  // K-split reduction: waves 2,3 -> LDS, waves 0,1 add; wave 1 -> LDS, wave 0 adds.
-  auto spill = [&](float* dst) {
-#pragma unroll
-    for (int t4 = 0; t4 < 4; ++t4)
-#pragma unroll
-      for (int fm = 0; fm < FM; ++fm)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) dst[((t4 * FM + fm) * 16 + v) * 64 + lane] = acc[t4][fm][v];
-  };
-  auto absorb = [&](const float* src) {
-#pragma unroll
-    for (int t4 = 0; t4 < 4; ++t4)
-#pragma unroll
-      for (int fm = 0; fm < FM; ++fm)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t4][fm][v] += src[((t4 * FM + fm) * 16 + v) * 64 + lane];
-  };
-  // pairwise tree over the waves with two LDS regions: in each round two waves spill and two
-  // absorb, in a fixed order
-#pragma unroll
-  for (int half = WAVES / 2; half >= 1; half /= 2) {
-    // waves [half, 2*half) add into waves [0, half), two at a time
-#pragma unroll
-    for (int base = 0; base < half; base += 2) {
-      if (wave >= half + base && wave < half + base + 2 && wave < 2 * half) spill(red[wave - half - base]);
-      __syncthreads();
-      if (wave >= base && wave < base + 2 && wave < half) absorb(red[wave - base]);
-      __syncthreads();
-    }
-  }
-  if (wave != 0) return;
-
+  // K-split reduction, spread over all waves.  The tile goes through LDS in phases of WAVES
+  // accumulator registers per lane (x 4 MFMAs): every wave writes its copy, then wave w adds the
+  // WAVES copies of register w in a fixed order and stores that part of the output.  In the
+  // 32x32 result, register v of lane (g2, i32) belongs to output slice 8*(v/4) + 4*g2 + v%4 and
+  // token i32, and the four MFMAs hold the slice's four channels: one 8-byte store.
   const __half* bias = static_cast<const __half*>(p.bias);
   __half* dst = static_cast<__half*>(p.dst);
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
     const int mi = m0 + fm * 32 + i32;
-    if (mi >= p.m) continue;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-      if (slice >= p.ns) continue;
-      __half h[4];
+    for (int ph = 0; ph < 16 / WAVES; ++ph) {
 #pragma unroll
-      for (int t4 = 0; t4 < 4; ++t4) {
-        h[t4] = __float2half_rn(acc[t4][fm][v]);
-        if (bias) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
+      for (int j = 0; j < WAVES; ++j) {
+        const int v = ph * WAVES + j;
+        red[wave][j][lane] = make_float4(acc[0][fm][v], acc[1][fm][v], acc[2][fm][v], acc[3][fm][v]);
       }
-      u32x2 o;
-      o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
-      o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-      *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+      LdsBarrier();
+      float4 sum = red[0][wave][lane];
+#pragma unroll
+      for (int c = 1; c < WAVES; ++c) {
+        const float4 o = red[c][wave][lane];
+        sum.x += o.x;
+        sum.y += o.y;
+        sum.z += o.z;
+        sum.w += o.w;
+      }
+      const int v = ph * WAVES + wave;
+      const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
+      if (mi < p.m && slice < p.ns) {
+        __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
+        if (bias) {
+#pragma unroll
+          for (int t4 = 0; t4 < 4; ++t4) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
+        }
+        u32x2 o;
+        o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+        o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+        *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+      }
+      if (fm + 1 < FM || ph + 1 < 16 / WAVES) LdsBarrier();
     }
   }
 }
@@ -579,6 +588,8 @@ bool FcW4MfmaSupported(const FcArgs& a) {
   if (a.scale_kind == kScaleBlock) {
     // an MFMA step of 16 input channels must not straddle scale groups
     if (a.groups <= 0 || a.k % a.groups != 0 || (a.k / a.groups) % 16 != 0) return false;
+    const int steps_per_group = (a.k / a.groups) / 16;
+    if (steps_per_group & (steps_per_group - 1)) return false;  // the kernel finds the group by a shift
   }
   return true;
 }
@@ -608,7 +619,6 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   p.s_bytes = (uint32_t)((size_t)p.groups * p.ns * 8);
   p.group_size = a.scale_kind == kScaleBlock ? a.k / a.groups : a.k;
   p.group_shift = -1;
-  p.debug = std::getenv("MLDHIP_DEBUG") ? std::atoi(std::getenv("MLDHIP_DEBUG")) : 0;
   if (a.scale_kind != kScaleBlock) {
     p.group_shift = 30;  // one group
   } else {
@@ -629,7 +639,7 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   if (const char* e = std::getenv("MLDHIP_GEMM_WAVES")) waves = std::atoi(e);
   if (fm == 2) {
     if (waves == 8)
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 2, 8>), grid, dim3(512), 0, stream, p);
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4, 8>), grid, dim3(512), 0, stream, p);
     else if (u == 8)
       hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 8, 4>), grid, dim3(256), 0, stream, p);
     else
