@@ -1,22 +1,18 @@
-// Prefill-side kernels for gfx950: LDS-tiled MFMA GEMMs.
+// Prefill-side kernels for gfx950: MFMA GEMMs.
 //
-//  fc_w4_mfma_gemm_kernel   multi-token FullyConnected over the packed int4 I4O4 buffer: the
-//                           work-group dequantizes its weight tile into LDS as fp16 (one
-//                           rounding per weight: round((u-8)*s), like the reference's
-//                           fma(u, s, -8s)), then v_mfma_f32_32x32x16_f16 with fp32 accumulation.
+//  fc_w4_mfma_gemm_kernel   multi-token FullyConnected over the packed int4 I4O4 buffer: every
+//                           wave dequantizes its weight operands in registers (one rounding per
+//                           weight: round((u-8)*s), like the reference's fma(u, s, -8s)), then
+//                           v_mfma_f32_32x32x16_f16 with fp32 accumulation; no LDS in the loop.
 //  conv_int8_mfma_kernel    int8 codes x int8 weights with v_mfma_i32_32x32x32_i8 (int32
-//                           accumulators, exact), then the reference's rescale epilogue.
+//                           accumulators, exact), tiles streamed global -> LDS without passing
+//                           through registers, then the reference's rescale epilogue.
 //
-// Both share one skeleton.  Operand roles: the MFMA "A" operand is the weight tile (rows =
-// output channels), "B" is the activation tile (columns = tokens).  In the 32x32 result a lane
-// then holds, for one token, groups of 4 consecutive output channels: exactly one 4-channel
-// slice of the slice-major output tensor, so a lane stores 8 (fp16) or 16 bytes and 32 lanes
-// store consecutive tokens.
-//
-// LDS holds both tiles as [k-group][row][16 bytes]; a k-group is 8 halfs (fp16 path) or 16
-// bytes (int8 path), i.e. what one lane feeds to one MFMA.  A K-step is 4 k-groups (32 or 64
-// input channels): two MFMA steps.  Tiles are double-buffered: the global loads of step t+1
-// are issued before the MFMAs of step t and written to the other buffer afterwards.
+// Operand roles in both: the MFMA "A" operand is the weight tile (rows = output channels), "B"
+// is the activation tile (columns = tokens).  In the 32x32 result a lane then holds, for one
+// token, groups of 4 consecutive output channels: exactly one 4-channel slice of the
+// slice-major output tensor, so a lane stores 8 (fp16) or 16 bytes and 32 lanes store
+// consecutive tokens.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -36,8 +32,6 @@ typedef int int4v_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;
-constexpr int KG = 4;  // k-groups per K-step
 
 struct GemmParams {
   int m, n, k;
@@ -100,258 +94,358 @@ __device__ __forceinline__ float Rescale(int acc, float ws, int wsum, float src_
 }
 #pragma clang fp contract(fast)
 
-template <bool W4, int FN, int FM, int D>  // D: register stages, even
-__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(GemmParams p) {
-  constexpr int BN = 2 * FN * 32;
-  constexpr int BM = 2 * FM * 32;
-  __shared__ u32x4 sA[2][KG][BN];
-  __shared__ u32x4 sB[2][KG][BM];
+// ------------------------------------------------------------------------------------------
+// int8 x int8 GEMM.
+//
+// Both operands are stored the way the MFMA wants them: [k16][row][16 bytes], i.e. a lane's
+// operand for v_mfma_i32_32x32x32_i8 (row r = lane % 32, 16 consecutive k of unit 2*step +
+// lane / 32) is one aligned 16-byte item, and 64 consecutive rows of a unit are 1 KB of
+// contiguous memory.  A work-group of 4 waves (2 x 2) owns 256 channels x BM tokens; each wave
+// 128 x (BM / 2).  K advances in stages of 4 units (64 values of k, two MFMA steps).  A stage of
+// both tiles is copied global -> LDS by buffer loads that write LDS directly (no registers, no
+// ds_write); rows past the matrix and units past K are out of the buffers' range and arrive
+// as zeros.  kStages stages rotate through LDS, so kStages - 1 stages of loads are in flight
+// behind the one being multiplied, and there is one barrier per stage.
+//
+// The compiler does not know what the LDS-writing loads touch, so the LDS side is explicit
+// here: operand reads are inline ds_read_b128, followed by a counter wait that is tied to the
+// registers it guards.
+// ------------------------------------------------------------------------------------------
+constexpr int kI8Stages = 4;
+constexpr int kI8Threads = 256;
+
+template <int OFF>
+__device__ __forceinline__ void DsRead128(u32x4& dst, uint32_t addr) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int N>
+__device__ __forceinline__ void LdsWait(u32x4 (&f)[N]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(f[i]));
+}
+
+// 64 lanes x 16 bytes from the buffer (a lane's offset beyond the range gives zeros) to 1 KB of
+// LDS starting at `dst`, which is the same for the whole wave.
+typedef __attribute__((address_space(3))) char* LdsPtr;
+__device__ __forceinline__ void CopyToLds(__amdgpu_buffer_rsrc_t rsrc, LdsPtr dst, uint32_t lane_offset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)dst, 16, lane_offset, 0, 0, 0);
+}
+
+// Operand read number i of one MFMA step: 4 weight items, then FM token items, 512 bytes apart.
+template <int FM, int OFF_A, int OFF_B>
+__device__ __forceinline__ void ReadOperand(int i, u32x4 (&a)[4], u32x4 (&b)[FM], uint32_t aa, uint32_t ab) {
+  switch (i) {  // i is a constant after unrolling
+    case 0: DsRead128<OFF_A + 0 * 512>(a[0], aa); break;
+    case 1: DsRead128<OFF_A + 1 * 512>(a[1], aa); break;
+    case 2: DsRead128<OFF_A + 2 * 512>(a[2], aa); break;
+    case 3: DsRead128<OFF_A + 3 * 512>(a[3], aa); break;
+    case 4: DsRead128<OFF_B + 0 * 512>(b[0], ab); break;
+    case 5: if constexpr (FM > 1) DsRead128<OFF_B + 1 * 512>(b[1], ab); break;
+    case 6: if constexpr (FM > 2) DsRead128<OFF_B + 2 * 512>(b[2], ab); break;
+    case 7: if constexpr (FM > 2) DsRead128<OFF_B + 3 * 512>(b[3], ab); break;
+  }
+}
+
+// One MFMA step on (cur_a, cur_b) with the wave's other work threaded between the MFMAs, so
+// that the matrix unit never waits for it: first the 4 + FM operand reads of the next step (into
+// nxt_a / nxt_b), then, if COPY, this wave's 4 + FM global -> LDS copies of a later stage.  The
+// fences fix that order; an MFMA occupies the unit for 32 cycles, the other instructions issue
+// in its shadow.
+template <int FM, int OFF_A, int OFF_B, bool COPY, typename CopyOne>
+__device__ __forceinline__ void MultiplyAndFetch(int16v_t (&acc)[4][FM], u32x4 (&cur_a)[4], u32x4 (&cur_b)[FM],
+                                                 u32x4 (&nxt_a)[4], u32x4 (&nxt_b)[FM], uint32_t aa, uint32_t ab,
+                                                 CopyOne&& copy_one) {
+  constexpr int kReads = 4 + FM;
+  constexpr int kItems = COPY ? 2 * kReads : kReads;
+  constexpr int kMfmas = 4 * FM;
+  constexpr int kPerSlot = (kItems + kMfmas - 1) / kMfmas;
+#pragma unroll
+  for (int idx = 0; idx < kMfmas; ++idx) {
+    const int fn = idx / FM, fm = idx % FM;
+    acc[fn][fm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4v_t, cur_a[fn]),
+                                                        __builtin_bit_cast(int4v_t, cur_b[fm]), acc[fn][fm], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int item = idx * kPerSlot; item < (idx + 1) * kPerSlot && item < kItems; ++item) {
+      if (item < kReads)
+        ReadOperand<FM, OFF_A, OFF_B>(item, nxt_a, nxt_b, aa, ab);
+      else
+        copy_one(item - kReads);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+// DST: element type of the output (MLDHIP_FLOAT16 / FLOAT32 / INT32); ZP: weights have a zero point.
+template <int FM, int DST, bool ZP>
+__global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p) {
+  constexpr int FN = 4;
+  constexpr int BN = 2 * FN * 32;              // 256 channels
+  constexpr int BM = 2 * FM * 32;              // tokens
+  constexpr int kABytes = 4 * BN * 16;         // one stage of the weight tile
+  constexpr int kBBytes = 4 * BM * 16;         // one stage of the token tile
+  constexpr int kStageBytes = kABytes + kBBytes;
+  constexpr int kLoadsPerStage = BN / 64 + BM / 64;  // per wave
+  __shared__ u32x4 smem[kI8Stages * kStageBytes / 16];
+  const LdsPtr lds = (LdsPtr)smem;
+  const uint32_t lds_base = (uint32_t)(size_t)lds;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
-  const int n0 = blockIdx.x * BN;
-  const int m0 = blockIdx.y * BM;
   const int r32 = lane & 31, g2 = lane >> 5;
 
-  // ---- staging registers -----------------------------------------------------------------
-  // fp16 path: A items (k-group g, slice nsl) -> two 8-byte blocks; B items (K-slice, token) 8 B.
-  // int8 path: A / B items (k-group, row) -> 16 bytes.
-  constexpr int A_ITEMS = W4 ? KG * (BN / 4) : KG * BN;
-  constexpr int B_ITEMS = W4 ? (KG * 2) * BM : KG * BM;
-  constexpr int NA = (A_ITEMS + kThreads - 1) / kThreads;
-  constexpr int NB = (B_ITEMS + kThreads - 1) / kThreads;
-  // D register stages: tile t is fetched D K-steps before it is multiplied, so D-1 tiles of
-  // global loads are in flight while the MFMAs of the current tile run.
-  u32x4 ra_[D][NA];  // fp16 path: {blk0.x, blk0.y, blk1.x, blk1.y}
-  u32x2 rs_[D][NA];  // fp16 path: the 4 scales of the item's slice
-  u32x4 rb_[D][W4 ? 1 : NB];
-  u32x2 rb2_[D][W4 ? NB : 1];  // fp16 path: 8-byte activation items
+  // Tile order.  Work-groups go round-robin to the 8 XCDs (id % 8), each with its own L2; XCD x
+  // takes the contiguous range [x*per_xcd, (x+1)*per_xcd) of a numbering that walks blocks of
+  // 8 channel tiles token-tile by token-tile, so the tiles that share an L2 form a compact
+  // rectangle and re-use each other's operands.
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const int tiles_m = (p.m + BM - 1) / BM;
+  const int per_xcd = (tiles_n * tiles_m + 7) / 8;
+  const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= tiles_n * tiles_m) return;
+  int tn, tm;
+  {
+    const int full = tiles_n / 8;
+    if (tile < full * 8 * tiles_m) {
+      const int sc = tile / (8 * tiles_m), within = tile % (8 * tiles_m);
+      tn = sc * 8 + within % 8;
+      tm = within / 8;
+    } else {
+      const int rest = tile - full * 8 * tiles_m, width = tiles_n - full * 8;
+      tn = full * 8 + rest % width;
+      tm = rest / width;
+    }
+  }
+  const int n0 = tn * BN;
+  const int m0 = tm * BM;
 
-  // All tile loads are raw buffer loads: out-of-range items get an offset beyond the buffer and
-  // read as zero, so the loop body stays free of branches and the loads of several stages stay
-  // in flight (a zero activation or a zero scale makes the padded product vanish).
   constexpr uint32_t kOob = 0x7FFFFFF0u;
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<void*>(W4 ? static_cast<const void*>(p.w4) : static_cast<const void*>(p.wi8)), 0, p.a_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<void*>(W4 ? static_cast<const void*>(p.act) : static_cast<const void*>(p.codes)), 0, p.b_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_s =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_a =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(p.wi8), 0, p.a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(p.codes), 0, p.b_bytes, 0x00020000);
 
-  auto load_tiles = [&](int kt, u32x4 (&ra)[NA], u32x2 (&rs)[NA], u32x4 (&rb)[W4 ? 1 : NB],
-                        u32x2 (&rb2)[W4 ? NB : 1]) {
-    if (W4) {
+  // Copy duty of this wave: unit `wave` of every stage, all rows, 64 rows per instruction.
+  // A lane's byte offset advances by one stage per copy; rows past the matrix stay parked
+  // beyond the range.
+  uint32_t va[BN / 64], vb[BM / 64], sa[BN / 64], sb[BM / 64];
 #pragma unroll
-      for (int q = 0; q < NA; ++q) {
-        const int it = tid + q * kThreads;
-        const int g = it / (BN / 4), nsl = it % (BN / 4);
-        const int nsi = n0 / 4 + nsl;
-        const int ksa = (kt * KG + g) * 2;
-        const bool ok = it < A_ITEMS && nsi < p.ns;
-        const uint32_t off0 = ok ? (uint32_t)(ksa * p.ns + nsi) * 8u : kOob;
-        const uint32_t off1 = ok ? off0 + (uint32_t)p.ns * 8u : kOob;
-        const u32x2 b0 = __builtin_amdgcn_raw_buffer_load_b64(rsrc_a, off0, 0, 0);
-        const u32x2 b1 = __builtin_amdgcn_raw_buffer_load_b64(rsrc_a, off1, 0, 0);
-        ra[q] = u32x4{b0[0], b0[1], b1[0], b1[1]};
-        int grp = kt / p.steps_per_group;
-        grp = grp < p.groups ? grp : p.groups - 1;
-        rs[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, ok ? (uint32_t)(grp * p.ns + nsi) * 8u : kOob, 0, 0);
-      }
+  for (int rg = 0; rg < BN / 64; ++rg) {
+    const int row = n0 + rg * 64 + lane;
+    va[rg] = row < p.n ? (uint32_t)(wave * p.n + row) * 16u : kOob;
+    sa[rg] = row < p.n ? (uint32_t)p.n * 64u : 0u;
+  }
 #pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        const int it = tid + q * kThreads;
-        const int ksl = it / BM, ml = it % BM;
-        const int ksi = kt * KG * 2 + ksl;
-        const int mi = m0 + ml;
-        const bool ok = it < B_ITEMS && mi < p.m;
-        rb2[q] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_b, ok ? (uint32_t)(ksi * p.m + mi) * 8u : kOob, 0, 0);
-      }
+  for (int rg = 0; rg < BM / 64; ++rg) {
+    const int row = m0 + rg * 64 + lane;
+    vb[rg] = row < p.m ? (uint32_t)(wave * p.m + row) * 16u : kOob;
+    sb[rg] = row < p.m ? (uint32_t)p.m * 64u : 0u;
+  }
+  // copy number c of a stage: weight row groups first, then token row groups
+  auto copy_one = [&](int slot, int c) {
+    const LdsPtr base = lds + slot * kStageBytes;
+    if (c < BN / 64) {
+      CopyToLds(rsrc_a, base + (wave * BN + c * 64) * 16, va[c]);
+      va[c] += sa[c];
     } else {
-#pragma unroll
-      for (int q = 0; q < NA; ++q) {
-        const int it = tid + q * kThreads;
-        const int g = it / BN, r = it % BN;
-        const int kg = kt * KG + g;
-        const bool ok = it < A_ITEMS && n0 + r < p.n;
-        ra[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? (uint32_t)(kg * p.n + n0 + r) * 16u : kOob, 0, 0);
-      }
-#pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        const int it = tid + q * kThreads;
-        const int g = it / BM, r = it % BM;
-        const int kg = kt * KG + g;
-        const bool ok = it < B_ITEMS && m0 + r < p.m;
-        rb[q] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? (uint32_t)(kg * p.m + m0 + r) * 16u : kOob, 0, 0);
-      }
+      const int rg = c - BN / 64;
+      CopyToLds(rsrc_b, base + kABytes + (wave * BM + rg * 64) * 16, vb[rg]);
+      vb[rg] += sb[rg];
     }
   };
 
-  auto store_tiles = [&](int buf, u32x4 (&ra)[NA], u32x2 (&rs)[NA], u32x4 (&rb)[W4 ? 1 : NB],
-                         u32x2 (&rb2)[W4 ? NB : 1]) {
-    if (W4) {
-      const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
-      const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
-#pragma unroll
-      for (int q = 0; q < NA; ++q) {
-        const int it = tid + q * kThreads;
-        if (it >= A_ITEMS) continue;
-        const int g = it / (BN / 4), nsl = it % (BN / 4);
-#pragma unroll
-        for (int o = 0; o < 4; ++o) {
-          // scale of output o in both halves
-          const uint32_t sw = rs[q][o >> 1];
-          const uint32_t s16 = (o & 1) ? (sw >> 16) : (sw & 0xFFFFu);
-          const half2_t s2 = AsHalf2(s16 | (s16 << 16));
-          u32x4 row;
-#pragma unroll
-          for (int wd = 0; wd < 4; ++wd) {
-            const uint32_t x = (o & 2) ? (ra[q][wd] >> 8) : ra[q][wd];
-            const uint32_t bits = (o & 1) ? AndOr(x, p.mask_hi, p.magic_hi) : AndOr(x, p.mask_lo, p.magic_lo);
-            const half2_t centered = AsHalf2(bits) + ((o & 1) ? off_hi : off_lo);
-            row[wd] = AsU32(centered * s2);
-          }
-          sA[buf][g][nsl * 4 + o] = row;
-        }
-      }
-#pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        const int it = tid + q * kThreads;
-        if (it >= B_ITEMS) continue;
-        const int ksl = it / BM, ml = it % BM;
-        u32x2* dst2 = reinterpret_cast<u32x2*>(&sB[buf][ksl >> 1][ml]) + (ksl & 1);
-        *dst2 = rb2[q];
-      }
-    } else {
-#pragma unroll
-      for (int q = 0; q < NA; ++q) {
-        const int it = tid + q * kThreads;
-        if (it < A_ITEMS) sA[buf][it / BN][it % BN] = ra[q];
-      }
-#pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        const int it = tid + q * kThreads;
-        if (it < B_ITEMS) sB[buf][it / BM][it % BM] = rb[q];
-      }
-    }
-  };
+  // operand addresses inside a stage
+  const uint32_t addr_a = lds_base + (uint32_t)(g2 * BN + wn * FN * 32 + r32) * 16u;
+  const uint32_t addr_b = lds_base + (uint32_t)kABytes + (uint32_t)(g2 * BM + wm * FM * 32 + r32) * 16u;
 
-  // ---- accumulators -----------------------------------------------------------------------
-  float16_t accf[FN][FM];
-  int16v_t acci[FN][FM];
+  int16v_t acc[FN][FM];
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn)
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        if (W4)
-          accf[fn][fm][v] = 0.0f;
-        else
-          acci[fn][fm][v] = 0;
-      }
+      for (int v = 0; v < 16; ++v) acc[fn][fm][v] = 0;
+  // Waits until at most `pending` stages of this wave's copies are still in flight, then meets
+  // the other waves: after it, the stage is complete in LDS and nobody reads the slot that the
+  // next copy overwrites.
+  auto stage_barrier = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((kI8Stages - 2) * kLoadsPerStage) : "memory");
+  };
 
-  // prologue: tiles 0 .. D-1 into the register stages, tile 0 on into LDS.  The loop below
-  // has no conditions: it runs a multiple of D steps, tiles beyond K read as zeros (buffer
-  // range check) and add nothing.
+  const int stages = (p.k16 + 3) / 4;
+  // prologue: stages 0 .. kStages-2 in flight, stage 0 landed, its first operands requested
 #pragma unroll
-  for (int d = 0; d < D; ++d) load_tiles(d, ra_[d], rs_[d], rb_[d], rb2_[d]);
-  store_tiles(0, ra_[0], rs_[0], rb_[0], rb2_[0]);
-  __syncthreads();
-  const int k_steps_padded = (p.k_steps + D - 1) / D * D;
-  for (int kt0 = 0; kt0 < k_steps_padded; kt0 += D) {
+  for (int s = 0; s < kI8Stages - 1; ++s)
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int kt = kt0 + d;
-      const int buf = d & 1;  // D is even, so the LDS buffer of a stage is fixed
-      // stage d held tile kt (already in LDS): refill it with tile kt + D
-      load_tiles(kt + D, ra_[d], rs_[d], rb_[d], rb2_[d]);
+    for (int c = 0; c < kLoadsPerStage; ++c) copy_one(s, c);
+  stage_barrier();
+  u32x4 fa[2][FN], fb[2][FM];
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        u32x4 a[FN], b[FM];
-#pragma unroll
-        for (int fn = 0; fn < FN; ++fn) a[fn] = sA[buf][2 * s + g2][(wn * FN + fn) * 32 + r32];
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm) b[fm] = sB[buf][2 * s + g2][(wm * FM + fm) * 32 + r32];
-#pragma unroll
-        for (int fn = 0; fn < FN; ++fn)
-#pragma unroll
-          for (int fm = 0; fm < FM; ++fm) {
-            if (W4)
-              accf[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                  __builtin_bit_cast(half8_t, a[fn]), __builtin_bit_cast(half8_t, b[fm]), accf[fn][fm], 0, 0, 0);
-            else
-              acci[fn][fm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
-                  __builtin_bit_cast(int4v_t, a[fn]), __builtin_bit_cast(int4v_t, b[fm]), acci[fn][fm], 0, 0, 0);
-          }
-      }
-      {
-        const int dn = (d + 1) % D;
-        store_tiles(buf ^ 1, ra_[dn], rs_[dn], rb_[dn], rb2_[dn]);
-      }
-      __syncthreads();
-    }
+  for (int i = 0; i < 4 + FM; ++i) ReadOperand<FM, 0, 0>(i, fa[0], fb[0], addr_a, addr_b);
+  int slot = 0;  // slot of stage t
+  for (int t = 0; t < stages; ++t) {
+    const uint32_t aa = addr_a + (uint32_t)(slot * kStageBytes);
+    const uint32_t ab = addr_b + (uint32_t)(slot * kStageBytes);
+    // the slot of stage t-1 takes stage t + kStages - 1 (copies past K read zeros)
+    const int refill = slot == 0 ? kI8Stages - 1 : slot - 1;
+    LdsWait(fa[0]);
+    LdsWait(fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    MultiplyAndFetch<FM, 2 * BN * 16, 2 * BM * 16, true>(acc, fa[0], fb[0], fa[1], fb[1], aa, ab,
+                                                         [&](int c) { copy_one(refill, c); });
+    LdsWait(fa[1]);
+    LdsWait(fb[1]);
+    stage_barrier();  // stage t+1 complete for every wave
+    slot = slot == kI8Stages - 1 ? 0 : slot + 1;
+    const uint32_t na = addr_a + (uint32_t)(slot * kStageBytes);
+    const uint32_t nb = addr_b + (uint32_t)(slot * kStageBytes);
+    __builtin_amdgcn_sched_barrier(0);
+    MultiplyAndFetch<FM, 0, 0, false>(acc, fa[1], fb[1], fa[0], fb[0], na, nb, [](int) {});
   }
+  // drain the copies that ran ahead before the work-group's LDS is released
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  if constexpr (DST == MLDHIP_FLOAT16) __syncthreads();  // LDS is reused for the output tile
 
   // ---- epilogue ---------------------------------------------------------------------------
+  // Register v of the 32x32 result belongs to channel 8*(v/4) + 4*g2 + v%4 of the MFMA's 32 and to
+  // token r32: four consecutive registers are one 4-channel slice of one token.  The channel
+  // constants are fetched once per slice and used for the FM token blocks.
+  int mi[FM];
+  float src_scale[FM], src_zp[FM], src_sum[FM];
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
-    const int mi = m0 + (wm * FM + fm) * 32 + r32;
-    if (mi >= p.m) continue;
-    float src_scale = 0.0f, src_zp = 0.0f, src_sum = 0.0f;
-    if (!W4 && p.dst_type != MLDHIP_INT32) {
-      const float4 pr = *reinterpret_cast<const float4*>(p.params + (size_t)mi * 4);
-      src_scale = pr.x;
-      src_zp = pr.y;
-      src_sum = pr.z;
+    mi[fm] = m0 + (wm * FM + fm) * 32 + r32;
+    src_scale[fm] = src_zp[fm] = src_sum[fm] = 0.0f;
+    if (DST != MLDHIP_INT32) {
+      const float4 pr = *reinterpret_cast<const float4*>(p.params + (size_t)min(mi[fm], p.m - 1) * 4);
+      src_scale[fm] = pr.x;
+      src_zp[fm] = pr.y;
+      src_sum[fm] = pr.z;
     }
+  }
+  constexpr bool has_zp = ZP;
+  const float in_channels = (float)p.k;
+  if constexpr (DST == MLDHIP_FLOAT16) {
+    // Straight-line: every register of the tile is rescaled and staged in LDS as
+    // [slice of the tile][token of the tile][4 halfs]; what lies outside the matrix is computed
+    // from clamped constants and never leaves LDS.
+    const bool has_bias = p.bias != nullptr;
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) {
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
-        const int nb = n0 + (wn * FN + fn) * 32 + 8 * v4 + 4 * g2;  // first of 4 consecutive channels
-        const int slice = nb >> 2;
-        if (slice >= p.ns) continue;
-        const size_t o_idx = ((size_t)slice * p.m + mi) * 4;
-        float r[4];
-        if (W4) {
+        const int slice_l = (wn * FN + fn) * 8 + v4 * 2 + g2;
+        const int nb = min(n0 / 4 + slice_l, p.ns - 1) * 4;  // first of 4 consecutive channels
+        // the per-channel tensors are padded to whole slices
+        const float4 ws = *reinterpret_cast<const float4*>(p.wscale + nb);
+        const int4v_t wsum = *reinterpret_cast<const int4v_t*>(p.wsum + nb);
+        const float4 wzp = has_zp ? *reinterpret_cast<const float4*>(p.wzp + nb) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        const float wsc[4] = {ws.x, ws.y, ws.z, ws.w};
+        const float wz[4] = {wzp.x, wzp.y, wzp.z, wzp.w};
+        u32x2 bias2 = {0x80008000u, 0x80008000u};  // -0.0: adding it changes nothing, not even the sign of a zero
+        if (has_bias) bias2 = *reinterpret_cast<const u32x2*>(static_cast<const __half*>(p.bias) + nb);
+        const __half bias_h[4] = {__ushort_as_half((unsigned short)(bias2[0] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[0] >> 16)),
+                                  __ushort_as_half((unsigned short)(bias2[1] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[1] >> 16))};
 #pragma unroll
-          for (int c = 0; c < 4; ++c) r[c] = accf[fn][fm][v4 * 4 + c];
-        } else if (p.dst_type == MLDHIP_INT32) {
-          int4v_t o = {acci[fn][fm][v4 * 4], acci[fn][fm][v4 * 4 + 1], acci[fn][fm][v4 * 4 + 2],
-                       acci[fn][fm][v4 * 4 + 3]};
-          *reinterpret_cast<int4v_t*>(static_cast<int*>(p.dst) + o_idx) = o;
-          continue;
-        } else {
-#pragma unroll
-          for (int c = 0; c < 4; ++c)
-            r[c] = Rescale(acci[fn][fm][v4 * 4 + c], p.wscale[nb + c], p.wsum[nb + c], src_scale, src_zp,
-                           p.wzp != nullptr, p.wzp ? p.wzp[nb + c] : 0.0f, src_sum, (float)p.k);
-        }
-        if (p.dst_type == MLDHIP_FLOAT32) {
-          const float* bias = static_cast<const float*>(p.bias);
-          float4 o = make_float4(r[0], r[1], r[2], r[3]);
-          if (bias) {
-            o.x += bias[nb];
-            o.y += bias[nb + 1];
-            o.z += bias[nb + 2];
-            o.w += bias[nb + 3];
-          }
-          *reinterpret_cast<float4*>(static_cast<float*>(p.dst) + o_idx) = o;
-        } else {
-          const __half* bias = static_cast<const __half*>(p.bias);
+        for (int fm = 0; fm < FM; ++fm) {
           __half h[4];
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            h[c] = __float2half_rn(r[c]);
-            if (bias) h[c] = __hadd(h[c], bias[nb + c]);
+            const float r = Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp, wz[c],
+                                    src_sum[fm], in_channels);
+            h[c] = __float2half_rn(r);
+            h[c] = __hadd(h[c], bias_h[c]);
           }
           u32x2 o;
           o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
           o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-          *reinterpret_cast<u32x2*>(static_cast<__half*>(p.dst) + o_idx) = o;
+          const int token_l = (wm * FM + fm) * 32 + r32;
+          reinterpret_cast<u32x2*>(smem)[slice_l * BM + token_l] = o;
         }
+      }
+    }
+  } else {
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int nb = n0 + (wn * FN + fn) * 32 + 8 * v4 + 4 * g2;  // first of 4 consecutive channels
+      const int slice = nb >> 2;
+      if (slice >= p.ns) continue;
+      if constexpr (DST == MLDHIP_INT32) {
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+          if (mi[fm] >= p.m) continue;
+          int4v_t o = {acc[fn][fm][v4 * 4], acc[fn][fm][v4 * 4 + 1], acc[fn][fm][v4 * 4 + 2], acc[fn][fm][v4 * 4 + 3]};
+          *reinterpret_cast<int4v_t*>(static_cast<int*>(p.dst) + ((size_t)slice * p.m + mi[fm]) * 4) = o;
+        }
+        continue;
+      } else {
+      // the per-channel tensors are padded to whole slices
+      const float4 ws = *reinterpret_cast<const float4*>(p.wscale + nb);
+      const int4v_t wsum = *reinterpret_cast<const int4v_t*>(p.wsum + nb);
+      const float4 wzp = has_zp ? *reinterpret_cast<const float4*>(p.wzp + nb) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      const float wsc[4] = {ws.x, ws.y, ws.z, ws.w};
+      const float wz[4] = {wzp.x, wzp.y, wzp.z, wzp.w};
+      float bias_f[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (p.bias) {
+        const float4 bv = *reinterpret_cast<const float4*>(static_cast<const float*>(p.bias) + nb);
+        bias_f[0] = bv.x;
+        bias_f[1] = bv.y;
+        bias_f[2] = bv.z;
+        bias_f[3] = bv.w;
+      }
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm) {
+        if (mi[fm] >= p.m) continue;
+        const size_t o_idx = ((size_t)slice * p.m + mi[fm]) * 4;
+        float r[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          r[c] = Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp, wz[c], src_sum[fm],
+                         in_channels);
+        {
+          float4 o = make_float4(r[0], r[1], r[2], r[3]);
+          if (p.bias) {
+            o.x += bias_f[0];
+            o.y += bias_f[1];
+            o.z += bias_f[2];
+            o.w += bias_f[3];
+          }
+          *reinterpret_cast<float4*>(static_cast<float*>(p.dst) + o_idx) = o;
+        }
+      }
+      }
+    }
+  }
+  }
+  if constexpr (DST == MLDHIP_FLOAT16) {
+    // The staged tile leaves as whole slice rows: BM tokens x 8 bytes contiguous in memory, 16
+    // bytes per lane.  Work-groups start at different rows, so that at any moment the stores
+    // of the chip are spread over the memory channels instead of all hitting the same offset
+    // of their rows.
+    __syncthreads();
+    constexpr int kLanesPerRow = BM / 2;               // 16 bytes = 2 tokens per lane
+    constexpr int kRowsPerPass = kI8Threads / kLanesPerRow;
+    const int row_lane = tid % kLanesPerRow;
+    const int t0 = m0 + row_lane * 2;
+    const int rot = tile * 5;
+    __half* dst = static_cast<__half*>(p.dst);
+    for (int pass = 0; pass < BN / 4 / kRowsPerPass; ++pass) {
+      const int slice_l = (pass * kRowsPerPass + tid / kLanesPerRow + rot) % (BN / 4);
+      const int slice = n0 / 4 + slice_l;
+      if (slice >= p.ns || t0 >= p.m) continue;
+      const u32x4 v = smem[slice_l * kLanesPerRow + row_lane];
+      __half* out = dst + ((size_t)slice * p.m + t0) * 4;
+      // (an odd token count makes every other row start 8 bytes off a 16-byte boundary)
+      if (t0 + 1 < p.m && (p.m & 1) == 0) {
+        *reinterpret_cast<u32x4*>(out) = v;
+      } else {
+        *reinterpret_cast<u32x2*>(out) = u32x2{v[0], v[1]};
+        if (t0 + 1 < p.m) *reinterpret_cast<u32x2*>(out + 4) = u32x2{v[2], v[3]};
       }
     }
   }
@@ -553,26 +647,21 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   }
 }
 
-template <bool W4>
-hipError_t LaunchGemm(const GemmParams& p, hipStream_t stream) {
-  // Tile choice: the largest work-group tile that still gives every CU a work-group;
-  // small problems fall back to 64x64-per-wave tiles... the candidates are (FN, FM) in
-  // {(4,4), (4,2), (2,2), (2,1)} -> work-group tiles 256x256, 256x128, 128x128, 128x64 (N x M).
-  auto groups = [&](int bn, int bm) { return (long)DivUp(p.n, bn) * DivUp(p.m, bm); };
-  const long want = 200;
-  if (groups(256, 256) >= want) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 4, 2>), dim3(DivUp(p.n, 256), DivUp(p.m, 256)), dim3(kThreads), 0,
-                       stream, p);
-  } else if (groups(256, 128) >= want) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 4, 2, (W4 ? 6 : 4)>), dim3(DivUp(p.n, 256), DivUp(p.m, 128)), dim3(kThreads), 0,
-                       stream, p);
-  } else if (groups(128, 128) >= want || p.m > 64) {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 2, (W4 ? 8 : 6)>), dim3(DivUp(p.n, 128), DivUp(p.m, 128)), dim3(kThreads), 0,
-                       stream, p);
-  } else {
-    hipLaunchKernelGGL((mfma_gemm_kernel<W4, 2, 1, (W4 ? 8 : 6)>), dim3(DivUp(p.n, 128), DivUp(p.m, 64)), dim3(kThreads), 0,
-                       stream, p);
-  }
+template <int FM>
+hipError_t LaunchConvInt8Tile(const GemmParams& p, hipStream_t stream) {
+  const int tiles = DivUp(p.n, 256) * DivUp(p.m, 2 * FM * 32);
+  const dim3 grid(DivUp(tiles, 8) * 8), block(kI8Threads);
+  const bool zp = p.wzp != nullptr;
+  if (p.dst_type == MLDHIP_INT32)
+    hipLaunchKernelGGL((conv_int8_mfma_kernel<FM, MLDHIP_INT32, false>), grid, block, 0, stream, p);
+  else if (p.dst_type == MLDHIP_FLOAT32 && zp)
+    hipLaunchKernelGGL((conv_int8_mfma_kernel<FM, MLDHIP_FLOAT32, true>), grid, block, 0, stream, p);
+  else if (p.dst_type == MLDHIP_FLOAT32)
+    hipLaunchKernelGGL((conv_int8_mfma_kernel<FM, MLDHIP_FLOAT32, false>), grid, block, 0, stream, p);
+  else if (zp)
+    hipLaunchKernelGGL((conv_int8_mfma_kernel<FM, MLDHIP_FLOAT16, true>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((conv_int8_mfma_kernel<FM, MLDHIP_FLOAT16, false>), grid, block, 0, stream, p);
   return hipGetLastError();
 }
 
@@ -660,7 +749,6 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
   p.k = a.k;
   p.ns = DivUp(a.n, 4);
   p.k16 = DivUp(a.k, 16);
-  p.k_steps = DivUp(p.k16, KG);
   p.dst = a.dst;
   p.bias = a.bias;
   p.dst_type = a.dst_type;
@@ -675,7 +763,11 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
   p.b_bytes = (uint32_t)((size_t)p.k16 * p.m * 16);
   p.s_bytes = 0;
   if (kernel_name) *kernel_name = "conv_int8_mfma_kernel";
-  return LaunchGemm<false>(p, stream);
+  // token tile: the largest of 256 / 128 / 64 that still gives most CUs a work-group
+  auto tiles = [&](int bm) { return (long)DivUp(p.n, 256) * DivUp(p.m, bm); };
+  if (tiles(256) >= 200) return LaunchConvInt8Tile<4>(p, stream);
+  if (tiles(128) >= 200) return LaunchConvInt8Tile<2>(p, stream);
+  return LaunchConvInt8Tile<1>(p, stream);
 }
 
 }  // namespace mldhip
