@@ -1,0 +1,104 @@
+"""The FullyConnected sequence of a decoder stack (Gemma-2B-like: hidden 2048, MQA k/v 256,
+gated MLP 16384, int4 group-32 weights, fp16 tensors), as the reference's model builder emits
+it per layer (samples/llm/gemma3_model_builder.cc:1115-1128): q, k, v, o, gate, up, down.
+
+Only the FCs are reproduced (no attention, norm or activation): every FC reads a synthetic
+N(0,1) activation tensor of its input width and writes its own output tensor, and the FCs run
+in the graph's order on one stream, i.e. with the dependencies of the real layer.  Every
+layer owns its device copy of the packed weights and scales, so a decode step streams the
+whole stack's 1.1 GB through HBM.
+
+Nothing here computes a result on the host.
+"""
+import numpy as np
+
+import mldhip as M
+import workloads as W
+
+
+class DecoderStack:
+    def __init__(self, layers=W.C5_LAYERS, max_tokens=128, seed=5, layer_shapes=None, device="cuda"):
+        import torch
+        self.torch = torch
+        self.layers = layers
+        self.max_tokens = max_tokens
+        self.shapes = list(layer_shapes or W.C5_LAYER)
+        self.device = device
+        # host-side cases of one layer (all layers hold the same values in distinct memory)
+        self.cases = []
+        for idx, (name, k, n) in enumerate(self.shapes):
+            case = W.make_fc_case(seed=seed * 100 + idx, m=max_tokens, k=k, n=n, weight_bits=4,
+                                  tensor_dtype=np.float16, groups=k // 32)
+            case["name"] = name
+            self.cases.append(case)
+        # one activation tensor per input width, shared by the FCs that read that width
+        self.inputs = {}
+        for case in self.cases:
+            k = case["k"]
+            if k not in self.inputs:
+                self.inputs[k] = case["act"]
+        for case in self.cases:
+            case["act"] = self.inputs[case["k"]]
+        self.tokens = None
+        self.src = {}
+        self.nodes = []  # (layer, case index, op, out tensor)
+        packed = []
+        for case in self.cases:
+            desc, w = W.pack_fc_weights(case)
+            sc = M.scale_to_tensor(case["scale"], M.FLOAT16).view(np.float16)
+            packed.append((desc, torch.from_numpy(w), torch.from_numpy(sc)))
+        self._weights = []
+        for layer in range(layers):
+            for idx, case in enumerate(self.cases):
+                desc, w_host, s_host = packed[idx]
+                w_dev = w_host.to(device)
+                s_dev = s_host.to(device)
+                out = torch.zeros((W.div_up(case["n"], 4), max_tokens, 4), dtype=torch.float16, device=device)
+                op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, case["n"], case["k"], desc,
+                                 scale_shape=(case["n"], case["groups"]), max_tokens=max_tokens)
+                self._weights.append((w_dev, s_dev))
+                self.nodes.append((layer, idx, op, out, w_dev, s_dev))
+        self.set_tokens(1)
+
+    def weight_bytes(self):
+        """Packed weights + scales of the whole stack (the bytes a decode step must stream)."""
+        return sum(w.numel() * w.element_size() + s.numel() * s.element_size() for w, s in self._weights)
+
+    def flops(self, tokens):
+        return self.layers * sum(2.0 * tokens * c["k"] * c["n"] for c in self.cases)
+
+    def set_tokens(self, tokens):
+        """Re-binds every FC for `tokens` tokens (the first `tokens` rows of the synthetic input)."""
+        assert 1 <= tokens <= self.max_tokens
+        torch = self.torch
+        self.tokens = tokens
+        self.src = {k: torch.from_numpy(W.to_slices(a[:tokens]).astype(np.float16)).to(self.device)
+                    for k, a in self.inputs.items()}
+        self.outs = []
+        for layer, idx, op, out, w_dev, s_dev in self.nodes:
+            case = self.cases[idx]
+            view = out.view(-1)[: W.div_up(case["n"], 4) * tokens * 4].view(W.div_up(case["n"], 4), tokens, 4)
+            op.bind([self.src[case["k"]], w_dev, s_dev], [view])
+            op.set_shape(1, 1, tokens)
+            self.outs.append(view)
+
+    def launch(self, stream=None):
+        s = self.torch.cuda.current_stream().cuda_stream if stream is None else stream
+        for _, _, op, _, _, _ in self.nodes:
+            op.launch(s)
+
+    def result(self, layer, idx):
+        self.torch.cuda.synchronize()
+        pos = layer * len(self.cases) + idx
+        return W.from_slices(self.outs[pos].cpu().numpy().astype(np.float32), self.cases[idx]["n"])
+
+    def case(self, idx, tokens=None):
+        """The host-side case of FC `idx` restricted to the current token count."""
+        t = self.tokens if tokens is None else tokens
+        c = dict(self.cases[idx])
+        c["m"] = t
+        c["act"] = c["act"][:t]
+        return c
+
+    def kernel_names(self):
+        return [op.kernel_name for _, _, op, _, _, _ in self.nodes]

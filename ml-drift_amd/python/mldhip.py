@@ -228,11 +228,12 @@ class Op:
         self.handle = handle
 
     def __del__(self):
-        self.destroy()
+        if _lib is not None:  # (module globals are already cleared at interpreter shutdown)
+            self.destroy()
 
     def destroy(self):
         if getattr(self, "handle", None):
-            lib().mldhip_op_destroy(self.handle)
+            _lib.mldhip_op_destroy(self.handle)
             self.handle = None
 
     @property
