@@ -1,4 +1,5 @@
 // C-ABI layer: argument validation, op objects (the node executors), kernel dispatch.
+#include <algorithm>
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
@@ -282,7 +283,8 @@ int mldhip_fc_is_recommended(int precision, int tokens) {
 static int AllocWorkspace(mldhip_op* op, int n) {
   if (op->partial) return MLDHIP_OK;
   const int n_pad = DivUp(n, 4) * 4;
-  op->partial_floats = (size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad;
+  op->partial_floats = std::max((size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad,
+                                FcW4MfmaWorkspaceFloats(op->fc.max_tokens, op->fc.i, op->fc.o));
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&op->partial), op->partial_floats * sizeof(float));
   if (e != hipSuccess) return HipFail(e, "hipMalloc(workspace)");
   return MLDHIP_OK;
@@ -547,7 +549,7 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
       a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
       // split-K workspace of the streaming kernel: allocated once, on the first launch
-      if (a.m <= kGemvMaxTokens && a.weight_bits == 4 && a.act_f16)
+      if (a.weight_bits == 4 && a.act_f16)
         if (int rc = AllocWorkspace(op, d.o)) return rc;
       a.partial = op->partial;
       a.partial_floats = op->partial_floats;

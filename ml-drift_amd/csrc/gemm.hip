@@ -16,6 +16,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
 
 #include "../../include/mldhip.h"
@@ -59,6 +60,8 @@ struct GemmParams {
   // byte sizes of the A (weights), B (activations / codes) and scale buffers
   uint32_t a_bytes, b_bytes, s_bytes;
   int group_size;   // input channels per scale group (fp16 path)
+  int ksplit;       // work-groups along K per output tile (fp16 path)
+  float* partial;   // [ksplit][Ns][m][4] fp32 sums when ksplit > 1
   int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
 };
 
@@ -501,8 +504,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // past K itself) read zeros without a test in the loop; a lane without an output slice or
   // a token gets an offset beyond every buffer.
   const int steps_total = (p.k + 15) / 16;
-  const int per_wave = ((steps_total + WAVES - 1) / WAVES + U - 1) / U * U;  // multiple of U
-  const int t_begin = __builtin_amdgcn_readfirstlane(wave * per_wave);
+  const int shares = WAVES * p.ksplit;  // blockIdx.y selects the work-group's part of K
+  const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
+  const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * WAVES + wave) * per_wave);
   const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
@@ -631,7 +635,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       }
       const int v = ph * WAVES + wave;
       const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-      if (mi < p.m && slice < p.ns) {
+      if (mi < p.m && slice < p.ns && p.ksplit > 1) {
+        // this work-group's share of K: fp32 sums for the second pass
+        *reinterpret_cast<float4*>(p.partial + (((size_t)blockIdx.y * p.ns + slice) * p.m + mi) * 4) = sum;
+      } else if (mi < p.m && slice < p.ns) {
         __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
         if (bias) {
 #pragma unroll
@@ -645,6 +652,49 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       if (fm + 1 < FM || ph + 1 < 16 / WAVES) LdsBarrier();
     }
   }
+}
+
+// Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
+// the bias.  One thread per (slice, token).
+__global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) {
+  const size_t items = (size_t)p.ns * p.m;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= items) return;
+  const float4* part = reinterpret_cast<const float4*>(p.partial);
+  float4 sum = part[idx];
+  for (int s = 1; s < p.ksplit; ++s) {
+    const float4 o = part[(size_t)s * items + idx];
+    sum.x += o.x;
+    sum.y += o.y;
+    sum.z += o.z;
+    sum.w += o.w;
+  }
+  __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
+  if (p.bias) {
+    const __half* bias = static_cast<const __half*>(p.bias) + (idx / p.m) * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) h[c] = __hadd(h[c], bias[c]);
+  }
+  u32x2 o;
+  o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+  o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+  reinterpret_cast<u32x2*>(p.dst)[idx] = o;
+}
+
+// Token tile of the int4 GEMM: 64 when that still yields a work-group for half the CUs or M is
+// large, else 32.
+int W4TokenBlocks(int m, int n) {
+  const long tiles64 = (long)DivUp(n, 128) * DivUp(m, 64);
+  return (m > 32 && (tiles64 >= 128 || m > 64)) ? 2 : 1;
+}
+// K split across work-groups: doubled while the grid stays within the CU count and every wave
+// keeps at least 4 steps of 16 channels.
+int W4KSplit(int m, int k, int n) {
+  const long tiles = (long)DivUp(n, 128) * DivUp(m, W4TokenBlocks(m, n) * 32);
+  const int steps = DivUp(k, 16);
+  int s = 1;
+  while (s < 8 && tiles * s * 2 <= 256 && steps / (8 * s * 2) >= 4) s *= 2;
+  return s;
 }
 
 template <int FM>
@@ -717,13 +767,22 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   }
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
   // token tile: 64 when that still yields a work-group per CU or M is large, else 32
-  const long tiles64 = (long)DivUp(a.n, 128) * DivUp(a.m, 64);
-  int fm = (a.m > 32 && (tiles64 >= 128 || a.m > 64)) ? 2 : 1;
+  int fm = W4TokenBlocks(a.m, a.n);
   int u = 4;
   if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e);
   if (const char* e = std::getenv("MLDHIP_GEMM_U")) u = std::atoi(e);
   const int tiles = DivUp(a.n, 128) * DivUp(a.m, fm * 32);
-  const dim3 grid(DivUp(tiles, 8) * 8);
+  p.ksplit = 1;
+  p.partial = a.partial;
+  if (fm == W4TokenBlocks(a.m, a.n)) {
+    p.ksplit = W4KSplit(a.m, a.k, a.n);
+    while (p.ksplit > 1 && (size_t)p.ksplit * p.ns * 4 * a.m > a.partial_floats) p.ksplit /= 2;
+  }
+  if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) {
+    const int want = std::atoi(e);
+    if (want >= 1 && (size_t)want * p.ns * 4 * a.m <= a.partial_floats) p.ksplit = want;
+  }
+  const dim3 grid(DivUp(tiles, 8) * 8, p.ksplit);
   int waves = 8;
   if (const char* e = std::getenv("MLDHIP_GEMM_WAVES")) waves = std::atoi(e);
   if (fm == 2) {
@@ -739,7 +798,18 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
     else
       hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4, 4>), grid, dim3(256), 0, stream, p);
   }
+  if (p.ksplit > 1)
+    hipLaunchKernelGGL(fc_w4_splitk_reduce_kernel, dim3(DivUp(p.ns * a.m, 256)), dim3(256), 0, stream, p);
   return hipGetLastError();
+}
+
+size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n) {
+  size_t need = 0;
+  for (int m = kGemvMaxTokens + 1; m <= max_tokens; ++m) {
+    const int s = W4KSplit(m, k, n);
+    if (s > 1) need = std::max(need, (size_t)s * DivUp(n, 4) * 4 * m);
+  }
+  return need;
 }
 
 hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char** kernel_name) {
