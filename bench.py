@@ -32,8 +32,11 @@ HBM_PEAK_GBS = 8000.0
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=4000)
-    p.add_argument("--warmup", type=int, default=400)
+    p.add_argument("--steps", type=int, default=None, help="default 4000 (c2), 200 (c3, c4), 20 (c5-*)")
+    p.add_argument("--warmup", type=int, default=None, help="default steps / 10")
+    p.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5-decode", "c5-prefill"],
+                   help="c2 (default) is the headline line; the others time the remaining configurations "
+                        "the same way (one JSON line each, no CPU baseline)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
@@ -41,7 +44,122 @@ def parse():
     p.add_argument("--traffic-probe", action="store_true",
                    help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a 256 MiB device copy (the known-size "
                         "reference dispatch) followed by 64 launches over the weight ring, then exit")
-    return p.parse_args()
+    a = p.parse_args()
+    if a.steps is None:
+        a.steps = {"c2": 4000, "c3": 200, "c4": 200}.get(a.workload, 20)
+    if a.warmup is None:
+        a.warmup = max(1, a.steps // 10)
+    return a
+
+
+def time_graph(torch, stream, launch_step, steps, warmup):
+    """`warmup` eager steps, then a graph of `steps` steps: one untimed replay, one timed between two
+    events on `stream`.  Returns (wall seconds, event milliseconds)."""
+    s = stream.cuda_stream
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            launch_step(s, i)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            cs = torch.cuda.current_stream().cuda_stream
+            for i in range(steps):
+                launch_step(cs, i)
+        graph.replay()
+        stream.synchronize()
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(stream)
+        graph.replay()
+        ev1.record(stream)
+        stream.synchronize()
+        wall = time.perf_counter() - t0
+    return wall, ev0.elapsed_time(ev1)
+
+
+def run_other(args, torch, M, W):
+    """The configurations other than c2: same timing method, metric of their own roofline."""
+    stream = torch.cuda.Stream()
+    base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "data": "synthetic"}
+    if args.workload == "c3":
+        case = W.make_fc_case(**W.CONFIGS["c3"])
+        dev = W.FcDevice(case)
+        wall, ev_ms = time_graph(torch, stream, lambda s, i: dev.op.launch(s), args.steps, args.warmup)
+        flops = 2.0 * case["m"] * case["k"] * case["n"]
+        us = ev_ms * 1e3 / args.steps
+        out = dict(base, metric="int4_prefill_gemm_throughput", value=round(flops * args.steps / wall / 1e12, 1),
+                   unit="TFLOP/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+                   dtype="u4 weights x f16 activations, f32 accumulate (fp16 MFMA)",
+                   config={"workload": "c3: FullyConnected prefill GEMM M=512 K=4096 N=4096 int4 group-32, fp16 act/out",
+                           "flops_per_step": flops},
+                   roofline={"bound": "mfma", "kernel": dev.op.kernel_name, "achieved": round(flops / us / 1e6, 1),
+                             "peak": 2500.0, "unit": "TFLOP/s", "frac": round(flops / us / 1e6 / 2500.0, 4),
+                             "traffic": None, "avg_launch_us": round(us, 3)})
+    elif args.workload == "c4":
+        cfg = W.CONFIGS["c4"]
+        m, k, n = cfg["m"], cfg["k"], cfg["n"]
+        rng = np.random.default_rng(cfg["seed"])
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        w = rng.integers(-127, 128, size=(n, k), dtype=np.int8)
+        src = torch.from_numpy(W.to_slices(x)).cuda()
+        k16, ns = (k + 15) // 16, (n + 3) // 4
+        codes = torch.zeros((k16, m, 16), dtype=torch.int8, device="cuda")
+        params = torch.zeros((m, 4), dtype=torch.float32, device="cuda")
+        q = M.quantization_create(M.FLOAT16, M.PACKED_INT8C16, k, calculate_sum=False, symmetric=True, max_tokens=m)
+        q.bind([src], [codes, params])
+        q.set_shape(1, 1, m)
+        wd = M.conv_int8_weights_desc(n, k)
+        wt = torch.from_numpy(M.rearrange_int8(w, wd)).cuda()
+        wsum = torch.from_numpy(np.pad(w.astype(np.int32).sum(axis=1), (0, ns * 4 - n)).astype(np.int32)).cuda()
+        wscale = torch.full((ns * 4,), 1e-4, dtype=torch.float32, device="cuda")
+        out_t = torch.zeros((ns, m, 4), dtype=torch.float16, device="cuda")
+        conv = M.conv_int8_create(M.FLOAT16, n, k, wd, max_tokens=m)
+        conv.bind([codes, wt, params, wsum, wscale], [out_t])
+        conv.set_shape(1, 1, m)
+
+        def step(s, i):
+            q.launch(s)
+            conv.launch(s)
+        wall, _ = time_graph(torch, stream, step, args.steps, args.warmup)
+        _, conv_ms = time_graph(torch, stream, lambda s, i: conv.launch(s), args.steps, args.warmup)
+        _, q_ms = time_graph(torch, stream, lambda s, i: q.launch(s), args.steps, args.warmup)
+        ops = 2.0 * m * k * n
+        us = conv_ms * 1e3 / args.steps
+        out = dict(base, metric="int8_dynamic_gemm_throughput", value=round(ops * args.steps / wall / 1e12, 1),
+                   unit="TOP/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+                   dtype="i8 x i8, i32 accumulate (int8 MFMA), f32 rescale",
+                   config={"workload": "c4: per-token int8 quantization + int8 x int8 GEMM M=2048 K=2048 N=8192, fp16 out",
+                           "ops_per_step": ops, "quantize_us": round(q_ms * 1e3 / args.steps, 3)},
+                   roofline={"bound": "mfma", "kernel": conv.kernel_name, "achieved": round(ops / us / 1e6, 1),
+                             "peak": 5000.0, "unit": "TOP/s", "frac": round(ops / us / 1e6 / 5000.0, 4),
+                             "traffic": None, "avg_launch_us": round(us, 3)})
+    else:
+        from decoder_stack import DecoderStack
+        tokens = 1 if args.workload == "c5-decode" else 128
+        st = DecoderStack(max_tokens=128)
+        st.set_tokens(tokens)
+        wall, ev_ms = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
+        us = ev_ms * 1e3 / args.steps
+        wb, fl = st.weight_bytes(), st.flops(tokens)
+        if tokens == 1:
+            out = dict(base, metric="int4_decoder_stack_decode_hbm_bandwidth", value=round(wb * args.steps / wall / 1e9, 1),
+                       unit="GB/s", roofline={"bound": "hbm", "kernel": "fc_w4_stream_kernel (126 launches per step)",
+                                              "achieved": round(wb / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                              "frac": round(wb / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                                              "avg_step_us": round(us, 1)})
+        else:
+            out = dict(base, metric="int4_decoder_stack_prefill_throughput", value=round(fl * args.steps / wall / 1e12, 1),
+                       unit="TFLOP/s", roofline={"bound": "mfma", "kernel": "fc_w4_mfma_gemm_kernel (126 FCs per step)",
+                                                 "achieved": round(fl / us / 1e6, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                                                 "frac": round(fl / us / 1e6 / 2500.0, 4), "traffic": None,
+                                                 "avg_step_us": round(us, 1)})
+        out.update(ms_per_step=round(wall * 1e3 / args.steps, 6), dtype="u4 weights x f16 activations, f32 accumulate",
+                   config={"workload": "c5: 18 layers x (q,k,v,o,gate,up,down) int4 group-32, hidden 2048, %d token(s) per step"
+                                       % tokens, "weight_bytes_per_step": wb, "flops_per_step": fl})
+    print(json.dumps(out))
 
 
 def cpu_baseline(case, seconds):
@@ -86,6 +204,9 @@ def main():
         print("no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.workload != "c2":
+        run_other(args, torch, M, W)
+        return
     cfg = W.CONFIGS["c2"]
     case = W.make_fc_case(**cfg)
     m, k, n = case["m"], case["k"], case["n"]

@@ -335,20 +335,14 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous
   // bytes) keep K inside one work-group for wide layers; when the layer is too narrow for
   // that, K is split across work-groups and a second kernel adds the partials.
+  // Narrow layers take narrower strips (LPR = 4 or 2: 64- or 32-byte segments) before K is split:
+  // a second kernel costs more than the poorer coalescing of a matrix of a few MB.
   int lpr = 8, waves = 16;
-  {
-    // rows needed to cover K in one work-group step
-    const int strips8 = DivUp(p.row_u4, 8);
-    if (strips8 >= 192) {
-      lpr = 8;
-    } else if (DivUp(p.row_u4, 16) >= 192) {
-      lpr = 16;
-    } else {
-      lpr = 8;
-    }
-  }
+  const size_t weight_bytes = (size_t)p.ks * p.ns * 8;
+  if (DivUp(p.row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
+    lpr = DivUp(p.row_u4, 4) >= 128 ? 4 : 2;
   lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
-  if (lpr != 8 && lpr != 16) lpr = 8;
+  if (lpr != 2 && lpr != 4 && lpr != 8 && lpr != 16) lpr = 8;
   waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
   const int strips = DivUp(p.row_u4, lpr);
@@ -374,7 +368,11 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   dim3 grid(strips, p.ksplit);
   if (kernel_name) *kernel_name = "fc_w4_stream_kernel";
   hipError_t e;
-  if (lpr == 8)
+  if (lpr == 2)
+    e = LaunchCfgW<2>(p, waves, grouped, grid, stream);
+  else if (lpr == 4)
+    e = LaunchCfgW<4>(p, waves, grouped, grid, stream);
+  else if (lpr == 8)
     e = LaunchCfgW<8>(p, waves, grouped, grid, stream);
   else
     e = LaunchCfgW<16>(p, waves, grouped, grid, stream);
