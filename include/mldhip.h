@@ -262,6 +262,14 @@ int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w);
 /* ClOperation::AddToQueue (cl/cl_operation.cc:84-88): enqueue on `stream` (hipStream_t). */
 int mldhip_op_launch(mldhip_op* op, void* stream);
 
+/* One launch for up to 3 FullyConnected ops that read the same "src_tensor" (same binding, same
+ * shape, same K and scale grouping) and are served by the streaming int4 kernel, e.g. the
+ * q / k / v projections or the gate / up projections of a decoder layer, which the reference
+ * emits as separate nodes over one input (samples/llm/gemma3_model_builder.cc:1115-1128).
+ * Results are identical to launching the ops one by one.  Returns FAILED_PRECONDITION (and
+ * launches nothing) when the ops cannot share a launch; the caller then launches them singly. */
+int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream);
+
 /* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
  * at the current shape (GPUOperation::flops_/read_size_/write_size_,
  * common/task/gpu_operation.h:190-195). */

@@ -518,6 +518,37 @@ static int EnvFlag(const char* name) {
   return v && v[0] && v[0] != '0';
 }
 
+// The launch arguments of a floating-point FC op at its current bindings and shape; allocates
+// the op's split-K workspace on first use.
+static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
+  const mldhip_fc_desc& d = op->fc;
+  FcArgs a;
+  a.act = op->src_ptr[0];
+  a.weights = static_cast<const uint8_t*>(op->src_ptr[1]);
+  a.scale = op->idx_scale >= 0 ? op->src_ptr[op->idx_scale] : nullptr;
+  a.zero_point = op->idx_zp >= 0 ? op->src_ptr[op->idx_zp] : nullptr;
+  a.bias = op->idx_bias >= 0 ? op->src_ptr[op->idx_bias] : nullptr;
+  a.dst = op->dst_ptr[0];
+  a.m = op->Tokens();
+  a.k = d.i;
+  a.n = d.o;
+  a.act_f16 = d.src_type == MLDHIP_FLOAT16;
+  a.dst_f16 = d.dst_type == MLDHIP_FLOAT16;
+  a.weight_bits = WeightBits(d.weights.type);
+  a.scale_kind = d.scale_o * d.scale_i == 1 ? kScaleScalar : (d.scale_i == 1 ? kScaleLinear : kScaleBlock);
+  a.groups = d.scale_i;
+  a.scalar_scale = d.scalar_scale;
+  a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
+  a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
+  // split-K workspace of the int4 kernels: allocated once, on the first launch
+  if (a.weight_bits == 4 && a.act_f16)
+    if (int rc = AllocWorkspace(op, d.o)) return rc;
+  a.partial = op->partial;
+  a.partial_floats = op->partial_floats;
+  *out = a;
+  return MLDHIP_OK;
+}
+
 int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
   if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
   if (int rc = CheckBindings(op)) return rc;
@@ -531,28 +562,7 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
                            WeightBits(d.weights.type), stream, &op->last_kernel);
     } else {
       FcArgs a;
-      a.act = op->src_ptr[0];
-      a.weights = static_cast<const uint8_t*>(op->src_ptr[1]);
-      a.scale = op->idx_scale >= 0 ? op->src_ptr[op->idx_scale] : nullptr;
-      a.zero_point = op->idx_zp >= 0 ? op->src_ptr[op->idx_zp] : nullptr;
-      a.bias = op->idx_bias >= 0 ? op->src_ptr[op->idx_bias] : nullptr;
-      a.dst = op->dst_ptr[0];
-      a.m = op->Tokens();
-      a.k = d.i;
-      a.n = d.o;
-      a.act_f16 = d.src_type == MLDHIP_FLOAT16;
-      a.dst_f16 = d.dst_type == MLDHIP_FLOAT16;
-      a.weight_bits = WeightBits(d.weights.type);
-      a.scale_kind = d.scale_o * d.scale_i == 1 ? kScaleScalar : (d.scale_i == 1 ? kScaleLinear : kScaleBlock);
-      a.groups = d.scale_i;
-      a.scalar_scale = d.scalar_scale;
-      a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
-      a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
-      // split-K workspace of the streaming kernel: allocated once, on the first launch
-      if (a.weight_bits == 4 && a.act_f16)
-        if (int rc = AllocWorkspace(op, d.o)) return rc;
-      a.partial = op->partial;
-      a.partial_floats = op->partial_floats;
+      if (int rc = BuildFcArgs(op, &a)) return rc;
       const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
       if (!force_generic && FcW4StreamSupported(a)) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);
@@ -596,6 +606,30 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     e = LaunchConvInt8(a, stream, &op->last_kernel);
   }
   if (e != hipSuccess) return HipFail(e, "kernel launch");
+  return MLDHIP_OK;
+}
+
+int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
+  if (!ops || count < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "no ops");
+  if (count > 3) return Fail(MLDHIP_FAILED_PRECONDITION, "at most 3 ops per fused launch");
+  FcArgs args[3];
+  for (int i = 0; i < count; ++i) {
+    mldhip_op* op = ops[i];
+    if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
+    if (op->kind != mldhip_op::kFc || op->fc.src_type == MLDHIP_INT8)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "fused launch takes floating-point FullyConnected ops");
+    if (int rc = CheckBindings(op)) return rc;
+    if (int rc = BuildFcArgs(op, &args[i])) return rc;
+    const FcArgs &a = args[i], &f = args[0];
+    if (!FcW4StreamSupported(a))
+      return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " is not served by the streaming int4 kernel at this shape");
+    if (a.act != f.act || a.m != f.m || a.k != f.k || a.scale_kind != f.scale_kind || a.groups != f.groups)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " does not read the same tensor with the same K and scale groups as op 0");
+  }
+  const char* name = nullptr;
+  hipError_t e = LaunchFcW4StreamFused(args, count, static_cast<hipStream_t>(stream_ptr), &name);
+  if (e != hipSuccess) return HipFail(e, "fused launch");
+  for (int i = 0; i < count; ++i) ops[i]->last_kernel = name;
   return MLDHIP_OK;
 }
 

@@ -48,15 +48,25 @@ __device__ __forceinline__ uint32_t AndOr(uint32_t x, uint32_t mask, uint32_t ma
   return d;
 }
 
-struct StreamParams {
+// One weight matrix of a launch.  A launch covers up to kMaxSegments matrices that read the
+// same activations (same K): work-groups [strip_end of the previous, strip_end) belong to it.
+constexpr int kMaxSegments = 3;
+struct StreamSegment {
   const u32x4* weights;
-  const __half* act;
   const __half* scale;
   const __half* bias;
   __half* dst;
-  float* partial;
-  int m, ks, ns, n_pad;  // n_pad = ns * 4
-  int row_u4;            // uint4 per packed row = ns / 2
+  int ns, n_pad;  // n_pad = ns * 4
+  int row_u4;     // uint4 per packed row = ns / 2
+  int strip_end;
+};
+
+struct StreamParams {
+  StreamSegment seg[kMaxSegments];
+  int segments;
+  const __half* act;
+  float* partial;  // split-K sums (single-matrix launches only)
+  int m, ks;
   int chunks;            // ceil(ks / 8)
   int chunks_per_split;
   int ksplit;
@@ -74,14 +84,14 @@ __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const 
 }
 
 template <int M>
-__device__ __forceinline__ void LoadChunk(const StreamParams& p, int c, int pcol, u32x4 w[8],
-                                          u32x2 a[8][M]) {
+__device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* weights, int row_u4, int c, int pcol,
+                                          u32x4 w[8], u32x2 a[8][M]) {
   const int ks0 = c * 8;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int ks = ks0 + j;
     if (ks < p.ks) {
-      w[j] = __builtin_nontemporal_load(p.weights + (size_t)ks * p.row_u4 + pcol);
+      w[j] = __builtin_nontemporal_load(weights + (size_t)ks * row_u4 + pcol);
 #pragma unroll
       for (int m = 0; m < M; ++m)
         a[j][m] = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ks * M + m) * 4);
@@ -145,9 +155,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   const int wave = tid >> 6;
   const int col = lane % LPR;
   const int row = wave * RPW + lane / LPR;
-  const int pcol_raw = blockIdx.x * LPR + col;  // uint4 column = output channels 8*pcol .. +7
-  const bool col_ok = pcol_raw < p.row_u4;
-  const int pcol = col_ok ? pcol_raw : p.row_u4 - 1;  // clamp: loads stay in range, result unused
+  // which matrix of the launch this work-group belongs to, and which strip of it
+  int si = 0, strip = blockIdx.x;
+  if (p.segments > 1 && strip >= p.seg[0].strip_end) {
+    si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
+    strip -= p.seg[si - 1].strip_end;
+  }
+  const StreamSegment& sg = p.seg[si];
+  const u32x4* weights = sg.weights;
+  const int row_u4 = sg.row_u4;
+  const int pcol_raw = strip * LPR + col;  // uint4 column = output channels 8*pcol .. +7
+  const bool col_ok = pcol_raw < row_u4;
+  const int pcol = col_ok ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
   const int ky = blockIdx.y;
   const int c_begin = ky * p.chunks_per_split;
   const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
@@ -162,18 +181,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   if (c < c_end) {
     u32x4 w[8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, c, pcol, w, a);
+    LoadChunk<M>(p, weights, row_u4, c, pcol, w, a);
     while (true) {
       const int cn = c + ROWS;
       const bool more = cn < c_end;
       u32x4 wn[8];
       u32x2 an[8][M];
-      if (more) LoadChunk<M>(p, cn, pcol, wn, an);
+      if (more) LoadChunk<M>(p, weights, row_u4, cn, pcol, wn, an);
       u32x4 sv;
       if (GROUPED) {
         int g = c / p.group_chunks;
         if (g >= p.groups) g = p.groups - 1;
-        sv = *reinterpret_cast<const u32x4*>(p.scale + ((size_t)g * p.ns + 2 * pcol) * 4);
+        sv = *reinterpret_cast<const u32x4*>(sg.scale + ((size_t)g * sg.ns + 2 * pcol) * 4);
       }
       float t[M][8], asum[M];
 #pragma unroll
@@ -230,19 +249,19 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
     }
   }
   __syncthreads();
-  const int n0 = blockIdx.x * STRIP;
+  const int n0 = strip * STRIP;
   for (int idx = tid; idx < M * STRIP; idx += THREADS) {
     const int m = idx / STRIP, ol = idx % STRIP;
     const int n = n0 + ol;
-    if (n >= p.n_pad) continue;
+    if (n >= sg.n_pad) continue;
     float v = 0.0f;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
     if (p.ksplit == 1) {
-      if (!GROUPED) v *= __half2float(p.scale[n]);
-      StoreHalf(p.dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, p.bias, (size_t)n);
+      if (!GROUPED) v *= __half2float(sg.scale[n]);
+      StoreHalf(sg.dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, sg.bias, (size_t)n);
     } else {
-      p.partial[((size_t)ky * M + m) * p.n_pad + n] = v;
+      p.partial[((size_t)ky * M + m) * sg.n_pad + n] = v;
     }
   }
 }
@@ -250,13 +269,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
 // Adds the split-K partial sums in split order and writes the output.
 template <bool GROUPED>
 __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
+  const StreamSegment& sg = p.seg[0];
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= p.m * p.n_pad) return;
-  const int m = idx / p.n_pad, n = idx % p.n_pad;
+  if (idx >= p.m * sg.n_pad) return;
+  const int m = idx / sg.n_pad, n = idx % sg.n_pad;
   float v = 0.0f;
-  for (int s = 0; s < p.ksplit; ++s) v += p.partial[((size_t)s * p.m + m) * p.n_pad + n];
-  if (!GROUPED) v *= __half2float(p.scale[n]);
-  StoreHalf(p.dst, ((size_t)(n >> 2) * p.m + m) * 4 + (n & 3), v, p.bias, (size_t)n);
+  for (int s = 0; s < p.ksplit; ++s) v += p.partial[((size_t)s * p.m + m) * sg.n_pad + n];
+  if (!GROUPED) v *= __half2float(sg.scale[n]);
+  StoreHalf(sg.dst, ((size_t)(n >> 2) * p.m + m) * 4 + (n & 3), v, sg.bias, (size_t)n);
 }
 
 template <int LPR, int WAVES, int M>
@@ -309,19 +329,15 @@ bool FcW4StreamSupported(const FcArgs& a) {
   return a.partial != nullptr;
 }
 
-hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name) {
+  if (count < 1 || count > kMaxSegments) return hipErrorInvalidValue;
+  const FcArgs& a = args[0];
   StreamParams p;
-  p.weights = reinterpret_cast<const u32x4*>(a.weights);
+  p.segments = count;
   p.act = static_cast<const __half*>(a.act);
-  p.scale = static_cast<const __half*>(a.scale);
-  p.bias = static_cast<const __half*>(a.bias);
-  p.dst = static_cast<__half*>(a.dst);
   p.partial = a.partial;
   p.m = a.m;
   p.ks = DivUp(a.k, 4);
-  p.ns = DivUp(a.n, 4);
-  p.n_pad = p.ns * 4;
-  p.row_u4 = p.ns / 2;
   p.chunks = DivUp(p.ks, 8);
   const bool grouped = a.scale_kind == kScaleBlock;
   p.groups = grouped ? a.groups : 1;
@@ -330,22 +346,40 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   p.mask_hi = 0x00F000F0u;
   p.magic_lo = 0x64006400u;
   p.magic_hi = 0x54005400u;
+  int total_row_u4 = 0;
+  size_t weight_bytes = 0;
+  for (int i = 0; i < count; ++i) {
+    StreamSegment& sg = p.seg[i];
+    sg.weights = reinterpret_cast<const u32x4*>(args[i].weights);
+    sg.scale = static_cast<const __half*>(args[i].scale);
+    sg.bias = static_cast<const __half*>(args[i].bias);
+    sg.dst = static_cast<__half*>(args[i].dst);
+    sg.ns = DivUp(args[i].n, 4);
+    sg.n_pad = sg.ns * 4;
+    sg.row_u4 = sg.ns / 2;
+    total_row_u4 += sg.row_u4;
+    weight_bytes += (size_t)p.ks * sg.ns * 8;
+  }
+  for (int i = count; i < kMaxSegments; ++i) p.seg[i] = p.seg[0];
 
   // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the
   // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous
   // bytes) keep K inside one work-group for wide layers; when the layer is too narrow for
   // that, K is split across work-groups and a second kernel adds the partials.
-  // Narrow layers take narrower strips (LPR = 4 or 2: 64- or 32-byte segments) before K is split:
-  // a second kernel costs more than the poorer coalescing of a matrix of a few MB.
+  // Narrow layers of a few MB take narrower strips first (LPR = 4 or 2: 64- or 32-byte
+  // segments): there a second kernel costs more than the poorer coalescing.
   int lpr = 8, waves = 16;
-  const size_t weight_bytes = (size_t)p.ks * p.ns * 8;
-  if (DivUp(p.row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
-    lpr = DivUp(p.row_u4, 4) >= 128 ? 4 : 2;
+  if (DivUp(total_row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
+    lpr = DivUp(total_row_u4, 4) >= 128 ? 4 : 2;
   lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
   if (lpr != 2 && lpr != 4 && lpr != 8 && lpr != 16) lpr = 8;
   waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
-  const int strips = DivUp(p.row_u4, lpr);
+  int strips = 0;
+  for (int i = 0; i < count; ++i) {
+    strips += DivUp(p.seg[i].row_u4, lpr);
+    p.seg[i].strip_end = strips;
+  }
   int rows = waves * 64 / lpr;
   // shrink the work-group while it would leave rows without a chunk
   while (waves > 4 && rows / 2 >= p.chunks) {
@@ -353,15 +387,15 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
     rows /= 2;
   }
   int ksplit = 1;
-  if (strips < 128) {
+  if (strips < 128 && count == 1) {
     ksplit = DivUp(256, strips);
     const int max_split = DivUp(p.chunks, rows);
     if (ksplit > max_split) ksplit = max_split;
   }
-  ksplit = EnvInt("MLDHIP_GEMV_KSPLIT", ksplit);
+  if (count == 1) ksplit = EnvInt("MLDHIP_GEMV_KSPLIT", ksplit);
   if (ksplit > kGemvMaxKSplit) ksplit = kGemvMaxKSplit;
   if (ksplit < 1) ksplit = 1;
-  while (ksplit > 1 && (size_t)ksplit * p.m * p.n_pad > a.partial_floats) --ksplit;
+  while (ksplit > 1 && (size_t)ksplit * p.m * p.seg[0].n_pad > a.partial_floats) --ksplit;
   // every thread row gets the same number of chunks
   p.chunks_per_split = DivUp(DivUp(p.chunks, ksplit), rows) * rows;
   p.ksplit = DivUp(p.chunks, p.chunks_per_split);
@@ -377,12 +411,16 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   else
     e = LaunchCfgW<16>(p, waves, grouped, grid, stream);
   if (e != hipSuccess || p.ksplit == 1) return e;
-  const int total = p.m * p.n_pad;
+  const int total = p.m * p.seg[0].n_pad;
   if (grouped)
     hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
   else
     hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
   return hipGetLastError();
+}
+
+hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+  return LaunchFcW4StreamFused(&a, 1, stream, kernel_name);
 }
 
 }  // namespace mldhip

@@ -129,6 +129,7 @@ class HipOperation {
   Status AddToQueue(void* hip_stream) { return Status::FromCode(mldhip_op_launch(op_.get(), hip_stream)); }
   const char* kernel_name() const { return mldhip_op_kernel_name(op_.get()); }
   bool valid() const { return op_ != nullptr; }
+  mldhip_op* handle() const { return op_.get(); }
 
  private:
   std::unique_ptr<mldhip_op, void (*)(mldhip_op*)> op_{nullptr, &mldhip_op_destroy};
@@ -186,6 +187,14 @@ inline Status CreateConvInt8WithDequantization(DataType dst_type, const OHWI& we
   if (rc != MLDHIP_OK) return Status::FromCode(rc);
   *result = HipOperation(op);
   return {};
+}
+
+// One launch for FullyConnected nodes that read the same tensor (q/k/v, gate/up); the caller
+// falls back to AddToQueue per node when the status is FAILED_PRECONDITION.
+inline Status AddToQueueFused(const std::vector<HipOperation*>& ops, void* hip_stream) {
+  std::vector<mldhip_op*> handles;
+  for (HipOperation* op : ops) handles.push_back(op->handle());
+  return Status::FromCode(mldhip_fc_launch_fused(handles.data(), (int)handles.size(), hip_stream));
 }
 
 // One graph node: operation + the ids of its inputs/outputs in the caller's tensor table,

@@ -82,10 +82,33 @@ class DecoderStack:
             op.set_shape(1, 1, tokens)
             self.outs.append(view)
 
-    def launch(self, stream=None):
+    def launch(self, stream=None, fused=True):
+        """One pass over the stack in node order.  With `fused`, the FCs of a layer that read the
+        same tensor (q/k/v; gate/up) go out as one launch where the library can serve them
+        together (decode), singly otherwise."""
         s = self.torch.cuda.current_stream().cuda_stream if stream is None else stream
-        for _, _, op, _, _, _ in self.nodes:
-            op.launch(s)
+        if not fused:
+            for _, _, op, _, _, _ in self.nodes:
+                op.launch(s)
+            return
+        names = [c["name"] for c in self.cases]
+        per_layer = len(self.cases)
+        groups = [[names.index(n) for n in grp] for grp in self.PARALLEL if all(n in names for n in grp)]
+        for layer in range(self.layers):
+            idx = 0
+            while idx < per_layer:
+                grp = next((g for g in groups if g[0] == idx and g == list(range(idx, idx + len(g)))), None)
+                if grp is not None:
+                    ops = [self.nodes[layer * per_layer + i][2] for i in grp]
+                    try:
+                        M.fc_launch_fused(ops, s)
+                        idx += len(grp)
+                        continue
+                    except M.MldhipError as e:
+                        if e.code != M.FAILED_PRECONDITION:
+                            raise
+                self.nodes[layer * per_layer + idx][2].launch(s)
+                idx += 1
 
     # FCs of a layer that read the same tensor and do not depend on each other
     PARALLEL = (("q", "k", "v"), ("gate", "up"))
@@ -98,7 +121,7 @@ class DecoderStack:
         (On MI355X the fork/join of the branches costs more than the overlap gains: 1093 us
         against 873 us for a decode step, hence the default.)"""
         torch = self.torch
-        self.launch()  # workspaces are allocated on the first launch, outside the capture
+        self.launch(fused=False)  # workspaces are allocated on the first launch, outside the capture
         torch.cuda.synchronize()
         main = torch.cuda.Stream()
         side = [torch.cuda.Stream(), torch.cuda.Stream()]

@@ -28,7 +28,7 @@ SYMBOLS = [
     "mldhip_quantization_create", "mldhip_conv_int8_src_type", "mldhip_conv_int8_create",
     "mldhip_op_src_count", "mldhip_op_dst_count", "mldhip_op_src_name", "mldhip_op_dst_name",
     "mldhip_op_set_src", "mldhip_op_set_dst", "mldhip_op_set_shape", "mldhip_op_launch",
-    "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy",
+    "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
 ]
 
 
@@ -280,6 +280,13 @@ class Op:
         b, f = C.c_uint64(), C.c_uint64()
         check(lib().mldhip_op_cost(self.handle, C.byref(b), C.byref(f)))
         return b.value, f.value
+
+
+def fc_launch_fused(ops, stream=0):
+    """One launch for FC ops that read the same source tensor; raises MldhipError with
+    FAILED_PRECONDITION when they cannot share a launch."""
+    arr = (C.c_void_p * len(ops))(*[op.handle for op in ops])
+    check(lib().mldhip_fc_launch_fused(arr, len(ops), C.c_void_p(stream)))
 
 
 def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1, 1),

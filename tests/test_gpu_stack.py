@@ -42,3 +42,29 @@ def test_stack_accounting(stack):
     per_layer = sum(c["k"] * c["n"] // 2 + (c["k"] // 32) * c["n"] * 2 for c in stack.cases)
     assert stack.weight_bytes() == LAYERS * per_layer
     assert per_layer == 61931520  # one layer of config 5
+
+
+def test_fused_launch_matches_single_launches(stack):
+    """q/k/v and gate/up as one launch each give the bytes of the one-by-one launches."""
+    import mldhip as M
+    stack.set_tokens(1)
+    stack.launch(fused=False)
+    single = [stack.result(layer, idx) for layer in range(LAYERS) for idx in range(len(stack.cases))]
+    for out in stack.outs:
+        out.zero_()
+    stack.launch(fused=True)
+    fused = [stack.result(layer, idx) for layer in range(LAYERS) for idx in range(len(stack.cases))]
+    for a, b in zip(single, fused):
+        assert np.array_equal(a, b)
+    # ops over different inputs (o reads width 2048, down reads 16384) cannot share a launch
+    names = [c["name"] for c in stack.cases]
+    o_op = stack.nodes[names.index("o")][2]
+    down_op = stack.nodes[names.index("down")][2]
+    with pytest.raises(M.MldhipError) as err:
+        M.fc_launch_fused([o_op, down_op])
+    assert err.value.code == M.FAILED_PRECONDITION
+    # at 128 tokens the MFMA kernel serves the ops: no fused launch, the stack falls back
+    stack.set_tokens(128)
+    with pytest.raises(M.MldhipError) as err:
+        M.fc_launch_fused([stack.nodes[names.index("gate")][2], stack.nodes[names.index("up")][2]])
+    assert err.value.code == M.FAILED_PRECONDITION
