@@ -368,9 +368,12 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   // that, K is split across work-groups and a second kernel adds the partials.
   // Narrow layers of a few MB take narrower strips first (LPR = 4 or 2: 64- or 32-byte
   // segments): there a second kernel costs more than the poorer coalescing.
+  // Very wide launches (the fused gate / up pair) fill the chip with 256-byte segments (LPR = 16).
   int lpr = 8, waves = 16;
-  if (DivUp(total_row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
-    lpr = DivUp(total_row_u4, 4) >= 128 ? 4 : 2;
+  if (DivUp(total_row_u4, 16) >= 256)
+    lpr = 16;
+  else if (DivUp(total_row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
+    lpr = DivUp(total_row_u4, 4) >= 64 ? 4 : 2;
   lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
   if (lpr != 2 && lpr != 4 && lpr != 8 && lpr != 16) lpr = 8;
   waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
