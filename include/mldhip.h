@@ -176,6 +176,10 @@ int mldhip_fc_is_recommended(int precision, int tokens);
  *   4 "biases"                present iff has_bias, ceil(o/4)*4 values of dst_type
  * (absent objects do not take an index).  dst 0 "dst_tensor": [ceil(o/4)][tokens][4].
  *
+ * Zero points (fully_connected_util.cc:91-99: w = u*s - s*(shift + zp)) are taken by every
+ * kernel; the int4 fast kernels assume integral zero-point values (the builder converts them from
+ * int32, common/gpu_model_builder.cc:1917-1935).
+ *
  * src_type INT8 selects the integer-math variant (fully_connected.cc:543-621, 874-903):
  * no scales, dst_type must be INT32. */
 typedef struct {

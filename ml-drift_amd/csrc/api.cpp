@@ -623,7 +623,8 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
     const FcArgs &a = args[i], &f = args[0];
     if (!FcW4StreamSupported(a))
       return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " is not served by the streaming int4 kernel at this shape");
-    if (a.act != f.act || a.m != f.m || a.k != f.k || a.scale_kind != f.scale_kind || a.groups != f.groups)
+    if (a.act != f.act || a.m != f.m || a.k != f.k || a.scale_kind != f.scale_kind || a.groups != f.groups ||
+        a.has_zero_point != f.has_zero_point)
       return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " does not read the same tensor with the same K and scale groups as op 0");
   }
   const char* name = nullptr;

@@ -45,6 +45,7 @@ struct GemmParams {
   const uint8_t* w4;    // [Ks][Ns] blocks of 8 bytes
   const __half* act;    // [Ks][m][4]
   const __half* scale;  // [groups][Ns][4]
+  const __half* zp;     // zero points, same shape as scale, or null
   int ks;               // input slices, ceil(k/4)
   int steps_per_group;  // K-steps per scale group
   int groups;
@@ -474,7 +475,9 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
 // it stay in flight.
 __device__ __forceinline__ void LdsBarrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int FM, int U, int WAVES>
+// ZP: the weights have a zero-point tensor (same shape as the scales); the centre of the codes
+// moves from 8 to 8 + zp (exact in fp16 for integral zero points).
+template <int FM, int U, int WAVES, bool ZP>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
@@ -520,6 +523,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, x_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_s =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_z =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(ZP ? p.zp : p.scale), 0, p.s_bytes, 0x00020000);
 
   // Per-lane byte offsets of the next step to fetch; each fetch advances them by one step.
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
@@ -537,8 +542,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   }
   const uint32_t group_bytes = row_w;  // one scale group: [Ns][4] halfs
 
-  u32x2 rw[U][2], rsc[U], rx[U][FM][2];
-  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2 (&x)[FM][2]) {
+  u32x2 rw[U][2], rsc[U], rzp[U], rx[U][FM][2];
+  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[FM][2]) {
     w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
     w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw1, 0, 0);
     vw0 += step_w;
@@ -546,6 +551,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     // scale group of this step (groups hold a power-of-two number of steps); a group past the
     // last one reads zeros
     sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
+    if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
       x[fm][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[fm][0], 0, 0);
@@ -569,7 +575,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    load_step(t_begin + u, rw[u], rsc[u], rx[u]);
+    load_step(t_begin + u, rw[u], rsc[u], rzp[u], rx[u]);
     __builtin_amdgcn_sched_barrier(0);
   }
   for (int tt = 0; tt < per_wave; tt += U) {
@@ -580,16 +586,26 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       const u32x4 blk = {rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
       const u32x4 blk8 = {blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
       const half2_t sc01 = AsHalf2(rsc[u][0]), sc23 = AsHalf2(rsc[u][1]);
+      half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
+      if (ZP) {
+        zp01 = AsHalf2(rzp[u][0]);
+        zp23 = AsHalf2(rzp[u][1]);
+      }
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) {
         const half2_t sp = (t4 & 2) ? sc23 : sc01;
         const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
+        half2_t off = (t4 & 1) ? off_hi : off_lo;
+        if (ZP) {
+          const half2_t zq = (t4 & 2) ? zp23 : zp01;
+          off -= (t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0);
+        }
         u32x4 aop;
 #pragma unroll
         for (int wd = 0; wd < 4; ++wd) {
           const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
           const uint32_t bits = (t4 & 1) ? AndOr(x, p.mask_hi, p.magic_hi) : AndOr(x, p.mask_lo, p.magic_lo);
-          aop[wd] = AsU32((AsHalf2(bits) + ((t4 & 1) ? off_hi : off_lo)) * s2);
+          aop[wd] = AsU32((AsHalf2(bits) + off) * s2);
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -601,7 +617,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       // refill stage u with step t + U; the fences keep the loads of a stage together and in
       // program order, so that waiting for one stage leaves the younger ones in flight
       __builtin_amdgcn_sched_barrier(0);
-      load_step(t + U, rw[u], rsc[u], rx[u]);
+      load_step(t + U, rw[u], rsc[u], rzp[u], rx[u]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -652,6 +668,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       if (fm + 1 < FM || ph + 1 < 16 / WAVES) LdsBarrier();
     }
   }
+}
+
+template <int FM, int U, int WAVES>
+void LaunchDirect(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
+  if (zp)
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  else
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, p);
 }
 
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
@@ -719,7 +743,8 @@ hipError_t LaunchConvInt8Tile(const GemmParams& p, hipStream_t stream) {
 
 bool FcW4MfmaSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
-  if (a.has_zero_point || a.scale_kind == kScaleScalar) return false;
+  if (a.scale_kind == kScaleScalar) return false;
+  if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   if (a.m <= kGemvMaxTokens) return false;
   // 32-bit buffer offsets
   if ((size_t)DivUp(a.k, 4) * DivUp(a.n, 4) * 8 >= 0x7FFFFFF0u || (size_t)DivUp(a.k, 4) * a.m * 8 >= 0x7FFFFFF0u)
@@ -747,6 +772,7 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   p.w4 = a.weights;
   p.act = static_cast<const __half*>(a.act);
   p.scale = static_cast<const __half*>(a.scale);
+  p.zp = a.has_zero_point ? static_cast<const __half*>(a.zero_point) : nullptr;
   p.groups = a.scale_kind == kScaleBlock ? a.groups : 1;
   p.steps_per_group = a.scale_kind == kScaleBlock ? (a.k / a.groups) / 32 : p.k_steps;
   p.mask_lo = 0x000F000Fu;
@@ -785,19 +811,17 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   const dim3 grid(DivUp(tiles, 8) * 8, p.ksplit);
   int waves = 8;
   if (const char* e = std::getenv("MLDHIP_GEMM_WAVES")) waves = std::atoi(e);
-  if (fm == 2) {
-    if (waves == 8)
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4, 8>), grid, dim3(512), 0, stream, p);
-    else if (u == 8)
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 8, 4>), grid, dim3(256), 0, stream, p);
-    else
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<2, 4, 4>), grid, dim3(256), 0, stream, p);
-  } else {
-    if (waves == 8)
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4, 8>), grid, dim3(512), 0, stream, p);
-    else
-      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<1, 4, 4>), grid, dim3(256), 0, stream, p);
-  }
+  const bool zp = p.zp != nullptr;
+  if (fm == 2 && waves == 8)
+    LaunchDirect<2, 4, 8>(zp, grid, stream, p);
+  else if (fm == 2 && u == 8)
+    LaunchDirect<2, 8, 4>(zp, grid, stream, p);
+  else if (fm == 2)
+    LaunchDirect<2, 4, 4>(zp, grid, stream, p);
+  else if (waves == 8)
+    LaunchDirect<1, 4, 8>(zp, grid, stream, p);
+  else
+    LaunchDirect<1, 4, 4>(zp, grid, stream, p);
   if (p.ksplit > 1)
     hipLaunchKernelGGL(fc_w4_splitk_reduce_kernel, dim3(DivUp(p.ns * a.m, 256)), dim3(256), 0, stream, p);
   return hipGetLastError();

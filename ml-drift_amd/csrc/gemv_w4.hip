@@ -54,6 +54,7 @@ constexpr int kMaxSegments = 3;
 struct StreamSegment {
   const u32x4* weights;
   const __half* scale;
+  const __half* zero_point;  // same shape as scale, or null
   const __half* bias;
   __half* dst;
   int ns, n_pad;  // n_pad = ns * 4
@@ -141,7 +142,9 @@ __device__ __forceinline__ void ComputeChunk(const StreamParams& p, const u32x4 
   }
 }
 
-template <int LPR, int WAVES, int M, bool GROUPED>
+// ZP: the weights have a zero-point tensor (same shape as the scales): the centre of the codes
+// moves from 8 to 8 + zp, per channel or per (group, channel).
+template <int LPR, int WAVES, int M, bool GROUPED, bool ZP>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p) {
   constexpr int THREADS = WAVES * 64;
   constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
@@ -178,6 +181,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
     for (int o = 0; o < 8; ++o) acc[m][o] = 0.0f;
 
   int c = c_begin + row;
+  u32x4 zv = {0u, 0u, 0u, 0u};  // zero points of this thread's 8 channels (halfs)
+  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(sg.zero_point + (size_t)2 * pcol * 4);
   if (c < c_end) {
     u32x4 w[8];
     u32x2 a[8][M];
@@ -193,6 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
         int g = c / p.group_chunks;
         if (g >= p.groups) g = p.groups - 1;
         sv = *reinterpret_cast<const u32x4*>(sg.scale + ((size_t)g * sg.ns + 2 * pcol) * 4);
+        if (ZP) zv = *reinterpret_cast<const u32x4*>(sg.zero_point + ((size_t)g * sg.ns + 2 * pcol) * 4);
       }
       float t[M][8], asum[M];
 #pragma unroll
@@ -206,7 +212,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
       for (int m = 0; m < M; ++m)
 #pragma unroll
         for (int o = 0; o < 8; ++o) {
-          const float centered = fmaf((o & 1) ? -72.0f : -1032.0f, asum[m], t[m][o]);
+          float centre = (o & 1) ? -72.0f : -1032.0f;
+          if (ZP) centre -= (float)AsHalf2(zv[o >> 1])[o & 1];
+          const float centered = fmaf(centre, asum[m], t[m][o]);
           if (GROUPED) {
             const half2_t sp = AsHalf2(sv[o >> 1]);
             acc[m][o] = fmaf((float)sp[o & 1], centered, acc[m][o]);
@@ -281,10 +289,15 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
 
 template <int LPR, int WAVES, int M>
 hipError_t LaunchCfg(const StreamParams& p, bool grouped, dim3 grid, hipStream_t stream) {
-  if (grouped)
-    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  const bool zp = p.seg[0].zero_point != nullptr;
+  if (grouped && zp)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  else if (grouped)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true, false>), grid, dim3(WAVES * 64), 0, stream, p);
+  else if (zp)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false, true>), grid, dim3(WAVES * 64), 0, stream, p);
   else
-    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false>), grid, dim3(WAVES * 64), 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false, false>), grid, dim3(WAVES * 64), 0, stream, p);
   return hipGetLastError();
 }
 
@@ -318,7 +331,7 @@ int EnvInt(const char* name, int fallback) {
 bool FcW4StreamSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
   if (a.m < 1 || a.m > kGemvMaxTokens) return false;
-  if (a.has_zero_point) return false;
+  if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   const int ks = DivUp(a.k, 4), ns = DivUp(a.n, 4);
   if (ns % 2 != 0) return false;  // 16-byte loads need an even number of 8-byte blocks per row
   if (a.scale_kind == kScaleScalar) return false;
@@ -352,6 +365,7 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     StreamSegment& sg = p.seg[i];
     sg.weights = reinterpret_cast<const u32x4*>(args[i].weights);
     sg.scale = static_cast<const __half*>(args[i].scale);
+    sg.zero_point = args[i].has_zero_point ? static_cast<const __half*>(args[i].zero_point) : nullptr;
     sg.bias = static_cast<const __half*>(args[i].bias);
     sg.dst = static_cast<__half*>(args[i].dst);
     sg.ns = DivUp(args[i].n, 4);

@@ -134,6 +134,15 @@ def test_stream_kernel_tokens_and_groups(oracle, m, groups):
     run_case(oracle, case, "fc_w4_stream_kernel")
 
 
+@pytest.mark.parametrize("m", [1, 3, 4])
+@pytest.mark.parametrize("groups", [1, 64])
+def test_stream_kernel_zero_points(oracle, m, groups):
+    """Asymmetric int4 weights (a zero-point tensor shaped like the scales) on the streaming kernel."""
+    case = W.make_fc_case(seed=23 + m, m=m, k=2048, n=1032, weight_bits=4, tensor_dtype=np.float16,
+                          groups=groups, with_bias=True, with_zero_point=True)
+    run_case(oracle, case, "fc_w4_stream_kernel")
+
+
 @pytest.mark.parametrize("name,k,n", W.C5_LAYER)
 def test_config5_decode_layer_shapes(oracle, name, k, n):
     case = W.make_fc_case(seed=7, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=k // 32)

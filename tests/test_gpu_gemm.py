@@ -40,6 +40,17 @@ def test_w4_gemm_shapes(oracle, m, k, n, groups):
         check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
 
 
+@pytest.mark.parametrize("m,k,n,groups", [(16, 256, 128, 8), (77, 1024, 200, 1), (128, 2048, 2048, 64)])
+def test_w4_gemm_zero_points(oracle, m, k, n, groups):
+    """Asymmetric int4 weights (a zero-point tensor shaped like the scales) on the MFMA kernel."""
+    case = W.make_fc_case(seed=m + 3 * n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True, with_zero_point=True)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    if m * k * n <= 1 << 26:
+        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+
+
 def test_config3_prefill_gemm(oracle):
     case = W.make_fc_case(**W.CONFIGS["c3"])
     got = run_w4(case)
