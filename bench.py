@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Benchmark of the int4 decode GEMV (BASELINE.json config 2) on one MI355X.
+"""Benchmark of the int4 decode GEMV (benchmark configuration 2) on one MI355X.
 
 Workload: FullyConnected, 1 token, K=4096, N=14336, int4 per-channel weights in the packed
 I4O4 layout, fp16 activations / scales / output, fp32 accumulation.  One step = one launch

@@ -133,7 +133,7 @@ def dequantized_weights(case):
     return q * s
 
 
-# BASELINE.json configurations 1-4 as make_fc_case arguments.
+# The benchmark configurations 1-4 as make_fc_case arguments.
 CONFIGS = {
     "c1": dict(seed=0, m=1, k=2048, n=2048, weight_bits=8, tensor_dtype=np.float32, groups=1),
     "c2": dict(seed=0, m=1, k=4096, n=14336, weight_bits=4, tensor_dtype=np.float16, groups=1),
