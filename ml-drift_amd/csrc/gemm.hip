@@ -18,6 +18,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "../../include/mldhip.h"
 #include "kernels.h"
@@ -95,6 +96,12 @@ __device__ __forceinline__ float Rescale(int acc, float ws, int wsum, float src_
     res = res + g3;
   }
   return res;
+}
+// The same with a zero activation offset and no weight zero point: the offset terms are exact
+// zeros there, and adding a zero changes nothing (but possibly the sign of a zero result).
+__device__ __forceinline__ float RescaleNoOffset(int acc, float ws, float src_scale) {
+  const float f0 = ws * src_scale;
+  return (float)acc * f0;
 }
 #pragma clang fp contract(fast)
 
@@ -337,20 +344,49 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
     // [slice of the tile][token of the tile][4 halfs]; what lies outside the matrix is computed
     // from clamped constants and never leaves LDS.
     const bool has_bias = p.bias != nullptr;
+    // the channel constants of the wave's 16 slices, all requested before any is used (one memory
+    // latency instead of sixteen); the per-channel tensors are padded to whole slices
+    float4 ws_all[FN * 4];
+    int4v_t wsum_all[FN * 4];
+    float4 wzp_all[ZP ? FN * 4 : 1];
+    u32x2 bias_all[FN * 4];
+#pragma unroll
+    for (int g = 0; g < FN * 4; ++g) {
+      const int slice_l = (wn * FN + g / 4) * 8 + (g % 4) * 2 + g2;
+      const int nb = min(n0 / 4 + slice_l, p.ns - 1) * 4;  // first of 4 consecutive channels
+      ws_all[g] = *reinterpret_cast<const float4*>(p.wscale + nb);
+      wsum_all[g] = *reinterpret_cast<const int4v_t*>(p.wsum + nb);
+      if (ZP) wzp_all[g] = *reinterpret_cast<const float4*>(p.wzp + nb);
+      bias_all[g] = u32x2{0x80008000u, 0x80008000u};  // -0.0: adding it changes nothing, not even the sign of a zero
+    }
+    if (has_bias) {
+#pragma unroll
+      for (int g = 0; g < FN * 4; ++g) {
+        const int slice_l = (wn * FN + g / 4) * 8 + (g % 4) * 2 + g2;
+        const int nb = min(n0 / 4 + slice_l, p.ns - 1) * 4;
+        bias_all[g] = *reinterpret_cast<const u32x2*>(static_cast<const __half*>(p.bias) + nb);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // symmetric activation quantization gives a zero offset for every token: then two of the
+    // three products and the sum of the rescale drop out (decided per wave)
+    bool all_zero_offset = !has_zp;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) all_zero_offset = all_zero_offset && src_zp[fm] == 0.0f;
+    const bool no_offset = __all(all_zero_offset);
+    auto stage_tile = [&](auto no_offset_tag) {
+    constexpr bool kNoOffset = decltype(no_offset_tag)::value;
 #pragma unroll
     for (int fn = 0; fn < FN; ++fn) {
 #pragma unroll
       for (int v4 = 0; v4 < 4; ++v4) {
         const int slice_l = (wn * FN + fn) * 8 + v4 * 2 + g2;
-        const int nb = min(n0 / 4 + slice_l, p.ns - 1) * 4;  // first of 4 consecutive channels
-        // the per-channel tensors are padded to whole slices
-        const float4 ws = *reinterpret_cast<const float4*>(p.wscale + nb);
-        const int4v_t wsum = *reinterpret_cast<const int4v_t*>(p.wsum + nb);
-        const float4 wzp = has_zp ? *reinterpret_cast<const float4*>(p.wzp + nb) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        const float4 ws = ws_all[fn * 4 + v4];
+        const int4v_t wsum = wsum_all[fn * 4 + v4];
+        const float4 wzp = ZP ? wzp_all[ZP ? fn * 4 + v4 : 0] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         const float wsc[4] = {ws.x, ws.y, ws.z, ws.w};
         const float wz[4] = {wzp.x, wzp.y, wzp.z, wzp.w};
-        u32x2 bias2 = {0x80008000u, 0x80008000u};  // -0.0: adding it changes nothing, not even the sign of a zero
-        if (has_bias) bias2 = *reinterpret_cast<const u32x2*>(static_cast<const __half*>(p.bias) + nb);
+        const u32x2 bias2 = bias_all[fn * 4 + v4];
         const __half bias_h[4] = {__ushort_as_half((unsigned short)(bias2[0] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[0] >> 16)),
                                   __ushort_as_half((unsigned short)(bias2[1] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[1] >> 16))};
 #pragma unroll
@@ -358,8 +394,9 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
           __half h[4];
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            const float r = Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp, wz[c],
-                                    src_sum[fm], in_channels);
+            const float r = kNoOffset ? RescaleNoOffset(acc[fn][fm][v4 * 4 + c], wsc[c], src_scale[fm])
+                                      : Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp,
+                                                wz[c], src_sum[fm], in_channels);
             h[c] = __float2half_rn(r);
             h[c] = __hadd(h[c], bias_h[c]);
           }
@@ -371,6 +408,11 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
         }
       }
     }
+    };
+    if (no_offset)
+      stage_tile(std::true_type{});
+    else
+      stage_tile(std::false_type{});
   } else {
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
