@@ -519,8 +519,11 @@ __device__ __forceinline__ void LdsBarrier() { asm volatile("s_waitcnt lgkmcnt(0
 
 // ZP: the weights have a zero-point tensor (same shape as the scales); the centre of the codes
 // moves from 8 to 8 + zp (exact in fp16 for integral zero points).
-template <int FM, int U, int WAVES, bool ZP>
+// PAIR (FM even, token count even): a lane's tokens for the MFMA pair (fm, fm+1) are neighbours
+// (2j, 2j+1 instead of j, j+32), so one 16-byte load brings both activation operands.
+template <int FM, int U, int WAVES, bool ZP, bool PAIR>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
+  static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
   static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "the reduction handles WAVES registers per phase");
@@ -575,17 +578,21 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * 8u : kOob;
   uint32_t vw1 = n_ok ? vw0 + row_w : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
-  uint32_t vx[FM][2];
+  // token of this lane in MFMA token block fm
+  auto token = [&](int fm) { return PAIR ? m0 + (fm / 2) * 64 + 2 * i32 + (fm & 1) : m0 + fm * 32 + i32; };
+  constexpr int NX = PAIR ? FM / 2 : FM;  // activation load items per K-slice row
+  uint32_t vx[NX][2];
 #pragma unroll
-  for (int fm = 0; fm < FM; ++fm) {
-    const int mi = m0 + fm * 32 + i32;
-    vx[fm][0] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
-    vx[fm][1] = mi < p.m ? vx[fm][0] + row_x : kOob;
+  for (int i = 0; i < NX; ++i) {
+    const int mi = token(PAIR ? 2 * i : i);
+    vx[i][0] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
+    vx[i][1] = mi < p.m ? vx[i][0] + row_x : kOob;
   }
   const uint32_t group_bytes = row_w;  // one scale group: [Ns][4] halfs
 
-  u32x2 rw[U][2], rsc[U], rzp[U], rx[U][FM][2];
-  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[FM][2]) {
+  u32x2 rw[U][2], rsc[U], rzp[U], rx[U][NX][2];
+  u32x4 rxp[U][NX][2];  // PAIR: {token 2j: 4 halfs, token 2j+1: 4 halfs} per K-slice row
+  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[NX][2], u32x4 (&xp)[NX][2]) {
     w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
     w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw1, 0, 0);
     vw0 += step_w;
@@ -595,11 +602,16 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
     if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm) {
-      x[fm][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[fm][0], 0, 0);
-      x[fm][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[fm][1], 0, 0);
-      vx[fm][0] += step_x;
-      vx[fm][1] += step_x;
+    for (int i = 0; i < NX; ++i) {
+      if (PAIR) {
+        xp[i][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, vx[i][0], 0, 0);
+        xp[i][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, vx[i][1], 0, 0);
+      } else {
+        x[i][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[i][0], 0, 0);
+        x[i][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[i][1], 0, 0);
+      }
+      vx[i][0] += step_x;
+      vx[i][1] += step_x;
     }
   };
 
@@ -617,7 +629,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    load_step(t_begin + u, rw[u], rsc[u], rzp[u], rx[u]);
+    load_step(t_begin + u, rw[u], rsc[u], rzp[u], rx[u], rxp[u]);
     __builtin_amdgcn_sched_barrier(0);
   }
   for (int tt = 0; tt < per_wave; tt += U) {
@@ -651,7 +663,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
-          const u32x4 bop = {rx[u][fm][0][0], rx[u][fm][0][1], rx[u][fm][1][0], rx[u][fm][1][1]};
+          const int h2 = 2 * (fm & 1);
+          const u32x4 bop = PAIR ? u32x4{rxp[u][fm / 2][0][h2], rxp[u][fm / 2][0][h2 + 1], rxp[u][fm / 2][1][h2],
+                                         rxp[u][fm / 2][1][h2 + 1]}
+                                 : u32x4{rx[u][PAIR ? 0 : fm][0][0], rx[u][PAIR ? 0 : fm][0][1], rx[u][PAIR ? 0 : fm][1][0],
+                                         rx[u][PAIR ? 0 : fm][1][1]};
           acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
                                                                __builtin_bit_cast(half8_t, bop), acc[t4][fm], 0, 0, 0);
         }
@@ -659,7 +675,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       // refill stage u with step t + U; the fences keep the loads of a stage together and in
       // program order, so that waiting for one stage leaves the younger ones in flight
       __builtin_amdgcn_sched_barrier(0);
-      load_step(t + U, rw[u], rsc[u], rzp[u], rx[u]);
+      load_step(t + U, rw[u], rsc[u], rzp[u], rx[u], rxp[u]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -673,7 +689,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   __half* dst = static_cast<__half*>(p.dst);
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
-    const int mi = m0 + fm * 32 + i32;
+    const int mi = token(fm);
 #pragma unroll
     for (int ph = 0; ph < 16 / WAVES; ++ph) {
 #pragma unroll
@@ -712,12 +728,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   }
 }
 
-template <int FM, int U, int WAVES>
+template <int FM, int U, int WAVES, bool PAIR>
 void LaunchDirect(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
   if (zp)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR>), grid, dim3(WAVES * 64), 0, stream, p);
   else
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR>), grid, dim3(WAVES * 64), 0, stream, p);
 }
 
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
@@ -836,9 +852,7 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
   // token tile: 64 when that still yields a work-group per CU or M is large, else 32
   int fm = W4TokenBlocks(a.m, a.n);
-  int u = 4;
-  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e);
-  if (const char* e = std::getenv("MLDHIP_GEMM_U")) u = std::atoi(e);
+  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : 2;
   const int tiles = DivUp(a.n, 128) * DivUp(a.m, fm * 32);
   p.ksplit = 1;
   p.partial = a.partial;
@@ -851,19 +865,14 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
     if (want >= 1 && (size_t)want * p.ns * 4 * a.m <= a.partial_floats) p.ksplit = want;
   }
   const dim3 grid(DivUp(tiles, 8) * 8, p.ksplit);
-  int waves = 8;
-  if (const char* e = std::getenv("MLDHIP_GEMM_WAVES")) waves = std::atoi(e);
   const bool zp = p.zp != nullptr;
-  if (fm == 2 && waves == 8)
-    LaunchDirect<2, 4, 8>(zp, grid, stream, p);
-  else if (fm == 2 && u == 8)
-    LaunchDirect<2, 8, 4>(zp, grid, stream, p);
+  const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
+  if (fm == 2 && pair)
+    LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
   else if (fm == 2)
-    LaunchDirect<2, 4, 4>(zp, grid, stream, p);
-  else if (waves == 8)
-    LaunchDirect<1, 4, 8>(zp, grid, stream, p);
+    LaunchDirect<2, 4, 8, false>(zp, grid, stream, p);
   else
-    LaunchDirect<1, 4, 4>(zp, grid, stream, p);
+    LaunchDirect<1, 4, 8, false>(zp, grid, stream, p);
   if (p.ksplit > 1)
     hipLaunchKernelGGL(fc_w4_splitk_reduce_kernel, dim3(DivUp(p.ns * a.m, 256)), dim3(256), 0, stream, p);
   return hipGetLastError();
