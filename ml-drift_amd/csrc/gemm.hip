@@ -592,15 +592,20 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
 
   u32x2 rw[U][2], rsc[U], rzp[U], rx[U][NX][2];
   u32x4 rxp[U][NX][2];  // PAIR: {token 2j: 4 halfs, token 2j+1: 4 halfs} per K-slice row
-  auto load_step = [&](int t, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[NX][2], u32x4 (&xp)[NX][2]) {
+  auto load_step = [&](int t, bool with_scale, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[NX][2],
+                       u32x4 (&xp)[NX][2]) {
+    // The scales (and zero points) of a pair of steps (t - 1, t), t odd, which share a group
+    // because a group holds an even number of steps.  They travel with the odd step: by then
+    // both users of the previous pair are done with the registers.  First in the stage, so
+    // that waiting for them holds back as few younger loads as possible.
+    if (with_scale) {
+      sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
+      if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
+    }
     w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
     w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw1, 0, 0);
     vw0 += step_w;
     vw1 += step_w;
-    // scale group of this step (groups hold a power-of-two number of steps); a group past the
-    // last one reads zeros
-    sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
-    if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       if (PAIR) {
@@ -629,7 +634,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    load_step(t_begin + u, rw[u], rsc[u], rzp[u], rx[u], rxp[u]);
+    load_step(t_begin + u, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
     __builtin_amdgcn_sched_barrier(0);
   }
   for (int tt = 0; tt < per_wave; tt += U) {
@@ -639,11 +644,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       // consume stage u
       const u32x4 blk = {rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
       const u32x4 blk8 = {blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
-      const half2_t sc01 = AsHalf2(rsc[u][0]), sc23 = AsHalf2(rsc[u][1]);
+      const half2_t sc01 = AsHalf2(rsc[u & ~1][0]), sc23 = AsHalf2(rsc[u & ~1][1]);
       half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
       if (ZP) {
-        zp01 = AsHalf2(rzp[u][0]);
-        zp23 = AsHalf2(rzp[u][1]);
+        zp01 = AsHalf2(rzp[u & ~1][0]);
+        zp23 = AsHalf2(rzp[u & ~1][1]);
       }
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) {
@@ -675,7 +680,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       // refill stage u with step t + U; the fences keep the loads of a stage together and in
       // program order, so that waiting for one stage leaves the younger ones in flight
       __builtin_amdgcn_sched_barrier(0);
-      load_step(t + U, rw[u], rsc[u], rzp[u], rx[u], rxp[u]);
+      load_step(t + U, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -812,6 +817,7 @@ bool FcW4MfmaSupported(const FcArgs& a) {
     if (a.groups <= 0 || a.k % a.groups != 0 || (a.k / a.groups) % 16 != 0) return false;
     const int steps_per_group = (a.k / a.groups) / 16;
     if (steps_per_group & (steps_per_group - 1)) return false;  // the kernel finds the group by a shift
+    if (steps_per_group < 2) return false;                      // and loads the scales once per two steps
   }
   return true;
 }
