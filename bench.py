@@ -146,7 +146,7 @@ def run_other(args, torch, M, W):
         wb, fl = st.weight_bytes(), st.flops(tokens)
         if tokens == 1:
             out = dict(base, metric="int4_decoder_stack_decode_hbm_bandwidth", value=round(wb * args.steps / wall / 1e9, 1),
-                       unit="GB/s", roofline={"bound": "hbm", "kernel": "fc_w4_stream_kernel (126 launches per step)",
+                       unit="GB/s", roofline={"bound": "hbm", "kernel": "fc_w4_stream_kernel (126 FCs per step; q/k/v and gate/up share a launch)",
                                               "achieved": round(wb / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                               "frac": round(wb / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
                                               "avg_step_us": round(us, 1)})
