@@ -267,10 +267,13 @@ int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w);
 int mldhip_op_launch(mldhip_op* op, void* stream);
 
 /* One launch for up to 3 FullyConnected ops that read the same "src_tensor" (same binding, same
- * shape, same K and scale grouping) and are served by the streaming int4 kernel, e.g. the
+ * shape, same K and scale grouping) and are served by the same int4 kernel (streaming GEMV at a
+ * few tokens, MFMA GEMM beyond), e.g. the
  * q / k / v projections or the gate / up projections of a decoder layer, which the reference
  * emits as separate nodes over one input (samples/llm/gemma3_model_builder.cc:1115-1128).
- * Results are identical to launching the ops one by one.  Returns FAILED_PRECONDITION (and
+ * Results are those of launching the ops one by one (bit for bit, except that a fused MFMA launch
+ * may split K across work-groups differently, which changes the fp32 summation order).  Returns
+ * FAILED_PRECONDITION (and
  * launches nothing) when the ops cannot share a launch; the caller then launches them singly. */
 int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream);
 

@@ -613,6 +613,7 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
   if (!ops || count < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "no ops");
   if (count > 3) return Fail(MLDHIP_FAILED_PRECONDITION, "at most 3 ops per fused launch");
   FcArgs args[3];
+  bool stream_ok = true, mfma_ok = true;
   for (int i = 0; i < count; ++i) {
     mldhip_op* op = ops[i];
     if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
@@ -621,14 +622,17 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
     if (int rc = CheckBindings(op)) return rc;
     if (int rc = BuildFcArgs(op, &args[i])) return rc;
     const FcArgs &a = args[i], &f = args[0];
-    if (!FcW4StreamSupported(a))
-      return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " is not served by the streaming int4 kernel at this shape");
+    stream_ok = stream_ok && FcW4StreamSupported(a);
+    mfma_ok = mfma_ok && FcW4MfmaSupported(a);
     if (a.act != f.act || a.m != f.m || a.k != f.k || a.scale_kind != f.scale_kind || a.groups != f.groups ||
         a.has_zero_point != f.has_zero_point)
       return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " does not read the same tensor with the same K and scale groups as op 0");
   }
+  if (!stream_ok && !mfma_ok)
+    return Fail(MLDHIP_FAILED_PRECONDITION, "the ops are not all served by the same int4 kernel at this shape");
   const char* name = nullptr;
-  hipError_t e = LaunchFcW4StreamFused(args, count, static_cast<hipStream_t>(stream_ptr), &name);
+  hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
+  hipError_t e = stream_ok ? LaunchFcW4StreamFused(args, count, stream, &name) : LaunchFcW4MfmaFused(args, count, stream, &name);
   if (e != hipSuccess) return HipFail(e, "fused launch");
   for (int i = 0; i < count; ++i) ops[i]->last_kernel = name;
   return MLDHIP_OK;

@@ -35,7 +35,25 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 
+// One weight matrix of an int4 GEMM launch.  A launch covers up to kMaxW4Segments matrices
+// that read the same activations (same K): channel tiles [tile_end of the previous, tile_end)
+// belong to it.
+constexpr int kMaxW4Segments = 3;
+struct W4Segment {
+  const uint8_t* w4;    // [Ks][Ns] blocks of 8 bytes
+  const __half* scale;  // [groups][Ns][4]
+  const __half* zp;     // zero points, same shape as scale, or null
+  const __half* bias;
+  __half* dst;
+  float* partial;  // [ksplit][Ns][m][4] fp32 sums when ksplit > 1
+  int n, ns;
+  int tile_end;
+  uint32_t a_bytes, s_bytes;
+};
+
 struct GemmParams {
+  W4Segment seg[kMaxW4Segments];
+  int segments;
   int m, n, k;
   int ns;        // output slices, ceil(n/4)
   int k_steps;   // K-steps
@@ -43,10 +61,7 @@ struct GemmParams {
   const void* bias;
   int dst_type;
   // fp16 / int4 path
-  const uint8_t* w4;    // [Ks][Ns] blocks of 8 bytes
   const __half* act;    // [Ks][m][4]
-  const __half* scale;  // [groups][Ns][4]
-  const __half* zp;     // zero points, same shape as scale, or null
   int ks;               // input slices, ceil(k/4)
   int steps_per_group;  // K-steps per scale group
   int groups;
@@ -63,7 +78,6 @@ struct GemmParams {
   uint32_t a_bytes, b_bytes, s_bytes;
   int group_size;   // input channels per scale group (fp16 path)
   int ksplit;       // work-groups along K per output tile (fp16 path)
-  float* partial;   // [ksplit][Ns][m][4] fp32 sums when ksplit > 1
   int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
 };
 
@@ -537,15 +551,21 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // L2.  Tiles are numbered token-tile-major and XCD x takes the contiguous range
   // [x*per_xcd, (x+1)*per_xcd): the work-groups that share an L2 then share a few activation
   // tiles (the big fp16 operand), and every weight tile streams through that L2 once.
-  const int tiles_n = (p.n + BN - 1) / BN;
+  const int tiles_n = p.seg[p.segments - 1].tile_end;  // channel tiles of all matrices of the launch
   const int tiles_m = (p.m + BM - 1) / BM;
   const int per_xcd = (tiles_n * tiles_m + 7) / 8;
   const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= tiles_n * tiles_m) return;
-  const int n0 = (tile % tiles_n) * BN;
+  int tn = tile % tiles_n, si = 0;
+  if (p.segments > 1 && tn >= p.seg[0].tile_end) {
+    si = (p.segments > 2 && tn >= p.seg[1].tile_end) ? 2 : 1;
+    tn -= p.seg[si - 1].tile_end;
+  }
+  const W4Segment& sg = p.seg[si];
+  const int n0 = tn * BN;
   const int m0 = (tile / tiles_n) * BM;
   const int nsi = n0 / 4 + i32;
-  const bool n_ok = nsi < p.ns;
+  const bool n_ok = nsi < sg.ns;
 
   // This wave's range of 16-channel steps.  The buffer descriptors of the weights and the
   // activations end where the wave's share of K ends, so the prefetches that run past it (and
@@ -555,21 +575,21 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int shares = WAVES * p.ksplit;  // blockIdx.y selects the work-group's part of K
   const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
   const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * WAVES + wave) * per_wave);
-  const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
+  const uint32_t row_w = (uint32_t)sg.ns * 8u;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
-  const uint32_t w_end = min((uint64_t)p.a_bytes, (uint64_t)k_slices_end * row_w);
+  const uint32_t w_end = min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w);
   const uint32_t x_end = min((uint64_t)p.b_bytes, (uint64_t)k_slices_end * row_x);
 
   constexpr uint32_t kOob = 0x7FFFFFF0u;
   const __amdgpu_buffer_rsrc_t rsrc_w =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(p.w4), 0, w_end, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sg.w4), 0, w_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_x =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, x_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_s =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.scale), 0, p.s_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(sg.scale), 0, sg.s_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_z =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(ZP ? p.zp : p.scale), 0, p.s_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(ZP ? sg.zp : sg.scale), 0, sg.s_bytes, 0x00020000);
 
   // Per-lane byte offsets of the next step to fetch; each fetch advances them by one step.
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
@@ -690,8 +710,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // WAVES copies of register w in a fixed order and stores that part of the output.  In the
   // 32x32 result, register v of lane (g2, i32) belongs to output slice 8*(v/4) + 4*g2 + v%4 and
   // token i32, and the four MFMAs hold the slice's four channels: one 8-byte store.
-  const __half* bias = static_cast<const __half*>(p.bias);
-  __half* dst = static_cast<__half*>(p.dst);
+  const __half* bias = sg.bias;
+  __half* dst = sg.dst;
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
     const int mi = token(fm);
@@ -714,10 +734,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       }
       const int v = ph * WAVES + wave;
       const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-      if (mi < p.m && slice < p.ns && p.ksplit > 1) {
+      if (mi < p.m && slice < sg.ns && p.ksplit > 1) {
         // this work-group's share of K: fp32 sums for the second pass
-        *reinterpret_cast<float4*>(p.partial + (((size_t)blockIdx.y * p.ns + slice) * p.m + mi) * 4) = sum;
-      } else if (mi < p.m && slice < p.ns) {
+        *reinterpret_cast<float4*>(sg.partial + (((size_t)blockIdx.y * sg.ns + slice) * p.m + mi) * 4) = sum;
+      } else if (mi < p.m && slice < sg.ns) {
         __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
         if (bias) {
 #pragma unroll
@@ -744,10 +764,17 @@ void LaunchDirect(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
 // the bias.  One thread per (slice, token).
 __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) {
-  const size_t items = (size_t)p.ns * p.m;
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= items) return;
-  const float4* part = reinterpret_cast<const float4*>(p.partial);
+  // items of all matrices of the launch, matrix after matrix
+  size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  int si = 0;
+  while (si < p.segments && idx >= (size_t)p.seg[si].ns * p.m) {
+    idx -= (size_t)p.seg[si].ns * p.m;
+    ++si;
+  }
+  if (si >= p.segments) return;
+  const W4Segment& sg = p.seg[si];
+  const size_t items = (size_t)sg.ns * p.m;
+  const float4* part = reinterpret_cast<const float4*>(sg.partial);
   float4 sum = part[idx];
   for (int s = 1; s < p.ksplit; ++s) {
     const float4 o = part[(size_t)s * items + idx];
@@ -757,15 +784,15 @@ __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) 
     sum.w += o.w;
   }
   __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
-  if (p.bias) {
-    const __half* bias = static_cast<const __half*>(p.bias) + (idx / p.m) * 4;
+  if (sg.bias) {
+    const __half* bias = sg.bias + (idx / p.m) * 4;
 #pragma unroll
     for (int c = 0; c < 4; ++c) h[c] = __hadd(h[c], bias[c]);
   }
   u32x2 o;
   o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
   o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-  reinterpret_cast<u32x2*>(p.dst)[idx] = o;
+  reinterpret_cast<u32x2*>(sg.dst)[idx] = o;
 }
 
 // Token tile of the int4 GEMM: 64 when that still yields a work-group for half the CUs or M is
@@ -822,30 +849,22 @@ bool FcW4MfmaSupported(const FcArgs& a) {
   return true;
 }
 
-hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name) {
+  if (count < 1 || count > kMaxW4Segments) return hipErrorInvalidValue;
+  const FcArgs& a = args[0];
   GemmParams p = {};
+  p.segments = count;
   p.m = a.m;
-  p.n = a.n;
   p.k = a.k;
-  p.ns = DivUp(a.n, 4);
   p.ks = DivUp(a.k, 4);
-  p.k_steps = DivUp(a.k, 32);
-  p.dst = a.dst;
-  p.bias = a.bias;
   p.dst_type = MLDHIP_FLOAT16;
-  p.w4 = a.weights;
   p.act = static_cast<const __half*>(a.act);
-  p.scale = static_cast<const __half*>(a.scale);
-  p.zp = a.has_zero_point ? static_cast<const __half*>(a.zero_point) : nullptr;
   p.groups = a.scale_kind == kScaleBlock ? a.groups : 1;
-  p.steps_per_group = a.scale_kind == kScaleBlock ? (a.k / a.groups) / 32 : p.k_steps;
   p.mask_lo = 0x000F000Fu;
   p.mask_hi = 0x00F000F0u;
   p.magic_lo = 0x64006400u;
   p.magic_hi = 0x54005400u;
-  p.a_bytes = (uint32_t)((size_t)p.ks * p.ns * 8);
   p.b_bytes = (uint32_t)((size_t)p.ks * p.m * 8);
-  p.s_bytes = (uint32_t)((size_t)p.groups * p.ns * 8);
   p.group_size = a.scale_kind == kScaleBlock ? a.k / a.groups : a.k;
   p.group_shift = -1;
   if (a.scale_kind != kScaleBlock) {
@@ -855,23 +874,36 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
     for (int sh = 0; sh < 30; ++sh)
       if ((1 << sh) == spg) p.group_shift = sh;
   }
+  int n_total = 0, tiles_n = 0;
+  for (int i = 0; i < count; ++i) {
+    W4Segment& sg = p.seg[i];
+    sg.w4 = args[i].weights;
+    sg.scale = static_cast<const __half*>(args[i].scale);
+    sg.zp = args[i].has_zero_point ? static_cast<const __half*>(args[i].zero_point) : nullptr;
+    sg.bias = static_cast<const __half*>(args[i].bias);
+    sg.dst = static_cast<__half*>(args[i].dst);
+    sg.partial = args[i].partial;
+    sg.n = args[i].n;
+    sg.ns = DivUp(args[i].n, 4);
+    sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * 8);
+    sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8);
+    tiles_n += DivUp(args[i].n, 128);
+    sg.tile_end = tiles_n;
+    n_total += args[i].n;
+  }
+  for (int i = count; i < kMaxW4Segments; ++i) p.seg[i] = p.seg[0];
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
-  // token tile: 64 when that still yields a work-group per CU or M is large, else 32
-  int fm = W4TokenBlocks(a.m, a.n);
+  // token tile and K split follow the launch as a whole (all channels of all matrices)
+  int fm = W4TokenBlocks(a.m, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : 2;
-  const int tiles = DivUp(a.n, 128) * DivUp(a.m, fm * 32);
+  const int tiles = tiles_n * DivUp(a.m, fm * 32);
   p.ksplit = 1;
-  p.partial = a.partial;
-  if (fm == W4TokenBlocks(a.m, a.n)) {
-    p.ksplit = W4KSplit(a.m, a.k, a.n);
-    while (p.ksplit > 1 && (size_t)p.ksplit * p.ns * 4 * a.m > a.partial_floats) p.ksplit /= 2;
-  }
-  if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) {
-    const int want = std::atoi(e);
-    if (want >= 1 && (size_t)want * p.ns * 4 * a.m <= a.partial_floats) p.ksplit = want;
-  }
+  if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
+  if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) p.ksplit = std::max(1, std::atoi(e));
+  for (int i = 0; i < count; ++i)
+    while (p.ksplit > 1 && (size_t)p.ksplit * p.seg[i].ns * 4 * a.m > args[i].partial_floats) p.ksplit /= 2;
   const dim3 grid(DivUp(tiles, 8) * 8, p.ksplit);
-  const bool zp = p.zp != nullptr;
+  const bool zp = p.seg[0].zp != nullptr;
   const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
   if (fm == 2 && pair)
     LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
@@ -879,9 +911,16 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
     LaunchDirect<2, 4, 8, false>(zp, grid, stream, p);
   else
     LaunchDirect<1, 4, 8, false>(zp, grid, stream, p);
-  if (p.ksplit > 1)
-    hipLaunchKernelGGL(fc_w4_splitk_reduce_kernel, dim3(DivUp(p.ns * a.m, 256)), dim3(256), 0, stream, p);
+  if (p.ksplit > 1) {
+    size_t items = 0;
+    for (int i = 0; i < count; ++i) items += (size_t)p.seg[i].ns * a.m;
+    hipLaunchKernelGGL(fc_w4_splitk_reduce_kernel, dim3((unsigned)DivUp((long)items, 256L)), dim3(256), 0, stream, p);
+  }
   return hipGetLastError();
+}
+
+hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+  return LaunchFcW4MfmaFused(&a, 1, stream, kernel_name);
 }
 
 size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n) {

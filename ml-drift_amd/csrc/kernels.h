@@ -77,6 +77,8 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
 // Multi-token FullyConnected with int4 weights on the MFMA units (fp16 tensors).
 bool FcW4MfmaSupported(const FcArgs& a);
 hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+// Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
+hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 // fp32 workspace the MFMA path wants for token counts up to max_tokens (K split across
 // work-groups); 0 when it never splits.
 size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n);
