@@ -535,7 +535,9 @@ __device__ __forceinline__ void LdsBarrier() { asm volatile("s_waitcnt lgkmcnt(0
 // moves from 8 to 8 + zp (exact in fp16 for integral zero points).
 // PAIR (FM even, token count even): a lane's tokens for the MFMA pair (fm, fm+1) are neighbours
 // (2j, 2j+1 instead of j, j+32), so one 16-byte load brings both activation operands.
-template <int FM, int U, int WAVES, bool ZP, bool PAIR>
+// MULTI: the launch covers more than one matrix (the single-matrix instantiation reads its
+// arguments at fixed offsets instead of through a dependent scalar load).
+template <int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
   constexpr int BN = 128;
@@ -551,17 +553,17 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // L2.  Tiles are numbered token-tile-major and XCD x takes the contiguous range
   // [x*per_xcd, (x+1)*per_xcd): the work-groups that share an L2 then share a few activation
   // tiles (the big fp16 operand), and every weight tile streams through that L2 once.
-  const int tiles_n = p.seg[p.segments - 1].tile_end;  // channel tiles of all matrices of the launch
+  const int tiles_n = p.seg[MULTI ? p.segments - 1 : 0].tile_end;  // channel tiles of all matrices of the launch
   const int tiles_m = (p.m + BM - 1) / BM;
   const int per_xcd = (tiles_n * tiles_m + 7) / 8;
   const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (tile >= tiles_n * tiles_m) return;
   int tn = tile % tiles_n, si = 0;
-  if (p.segments > 1 && tn >= p.seg[0].tile_end) {
+  if (MULTI && p.segments > 1 && tn >= p.seg[0].tile_end) {
     si = (p.segments > 2 && tn >= p.seg[1].tile_end) ? 2 : 1;
     tn -= p.seg[si - 1].tile_end;
   }
-  const W4Segment& sg = p.seg[si];
+  const W4Segment& sg = p.seg[MULTI ? si : 0];
   const int n0 = tn * BN;
   const int m0 = (tile / tiles_n) * BM;
   const int nsi = n0 / 4 + i32;
@@ -755,10 +757,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
 
 template <int FM, int U, int WAVES, bool PAIR>
 void LaunchDirect(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
-  if (zp)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR>), grid, dim3(WAVES * 64), 0, stream, p);
+  const dim3 block(WAVES * 64);
+  if (zp && p.segments > 1)
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR, true>), grid, block, 0, stream, p);
+  else if (zp)
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR, false>), grid, block, 0, stream, p);
+  else if (p.segments > 1)
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR, true>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR>), grid, dim3(WAVES * 64), 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR, false>), grid, block, 0, stream, p);
 }
 
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
