@@ -568,6 +568,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4MfmaSupported(a)) {
         e = LaunchFcW4Mfma(a, stream, &op->last_kernel);
+      } else if (!force_generic && FcW8StreamSupported(a)) {
+        e = LaunchFcW8Stream(a, stream, &op->last_kernel);
       } else {
         e = LaunchFcGeneric(a, stream, &op->last_kernel);
       }

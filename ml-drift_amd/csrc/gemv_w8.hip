@@ -1,0 +1,257 @@
+// Streaming int8 GEMV for gfx950 (decode: 1..4 tokens, fp32 or fp16 tensors, per-channel or
+// group-wise scales, optional zero points).
+//
+// Packed buffer (the reference's I4O4 layout with one byte per weight): row ks (4 input
+// channels) holds Ns blocks of 16 bytes; in a block, word i is input channel i and its bytes
+// are the output channels 0..3 of the slice, stored as u = w + 128.
+//
+// All arithmetic is fp32: a byte becomes a float with one conversion (v_cvt_f32_ubyte0..3) and
+// enters one fused multiply-add.  The constant centre is not subtracted per weight:
+// sum_k a_k (u_k - c) = sum_k a_k u_k - c sum_k a_k with c = 128 + zero point, removed once per
+// chunk of 32 input channels (one scale group when group-wise), where the scale is applied too.
+//
+// Thread layout as in the int4 kernel: LPR lanes cover one contiguous row segment (LPR x 16 B =
+// LPR slices), 64/LPR rows per wave, WAVES waves per work-group; a thread owns whole chunks of
+// 8 consecutive K-slices, issues its 8 weight loads back to back and prefetches the next
+// chunk while it computes.  K is reduced through LDS in a fixed order.
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace mldhip {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+struct W8Params {
+  const u32x4* weights;
+  const void* act;
+  const void* scale;
+  const void* zero_point;  // same shape as scale, or null
+  const void* bias;
+  void* dst;
+  int m, ks, ns;
+  int chunks;        // ceil(ks / 8)
+  int group_chunks;  // chunks per scale group (grouped only)
+  int groups;
+  int grouped;
+};
+
+__device__ __forceinline__ void Load4(const float* p, size_t i, float v[4]) {
+  const float4 r = *reinterpret_cast<const float4*>(p + i);
+  v[0] = r.x;
+  v[1] = r.y;
+  v[2] = r.z;
+  v[3] = r.w;
+}
+__device__ __forceinline__ void Load4(const __half* p, size_t i, float v[4]) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p + i);
+  const __half2 lo = *reinterpret_cast<const __half2*>(&r.x);
+  const __half2 hi = *reinterpret_cast<const __half2*>(&r.y);
+  v[0] = __low2float(lo);
+  v[1] = __high2float(lo);
+  v[2] = __low2float(hi);
+  v[3] = __high2float(hi);
+}
+__device__ __forceinline__ void Store1(float* dst, size_t i, float r, const float* bias, size_t bi) {
+  dst[i] = bias ? r + bias[bi] : r;
+}
+__device__ __forceinline__ void Store1(__half* dst, size_t i, float r, const __half* bias, size_t bi) {
+  __half h = __float2half_rn(r);
+  if (bias) h = __hadd(h, bias[bi]);
+  dst[i] = h;
+}
+
+template <typename T, int LPR, int WAVES, int M>
+__global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
+  constexpr int RPW = 64 / LPR;        // rows per wave
+  constexpr int STRIP = LPR * 4;       // output channels per work-group
+  constexpr int PARTS = THREADS / STRIP > ROWS ? ROWS : THREADS / STRIP;
+  constexpr int RPP = ROWS / PARTS;    // rows per part
+  __shared__ float red[ROWS][M][STRIP];
+  __shared__ float red2[PARTS][M][STRIP];
+
+  const T* act = static_cast<const T*>(p.act);
+  const T* scale = static_cast<const T*>(p.scale);
+  const T* zero_point = static_cast<const T*>(p.zero_point);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane % LPR;
+  const int row = wave * RPW + lane / LPR;
+  const int slice_raw = blockIdx.x * LPR + col;
+  const int slice = slice_raw < p.ns ? slice_raw : p.ns - 1;  // clamp: loads stay in range, result unused
+
+  float acc[M][4];
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+#pragma unroll
+    for (int o = 0; o < 4; ++o) acc[m][o] = 0.0f;
+
+  // per-channel constants
+  float s_lin[4] = {1.0f, 1.0f, 1.0f, 1.0f}, z_lin[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (!p.grouped) {
+    Load4(scale, (size_t)slice * 4, s_lin);
+    if (zero_point) Load4(zero_point, (size_t)slice * 4, z_lin);
+  }
+
+  auto load_weights = [&](int c, u32x4 (&w)[8]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int ks = min(c * 8 + j, p.ks - 1);  // rows past K re-read the last one; their activations are zero
+      w[j] = __builtin_nontemporal_load(p.weights + (size_t)ks * p.ns + slice);
+    }
+  };
+  auto load_acts = [&](int c, float (&a)[8][M][4]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int ks = c * 8 + j;
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        Load4(act, ((size_t)min(ks, p.ks - 1) * M + m) * 4, a[j][m]);
+        if (ks >= p.ks) a[j][m][0] = a[j][m][1] = a[j][m][2] = a[j][m][3] = 0.0f;
+      }
+    }
+  };
+
+  for (int c = row; c < p.chunks; c += ROWS) {
+    u32x4 w[8];
+    float a[8][M][4];
+    load_weights(c, w);
+    load_acts(c, a);
+    float s[4], z[4];
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      s[o] = s_lin[o];
+      z[o] = z_lin[o];
+    }
+    if (p.grouped) {
+      int g = c / p.group_chunks;
+      if (g >= p.groups) g = p.groups - 1;
+      Load4(scale, ((size_t)g * p.ns + slice) * 4, s);
+      if (zero_point) Load4(zero_point, ((size_t)g * p.ns + slice) * 4, z);
+    }
+    float t[M][4], asum[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      asum[m] = 0.0f;
+#pragma unroll
+      for (int o = 0; o < 4; ++o) t[m][o] = 0.0f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t word = w[j][i];
+        const float u0 = (float)(word & 0xFFu), u1 = (float)((word >> 8) & 0xFFu);
+        const float u2 = (float)((word >> 16) & 0xFFu), u3 = (float)(word >> 24);
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          const float av = a[j][m][i];
+          asum[m] += av;
+          t[m][0] = fmaf(av, u0, t[m][0]);
+          t[m][1] = fmaf(av, u1, t[m][1]);
+          t[m][2] = fmaf(av, u2, t[m][2]);
+          t[m][3] = fmaf(av, u3, t[m][3]);
+        }
+      }
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int o = 0; o < 4; ++o) acc[m][o] = fmaf(s[o], fmaf(-(128.0f + z[o]), asum[m], t[m][o]), acc[m][o]);
+  }
+
+  // K reduction through LDS: every thread stores its 4*M sums, PARTS threads per output add
+  // ROWS/PARTS rows each, then one thread per output adds the PARTS results.
+#pragma unroll
+  for (int m = 0; m < M; ++m)
+    *reinterpret_cast<float4*>(&red[row][m][col * 4]) = make_float4(acc[m][0], acc[m][1], acc[m][2], acc[m][3]);
+  __syncthreads();
+  const int nl = tid % STRIP;
+  const int part = tid / STRIP;
+  if (part < PARTS) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float v = 0.0f;
+#pragma unroll
+      for (int r = 0; r < RPP; ++r) v += red[part * RPP + r][m][nl];
+      red2[part][m][nl] = v;
+    }
+  }
+  __syncthreads();
+  T* dst = static_cast<T*>(p.dst);
+  const T* bias = static_cast<const T*>(p.bias);
+  const int n0 = blockIdx.x * STRIP;
+  for (int idx = tid; idx < M * STRIP; idx += THREADS) {
+    const int m = idx / STRIP, ol = idx % STRIP;
+    const int n = n0 + ol;
+    if (n >= p.ns * 4) continue;
+    float v = 0.0f;
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
+    Store1(dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, bias, (size_t)n);
+  }
+}
+
+template <typename T, int LPR, int WAVES>
+hipError_t LaunchM(const W8Params& p, dim3 grid, hipStream_t stream) {
+  const dim3 block(WAVES * 64);
+  switch (p.m) {
+    case 1: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1>), grid, block, 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 2>), grid, block, 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 3>), grid, block, 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 4>), grid, block, 0, stream, p); break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+template <typename T>
+hipError_t LaunchT(const W8Params& p, int lpr, int waves, hipStream_t stream) {
+  const dim3 grid(DivUp(p.ns, lpr));
+  if (lpr == 4) return waves == 4 ? LaunchM<T, 4, 4>(p, grid, stream) : LaunchM<T, 4, 16>(p, grid, stream);
+  return waves == 4 ? LaunchM<T, 8, 4>(p, grid, stream) : LaunchM<T, 8, 16>(p, grid, stream);
+}
+
+}  // namespace
+
+bool FcW8StreamSupported(const FcArgs& a) {
+  if (a.weight_bits != 8 || a.act_f16 != a.dst_f16) return false;
+  if (a.m < 1 || a.m > kGemvMaxTokens) return false;
+  if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
+  if (a.scale_kind == kScaleScalar) return false;
+  if (a.scale_kind == kScaleBlock) {
+    const int ks = DivUp(a.k, 4);
+    if (a.groups <= 0 || ks % a.groups != 0) return false;
+    if ((ks / a.groups) % 8 != 0) return false;  // a chunk of 8 K-slices must not straddle groups
+  }
+  return true;
+}
+
+hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+  W8Params p;
+  p.weights = reinterpret_cast<const u32x4*>(a.weights);
+  p.act = a.act;
+  p.scale = a.scale;
+  p.zero_point = a.has_zero_point ? a.zero_point : nullptr;
+  p.bias = a.bias;
+  p.dst = a.dst;
+  p.m = a.m;
+  p.ks = DivUp(a.k, 4);
+  p.ns = DivUp(a.n, 4);
+  p.chunks = DivUp(p.ks, 8);
+  p.grouped = a.scale_kind == kScaleBlock;
+  p.groups = p.grouped ? a.groups : 1;
+  p.group_chunks = p.grouped ? (p.ks / a.groups) / 8 : p.chunks;
+  // 128-byte row segments (8 slices) when that still gives a work-group to half the CUs, else
+  // 64-byte ones; small work-groups when K is covered by 64 / 128 rows of chunks
+  const int lpr = DivUp(p.ns, 8) >= 128 ? 8 : 4;
+  const int waves = p.chunks <= 4 * 64 / lpr ? 4 : 16;
+  if (kernel_name) *kernel_name = "fc_w8_stream_kernel";
+  return a.act_f16 ? LaunchT<__half>(p, lpr, waves, stream) : LaunchT<float>(p, lpr, waves, stream);
+}
+
+}  // namespace mldhip

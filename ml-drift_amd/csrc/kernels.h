@@ -44,6 +44,10 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 
+// Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
+bool FcW8StreamSupported(const FcArgs& a);
+hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+
 // int8 activations x uint8/uint4 weights -> int32 (no scales).
 hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k,
                             int n, int weight_bits, hipStream_t stream, const char** kernel_name);

@@ -100,7 +100,7 @@ def run_case(oracle, case, expect_kernel=None, env=None):
 
 def test_config1_int8_fp32(oracle):
     case = W.make_fc_case(**W.CONFIGS["c1"])
-    run_case(oracle, case, "fc_generic_kernel")
+    run_case(oracle, case, "fc_w8_stream_kernel")
 
 
 def test_config2_int4_decode(oracle):
@@ -143,6 +143,17 @@ def test_stream_kernel_zero_points(oracle, m, groups):
     run_case(oracle, case, "fc_w4_stream_kernel")
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("m,k,n,groups,zp", [(1, 2048, 2048, 1, False), (4, 1000, 1030, 1, True), (3, 2048, 516, 64, True),
+                                             (2, 4096, 8192, 16, False), (1, 64, 8, 1, False)])
+def test_w8_stream_kernel(oracle, dtype, m, k, n, groups, zp):
+    """int8 weights on the streaming kernel: both tensor types, per-channel and group-wise scales,
+    zero points, ragged K (1000) and N (1030), tiny layers."""
+    case = W.make_fc_case(seed=31 + m, m=m, k=k, n=n, weight_bits=8, tensor_dtype=dtype, groups=groups,
+                          with_bias=True, with_zero_point=zp)
+    run_case(oracle, case, "fc_w8_stream_kernel")
+
+
 @pytest.mark.parametrize("name,k,n", W.C5_LAYER)
 def test_config5_decode_layer_shapes(oracle, name, k, n):
     case = W.make_fc_case(seed=7, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=k // 32)
@@ -171,6 +182,8 @@ def test_generic_kernel_reference_test_shapes(oracle, bits, dtype, kind):
         expect = "fc_generic_kernel"
         if fast:  # symmetric fp16 int4: streaming GEMV up to 4 tokens, MFMA GEMM beyond
             expect = "fc_w4_stream_kernel" if m <= 4 else "fc_w4_mfma_gemm_kernel"
+        if bits == 8 and kind == "linear" and m <= 4:  # per-channel int8, either tensor type
+            expect = "fc_w8_stream_kernel"
         run_case(oracle, case, expect)
 
 
