@@ -29,8 +29,14 @@ __device__ __forceinline__ void StoreOut(__half* dst, size_t i, float r, const _
   dst[i] = h;
 }
 
+// Work-group geometry of both kernels: x = output slice inside a strip of kSl, y = K lane.
+// Narrow strips and many K lanes: a 14336-channel layer is 224 work-groups, and a lane's K loop
+// is short enough to unroll, so that several loads are in flight per thread.
+constexpr int kSl = 8;
+constexpr int kKl = 32;
+
 // ------------------------------------------------------------------------------------------
-// Generic kernel.  Block (64, 4): x = output slice inside a strip of 64, y = K lane.
+// Generic kernel.
 // ------------------------------------------------------------------------------------------
 struct GenericParams {
   const void* act;
@@ -47,9 +53,9 @@ struct GenericParams {
 
 template <typename ActT, typename DstT, int WBITS, int TB>
 __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
-  __shared__ float red[4][64][TB * 4];
+  __shared__ float red[kKl][kSl][TB * 4];
   const int tx = threadIdx.x, ty = threadIdx.y;
-  const int ds = blockIdx.x * 64 + tx;
+  const int ds = blockIdx.x * kSl + tx;
   const int tok0 = blockIdx.y * TB;
   const ActT* act = static_cast<const ActT*>(p.act);
   const ActT* scale = static_cast<const ActT*>(p.scale);
@@ -76,7 +82,8 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
         if (zp) z[c] = LoadF(zp, (size_t)ds * 4 + c);
       }
     }
-    for (int ks = ty; ks < p.ks; ks += 4) {
+#pragma unroll 4
+    for (int ks = ty; ks < p.ks; ks += kKl) {
       if (p.scale_kind == kScaleBlock) {
         int g = ks / p.group_slices;
         if (g >= p.groups) g = p.groups - 1;
@@ -132,8 +139,9 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
       if (tok >= p.m) continue;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const float r = (red[0][tx][t * 4 + c] + red[1][tx][t * 4 + c]) +
-                        (red[2][tx][t * 4 + c] + red[3][tx][t * 4 + c]);
+        float r = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kKl; ++q) r += red[q][tx][t * 4 + c];
         StoreOut(dst, ((size_t)ds * p.m + tok) * 4 + c, r, bias, (size_t)ds * 4 + c);
       }
     }
@@ -143,8 +151,8 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 template <typename ActT, typename DstT, int WBITS>
 hipError_t LaunchGenericT(const GenericParams& p, hipStream_t stream) {
   constexpr int TB = 4;
-  dim3 grid(DivUp(p.ns, 64), DivUp(p.m, TB));
-  dim3 block(64, 4);
+  dim3 grid(DivUp(p.ns, kSl), DivUp(p.m, TB));
+  dim3 block(kSl, kKl);
   hipLaunchKernelGGL((fc_generic_kernel<ActT, DstT, WBITS, TB>), grid, block, 0, stream, p);
   return hipGetLastError();
 }
@@ -157,9 +165,9 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
                                                            const uint8_t* __restrict__ weights,
                                                            int32_t* __restrict__ dst, int m, int ks_n,
                                                            int ns) {
-  __shared__ int red[4][64][TB * 4];
+  __shared__ int red[kKl][kSl][TB * 4];
   const int tx = threadIdx.x, ty = threadIdx.y;
-  const int ds = blockIdx.x * 64 + tx;
+  const int ds = blockIdx.x * kSl + tx;
   const int tok0 = blockIdx.y * TB;
   int acc[TB][4];
 #pragma unroll
@@ -167,7 +175,8 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[t][c] = 0;
   if (ds < ns) {
-    for (int ks = ty; ks < ks_n; ks += 4) {
+#pragma unroll 4
+    for (int ks = ty; ks < ks_n; ks += kKl) {
       const size_t blk = (size_t)ks * ns + ds;
       uint32_t w0, w1, w2, w3;  // per output channel: the 4 input-channel values, one per byte
       if (WBITS == 4) {
@@ -235,8 +244,12 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
       if (tok >= m) continue;
 #pragma unroll
       for (int c = 0; c < 4; ++c)
-        dst[((size_t)ds * m + tok) * 4 + c] = red[0][tx][t * 4 + c] + red[1][tx][t * 4 + c] +
-                                              red[2][tx][t * 4 + c] + red[3][tx][t * 4 + c];
+      {
+        int r = 0;
+#pragma unroll
+        for (int q = 0; q < kKl; ++q) r += red[q][tx][t * 4 + c];
+        dst[((size_t)ds * m + tok) * 4 + c] = r;
+      }
     }
   }
 }
@@ -275,8 +288,8 @@ hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* 
                             int n, int weight_bits, hipStream_t stream, const char** kernel_name) {
   constexpr int TB = 4;
   const int ks = DivUp(k, 4), ns = DivUp(n, 4);
-  dim3 grid(DivUp(ns, 64), DivUp(m, TB));
-  dim3 block(64, 4);
+  dim3 grid(DivUp(ns, kSl), DivUp(m, TB));
+  dim3 block(kSl, kKl);
   if (kernel_name) *kernel_name = "fc_int8_math_kernel";
   if (weight_bits == 8)
     hipLaunchKernelGGL((fc_int8_math_kernel<8, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns);
