@@ -84,6 +84,9 @@ __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const 
   dst[i] = h;
 }
 
+// Branch-free: a K-slice past the end re-reads the last row of weights against zeroed
+// activations, so the eight loads of a chunk are issued back to back and the waits for them can
+// be counted down one by one while the arithmetic of the earlier slices runs.
 template <int M>
 __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* weights, int row_u4, int c, int pcol,
                                           u32x4 w[8], u32x2 a[8][M]) {
@@ -91,16 +94,12 @@ __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* we
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int ks = ks0 + j;
-    if (ks < p.ks) {
-      w[j] = __builtin_nontemporal_load(weights + (size_t)ks * row_u4 + pcol);
+    const int ksc = min(ks, p.ks - 1);
+    w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * row_u4 + pcol);
 #pragma unroll
-      for (int m = 0; m < M; ++m)
-        a[j][m] = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ks * M + m) * 4);
-    } else {
-      // u = 8 everywhere: a zero weight
-      w[j] = u32x4{0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u};
-#pragma unroll
-      for (int m = 0; m < M; ++m) a[j][m] = u32x2{0u, 0u};
+    for (int m = 0; m < M; ++m) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksc * M + m) * 4);
+      a[j][m] = u32x2{ks < p.ks ? v[0] : 0u, ks < p.ks ? v[1] : 0u};
     }
   }
 }
@@ -399,6 +398,11 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     lpr = DivUp(total_row_u4, 4) >= 64 ? 4 : 2;
   lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
   if (lpr != 2 && lpr != 4 && lpr != 8 && lpr != 16) lpr = 8;
+  // two and more tokens need the registers of a small work-group (the 1024-thread shapes spill)
+  if (p.m >= 2) {
+    waves = 4;
+    if (lpr == 16) lpr = 8;
+  }
   waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
   int strips = 0;
