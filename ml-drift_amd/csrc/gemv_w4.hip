@@ -423,6 +423,11 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   int ksplit = 1;
   if (strips < 128 && count == 1) {
     ksplit = DivUp(256, strips);
+    // a smaller work-group (down to 8 waves) when K does not otherwise split that far
+    while (lpr == 8 && waves > 8 && DivUp(p.chunks, rows) < ksplit) {
+      waves /= 2;
+      rows /= 2;
+    }
     const int max_split = DivUp(p.chunks, rows);
     if (ksplit > max_split) ksplit = max_split;
   }
