@@ -79,6 +79,7 @@ struct GemmParams {
   int group_size;   // input channels per scale group (fp16 path)
   int ksplit;       // work-groups along K per output tile (fp16 path)
   int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
+  int xcd_m;        // fp16 path: the 8 XCDs form an xcd_m x (8 / xcd_m) grid over (token tiles, channel tiles)
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -550,22 +551,26 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int wave = tid >> 6;
   const int i32 = lane & 31, g2 = lane >> 5;
   // XCD-aware tile order.  Work-groups go round-robin to the 8 XCDs (id % 8), each with its own
-  // L2.  Tiles are numbered token-tile-major and XCD x takes the contiguous range
-  // [x*per_xcd, (x+1)*per_xcd): the work-groups that share an L2 then share a few activation
-  // tiles (the big fp16 operand), and every weight tile streams through that L2 once.
+  // L2.  The XCDs form an xcd_m x (8 / xcd_m) grid over the (token tile, channel tile) plane and
+  // each owns one rectangle of it: the work-groups that share an L2 then share the activation
+  // tiles and the weight tiles of that rectangle, and the L2 fetches each of them once.  Inside
+  // the rectangle the token tile runs fastest, so that the tiles in flight at any time reuse the
+  // same few activation tiles while the weights stream through.
   const int tiles_n = p.seg[MULTI ? p.segments - 1 : 0].tile_end;  // channel tiles of all matrices of the launch
   const int tiles_m = (p.m + BM - 1) / BM;
-  const int per_xcd = (tiles_n * tiles_m + 7) / 8;
-  const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (tile >= tiles_n * tiles_m) return;
-  int tn = tile % tiles_n, si = 0;
+  const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
+  const int xm = p.xcd_m, xn = 8 / xm;
+  const int rect_m = (tiles_m + xm - 1) / xm, rect_n = (tiles_n + xn - 1) / xn;
+  const int tm = (xcd % xm) * rect_m + local % rect_m;
+  int tn = (xcd / xm) * rect_n + local / rect_m, si = 0;
+  if (tm >= tiles_m || tn >= tiles_n) return;
   if (MULTI && p.segments > 1 && tn >= p.seg[0].tile_end) {
     si = (p.segments > 2 && tn >= p.seg[1].tile_end) ? 2 : 1;
     tn -= p.seg[si - 1].tile_end;
   }
   const W4Segment& sg = p.seg[MULTI ? si : 0];
   const int n0 = tn * BN;
-  const int m0 = (tile / tiles_n) * BM;
+  const int m0 = tm * BM;
   const int nsi = n0 / 4 + i32;
   const bool n_ok = nsi < sg.ns;
 
@@ -818,6 +823,29 @@ int W4KSplit(int m, int k, int n) {
   return s;
 }
 
+// Shape of the XCD grid over the (token tile, channel tile) plane: xcd_m x (8 / xcd_m), every XCD
+// owning a rectangle of rect_m x rect_n tiles.  Picks the shape with the smallest estimate of
+// rounds of 32 tiles per XCD plus the time its L2 needs to fetch the rectangle's activation and
+// weight tiles once (activations that do not stay resident, above 2 MB, count once per round).
+int W4XcdGrid(int tiles_m, int tiles_n, int bm, int k, int groups) {
+  const double act_tile = 2.0 * bm * k, weight_tile = 64.0 * k + 256.0 * groups;  // bytes
+  const double tile_us = 2.0 * bm * 128 * k / 4.0e6;  // one CU at 4 TFLOP/s
+  int best = 8;
+  double best_us = 0;
+  for (int xm = 8; xm >= 1; xm /= 2) {
+    const int rect_m = DivUp(tiles_m, xm), rect_n = DivUp(tiles_n, 8 / xm);
+    const double rounds = rect_m * (double)rect_n / 32.0;
+    const double act_bytes = rect_m * act_tile;
+    const double refetch = act_bytes > 2.0e6 ? std::max(1.0, rounds) : 1.0;
+    const double us = rounds * tile_us + (act_bytes * refetch + rect_n * weight_tile) / 1.5e6;
+    if (xm == 8 || us < best_us) {
+      best = xm;
+      best_us = us;
+    }
+  }
+  return best;
+}
+
 template <int FM>
 hipError_t LaunchConvInt8Tile(const GemmParams& p, hipStream_t stream) {
   const int tiles = DivUp(p.n, 256) * DivUp(p.m, 2 * FM * 32);
@@ -902,17 +930,22 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
-  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : 2;
-  const int tiles = tiles_n * DivUp(a.m, fm * 32);
+  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 ? 4 : 2);
   p.ksplit = 1;
   if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) p.ksplit = std::max(1, std::atoi(e));
   for (int i = 0; i < count; ++i)
     while (p.ksplit > 1 && (size_t)p.ksplit * p.seg[i].ns * 4 * a.m > args[i].partial_floats) p.ksplit /= 2;
-  const dim3 grid(DivUp(tiles, 8) * 8, p.ksplit);
+  const int tiles_m = DivUp(a.m, fm * 32);
+  p.xcd_m = W4XcdGrid(tiles_m, tiles_n, fm * 32, a.k, p.groups);
+  if (const char* e = std::getenv("MLDHIP_GEMM_XCD_M")) p.xcd_m = std::atoi(e);
+  if (p.xcd_m != 1 && p.xcd_m != 2 && p.xcd_m != 4 && p.xcd_m != 8) p.xcd_m = 8;
+  const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
   const bool zp = p.seg[0].zp != nullptr;
   const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
-  if (fm == 2 && pair)
+  if (fm == 4 && pair)
+    LaunchDirect<4, 4, 4, true>(zp, grid, stream, p);
+  else if (fm == 2 && pair)
     LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
   else if (fm == 2)
     LaunchDirect<2, 4, 8, false>(zp, grid, stream, p);
@@ -935,6 +968,7 @@ size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n) {
   for (int m = kGemvMaxTokens + 1; m <= max_tokens; ++m) {
     const int s = W4KSplit(m, k, n);
     if (s > 1) need = std::max(need, (size_t)s * DivUp(n, 4) * 4 * m);
+    need = std::max(need, (size_t)2 * DivUp(n, 4) * 4 * m);
   }
   return need;
 }
