@@ -532,6 +532,17 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
 // it stay in flight.
 __device__ __forceinline__ void LdsBarrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// {a0 a1 a2 a3}, {b0 b1 b2 b3} -> {a0 a1 b0 b1}, {a2 a3 b2 b3}, in place.
+__device__ __forceinline__ void SwapRegisters(u32x4& a, u32x4& b) {
+  uint32_t a2 = a[2], a3 = a[3], b0 = b[0], b1 = b[1];
+  asm volatile("v_swap_b32 %0, %1" : "+v"(a2), "+v"(b0));
+  asm volatile("v_swap_b32 %0, %1" : "+v"(a3), "+v"(b1));
+  a[2] = a2;
+  a[3] = a3;
+  b[0] = b0;
+  b[1] = b1;
+}
+
 // ZP: the weights have a zero-point tensor (same shape as the scales); the centre of the codes
 // moves from 8 to 8 + zp (exact in fp16 for integral zero points).
 // PAIR (FM even, token count even): a lane's tokens for the MFMA pair (fm, fm+1) are neighbours
@@ -593,6 +604,17 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sg.w4), 0, w_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_x =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, x_end, 0x00020000);
+  // Second descriptors, one K-slice row further: the loads of rows 2q and 2q+1 share an offset.
+  // (Base and size go through readfirstlane so that the descriptors stay in scalar registers.)
+  auto uniform_ptr = [](const void* ptr, uint32_t add) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr) + add;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<void*>(((uint64_t)hi << 32) | lo);
+  };
+  const uint32_t w1_bytes = __builtin_amdgcn_readfirstlane(w_end > row_w ? w_end - row_w : 0u);
+  const uint32_t x1_bytes = __builtin_amdgcn_readfirstlane(x_end > row_x ? x_end - row_x : 0u);
+  const __amdgpu_buffer_rsrc_t rsrc_w1 = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(sg.w4, row_w), 0, w1_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_x1 = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.act, row_x), 0, x1_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_s =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(sg.scale), 0, sg.s_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_z =
@@ -603,17 +625,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // address lives there.
   const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
   uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * 8u : kOob;
-  uint32_t vw1 = n_ok ? vw0 + row_w : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
   // token of this lane in MFMA token block fm
   auto token = [&](int fm) { return PAIR ? m0 + (fm / 2) * 64 + 2 * i32 + (fm & 1) : m0 + fm * 32 + i32; };
   constexpr int NX = PAIR ? FM / 2 : FM;  // activation load items per K-slice row
-  uint32_t vx[NX][2];
+  uint32_t vx[NX];
 #pragma unroll
   for (int i = 0; i < NX; ++i) {
     const int mi = token(PAIR ? 2 * i : i);
-    vx[i][0] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
-    vx[i][1] = mi < p.m ? vx[i][0] + row_x : kOob;
+    vx[i] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
   }
   const uint32_t group_bytes = row_w;  // one scale group: [Ns][4] halfs
 
@@ -630,20 +650,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
     }
     w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
-    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw1, 0, 0);
+    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w1, vw0, 0, 0);
     vw0 += step_w;
-    vw1 += step_w;
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       if (PAIR) {
-        xp[i][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, vx[i][0], 0, 0);
-        xp[i][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, vx[i][1], 0, 0);
+        xp[i][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, vx[i], 0, 0);
+        xp[i][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_x1, vx[i], 0, 0);
       } else {
-        x[i][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[i][0], 0, 0);
-        x[i][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[i][1], 0, 0);
+        x[i][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x, vx[i], 0, 0);
+        x[i][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_x1, vx[i], 0, 0);
       }
-      vx[i][0] += step_x;
-      vx[i][1] += step_x;
+      vx[i] += step_x;
     }
   };
 
@@ -677,6 +695,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
         zp01 = AsHalf2(rzp[u & ~1][0]);
         zp23 = AsHalf2(rzp[u & ~1][1]);
       }
+      if (PAIR) {
+        // The two 16-byte loads of a token pair hold {token 2j, token 2j+1} of K-slice rows 2q
+        // and 2q+1; exchanging the inner halves makes each of them one token's operand.
+#pragma unroll
+        for (int i = 0; i < NX; ++i) {
+          SwapRegisters(rxp[u][i][0], rxp[u][i][1]);
+        }
+      }
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) {
         const half2_t sp = (t4 & 2) ? sc23 : sc01;
@@ -695,9 +721,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
-          const int h2 = 2 * (fm & 1);
-          const u32x4 bop = PAIR ? u32x4{rxp[u][fm / 2][0][h2], rxp[u][fm / 2][0][h2 + 1], rxp[u][fm / 2][1][h2],
-                                         rxp[u][fm / 2][1][h2 + 1]}
+          const u32x4 bop = PAIR ? rxp[u][fm / 2][fm & 1]
                                  : u32x4{rx[u][PAIR ? 0 : fm][0][0], rx[u][PAIR ? 0 : fm][0][1], rx[u][PAIR ? 0 : fm][1][0],
                                          rx[u][PAIR ? 0 : fm][1][1]};
           acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
@@ -943,7 +967,9 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
   const bool zp = p.seg[0].zp != nullptr;
   const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
-  if (fm == 4 && pair)
+  if (fm == 4 && pair && std::getenv("MLDHIP_GEMM_U8"))
+    LaunchDirect<4, 8, 4, true>(zp, grid, stream, p);
+  else if (fm == 4 && pair)
     LaunchDirect<4, 4, 4, true>(zp, grid, stream, p);
   else if (fm == 2 && pair)
     LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
