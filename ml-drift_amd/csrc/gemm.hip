@@ -515,8 +515,10 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
 // ------------------------------------------------------------------------------------------
 // int4 prefill GEMM without LDS in the main loop.
 //
-// Work-group = 4 waves on one output tile of 128 channels x (FM*32) tokens; the waves split K
-// four ways and add their fp32 tiles through LDS at the end (fixed order).  Inside a wave every
+// Work-group = WAVES waves on one output tile of 128 channels x (FM*32) tokens; the waves split
+// K WAVES ways and add their fp32 tiles through LDS at the end (fixed order).  Compiled shapes:
+// 32 and 64 tokens with 8 waves (two per SIMD), 128 tokens with 4 waves (one per SIMD, its 256
+// accumulators in the AGPR half of the register file).  Inside a wave every
 // MFMA operand comes straight from global memory in the layout the instruction wants:
 //  - A (weights): the 32 "rows" of MFMA number t are the output channels 4*i + t, i = lane % 32,
 //    so a lane's two 8-byte blocks (K-slices 2q, 2q+1 of slice i; 8 input channels x 4 output
@@ -831,15 +833,21 @@ __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) 
   reinterpret_cast<u32x2*>(sg.dst)[idx] = o;
 }
 
-// Token tile of the int4 GEMM: 64 when that still yields a work-group for half the CUs or M is
-// large, else 32.
+// Token tile of the int4 GEMM in blocks of 32 tokens.  64 tokens when that still yields a
+// work-group for half the CUs or M is large, else 32.  128 tokens (one wave per SIMD, every
+// dequantized weight feeds four MFMAs) when the launch fills the chip anyway and the rounds of
+// 256 work-groups come out cheaper: a 128-token tile takes about 1.85 x the time of a 64-token
+// one.
 int W4TokenBlocks(int m, int n) {
-  const long tiles64 = (long)DivUp(n, 128) * DivUp(m, 64);
+  const long tiles_n = DivUp(n, 128);
+  const long tiles64 = tiles_n * DivUp(m, 64), tiles128 = tiles_n * DivUp(m, 128);
+  if (m % 2 == 0 && tiles128 >= 256 && 1.85 * DivUp(tiles128, 256L) < (double)DivUp(tiles64, 256L)) return 4;
   return (m > 32 && (tiles64 >= 128 || m > 64)) ? 2 : 1;
 }
 // K split across work-groups: doubled while the grid stays within the CU count and every wave
 // keeps at least 4 steps of 16 channels.
 int W4KSplit(int m, int k, int n) {
+  if (W4TokenBlocks(m, n) == 4) return 1;
   const long tiles = (long)DivUp(n, 128) * DivUp(m, W4TokenBlocks(m, n) * 32);
   const int steps = DivUp(k, 16);
   int s = 1;
@@ -954,7 +962,7 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
-  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 ? 4 : 2);
+  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 && a.m % 2 == 0 ? 4 : 2);
   p.ksplit = 1;
   if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) p.ksplit = std::max(1, std::atoi(e));
@@ -967,9 +975,7 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
   const bool zp = p.seg[0].zp != nullptr;
   const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
-  if (fm == 4 && pair && std::getenv("MLDHIP_GEMM_U8"))
-    LaunchDirect<4, 8, 4, true>(zp, grid, stream, p);
-  else if (fm == 4 && pair)
+  if (fm == 4)
     LaunchDirect<4, 4, 4, true>(zp, grid, stream, p);
   else if (fm == 2 && pair)
     LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
@@ -994,7 +1000,6 @@ size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n) {
   for (int m = kGemvMaxTokens + 1; m <= max_tokens; ++m) {
     const int s = W4KSplit(m, k, n);
     if (s > 1) need = std::max(need, (size_t)s * DivUp(n, 4) * 4 * m);
-    need = std::max(need, (size_t)2 * DivUp(n, 4) * 4 * m);
   }
   return need;
 }

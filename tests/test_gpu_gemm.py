@@ -51,6 +51,19 @@ def test_w4_gemm_zero_points(oracle, m, k, n, groups):
         check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
 
 
+@pytest.mark.parametrize("m,k,n,groups,zp", [(2048, 64, 4096, 2, False), (2050, 96, 4000, 1, False),
+                                             (4096, 128, 2048, 4, True)])
+def test_w4_gemm_wide_token_tile(oracle, m, k, n, groups, zp):
+    """Launches big enough for the 128-token tile (one wave per SIMD, four MFMAs per dequantized
+    operand), with ragged token / channel edges and K ranges that end inside a wave's share."""
+    case = W.make_fc_case(seed=m + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True, with_zero_point=zp)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    sub = dict(case, m=64, act=case["act"][:64])
+    check_fp(got[:64], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement (first 64 tokens)")
+
+
 def test_config3_prefill_gemm(oracle):
     case = W.make_fc_case(**W.CONFIGS["c3"])
     got = run_w4(case)
