@@ -33,6 +33,7 @@ typedef int int16v_t __attribute__((ext_vector_type(16)));
 typedef int int4v_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float float2v_t __attribute__((ext_vector_type(2)));
 
 
 // One weight matrix of an int4 GEMM launch.  A launch covers up to kMaxW4Segments matrices
@@ -402,22 +403,19 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
         const float wsc[4] = {ws.x, ws.y, ws.z, ws.w};
         const float wz[4] = {wzp.x, wzp.y, wzp.z, wzp.w};
         const u32x2 bias2 = bias_all[fn * 4 + v4];
-        const __half bias_h[4] = {__ushort_as_half((unsigned short)(bias2[0] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[0] >> 16)),
-                                  __ushort_as_half((unsigned short)(bias2[1] & 0xFFFFu)), __ushort_as_half((unsigned short)(bias2[1] >> 16))};
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
-          __half h[4];
+          float r[4];
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            const float r = kNoOffset ? RescaleNoOffset(acc[fn][fm][v4 * 4 + c], wsc[c], src_scale[fm])
-                                      : Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp,
-                                                wz[c], src_sum[fm], in_channels);
-            h[c] = __float2half_rn(r);
-            h[c] = __hadd(h[c], bias_h[c]);
+            r[c] = kNoOffset ? RescaleNoOffset(acc[fn][fm][v4 * 4 + c], wsc[c], src_scale[fm])
+                             : Rescale(acc[fn][fm][v4 * 4 + c], wsc[c], wsum[c], src_scale[fm], src_zp[fm], has_zp,
+                                       wz[c], src_sum[fm], in_channels);
           }
+          // two results per conversion (round to nearest even) and per bias add
           u32x2 o;
-          o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
-          o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+          o[0] = AsU32(__builtin_convertvector(float2v_t{r[0], r[1]}, half2_t) + AsHalf2(bias2[0]));
+          o[1] = AsU32(__builtin_convertvector(float2v_t{r[2], r[3]}, half2_t) + AsHalf2(bias2[1]));
           const int token_l = (wm * FM + fm) * 32 + r32;
           reinterpret_cast<u32x2*>(smem)[slice_l * BM + token_l] = o;
         }
