@@ -1025,6 +1025,12 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
   if (kernel_name) *kernel_name = "conv_int8_mfma_kernel";
   // token tile: the largest of 256 / 128 / 64 that still gives most CUs a work-group
   auto tiles = [&](int bm) { return (long)DivUp(p.n, 256) * DivUp(p.m, bm); };
+  if (const char* e = std::getenv("MLDHIP_GEMM_I8_FM")) {  // tuning override: token tile in blocks of 64
+    const int fm = std::atoi(e);
+    if (fm == 4) return LaunchConvInt8Tile<4>(p, stream);
+    if (fm == 2) return LaunchConvInt8Tile<2>(p, stream);
+    if (fm == 1) return LaunchConvInt8Tile<1>(p, stream);
+  }
   if (tiles(256) >= 200) return LaunchConvInt8Tile<4>(p, stream);
   if (tiles(128) >= 200) return LaunchConvInt8Tile<2>(p, stream);
   return LaunchConvInt8Tile<1>(p, stream);
