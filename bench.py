@@ -34,7 +34,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=None, help="default 4000 (c2), 200 (c3, c4), 20 (c5-*)")
     p.add_argument("--warmup", type=int, default=None, help="default steps / 10")
-    p.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5-decode", "c5-prefill"],
+    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2"],
                    help="c2 (default) is the headline line; the others time the remaining configurations "
                         "the same way (one JSON line each, no CPU baseline)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
@@ -46,7 +46,7 @@ def parse():
                         "reference dispatch) followed by 64 launches over the weight ring, then exit")
     a = p.parse_args()
     if a.steps is None:
-        a.steps = {"c2": 4000, "c3": 200, "c4": 200}.get(a.workload, 20)
+        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "c3": 200, "c4": 200}.get(a.workload, 20)
     if a.warmup is None:
         a.warmup = max(1, a.steps // 10)
     return a
@@ -84,7 +84,55 @@ def run_other(args, torch, M, W):
     stream = torch.cuda.Stream()
     base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic"}
-    if args.workload == "c3":
+    if args.workload in ("c1", "f2"):
+        # decode GEMVs over a ring of weight copies larger than the 256 MB cache
+        if args.workload == "c1":
+            case = W.make_fc_case(**W.CONFIGS["c1"])
+            dev0 = W.FcDevice(case)
+            m, k, n = case["m"], case["k"], case["n"]
+            ring = max(args.ring, 80)  # 80 x 4.2 MB
+            gen = torch.Generator(device="cuda").manual_seed(1)
+            ops, keep = [dev0.op], [dev0]
+            for r in range(1, ring):
+                wt = torch.randint(0, 256, dev0.weights.shape, dtype=torch.uint8, device="cuda", generator=gen)
+                op = M.fc_create(M.PRECISION_F32, M.FLOAT32, M.FLOAT32, n, k, dev0.desc, scale_shape=(n, 1), max_tokens=m)
+                op.bind([dev0.act, wt, dev0.scale], [dev0.out])
+                op.set_shape(1, 1, m)
+                ops.append(op)
+                keep.append(wt)
+            nbytes = n * k + k * 4 + n * 4 + n * 4  # W + act + scale + out (fp32 tensors)
+            label = "c1: FullyConnected decode GEMV M=1 K=2048 N=2048 int8 per-channel, fp32 act/out"
+            metric, dtype = "int8_decode_gemv_hbm_bandwidth", "u8 weights x f32 activations, f32 accumulate"
+        else:
+            m, k, n = 1, 4096, 14336
+            rng = np.random.default_rng(0)
+            w = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+            src = rng.integers(-128, 128, size=(m, k), dtype=np.int8)
+            desc = M.fc_int4_weights_desc(n, k)
+            packed = torch.from_numpy(M.rearrange_int8_as_uint4(w, desc))
+            act = torch.from_numpy(W.to_slices(src)).cuda()
+            out_t = torch.zeros(((n + 3) // 4, m, 4), dtype=torch.int32, device="cuda")
+            ring = args.ring
+            ops, keep = [], []
+            for r in range(ring):
+                wt = packed.cuda() if r == 0 else torch.randint(0, 256, packed.shape, dtype=torch.uint8, device="cuda")
+                op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=m)
+                op.bind([act, wt], [out_t])
+                op.set_shape(1, 1, m)
+                ops.append(op)
+                keep.append(wt)
+            nbytes = n * k // 2 + k + n * 4  # W + int8 act + int32 out
+            label = "f2: int8-math FullyConnected decode GEMV M=1 K=4096 N=14336, int8 act x uint4 weights -> int32"
+            metric, dtype = "int8_math_decode_gemv_hbm_bandwidth", "i8 x u4, i32 accumulate (v_dot4)"
+        wall, ev_ms = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup)
+        us = ev_ms * 1e3 / args.steps
+        out = dict(base, metric=metric, value=round(nbytes * args.steps / wall / 1e9, 1), unit="GB/s",
+                   ms_per_step=round(wall * 1e3 / args.steps, 6), dtype=dtype,
+                   config={"workload": label, "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes},
+                   roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "traffic": None, "avg_launch_us": round(us, 3)})
+    elif args.workload == "c3":
         case = W.make_fc_case(**W.CONFIGS["c3"])
         dev = W.FcDevice(case)
         wall, ev_ms = time_graph(torch, stream, lambda s, i: dev.op.launch(s), args.steps, args.warmup)

@@ -557,9 +557,16 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
   if (op->kind == mldhip_op::kFc) {
     const mldhip_fc_desc& d = op->fc;
     if (d.src_type == MLDHIP_INT8) {
-      e = LaunchFcInt8Math(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
-                           static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o,
-                           WeightBits(d.weights.type), stream, &op->last_kernel);
+      const int bits = WeightBits(d.weights.type);
+      if (!EnvFlag("MLDHIP_FORCE_GENERIC") && FcInt8MathStreamSupported(op->Tokens(), d.i, d.o, bits)) {
+        e = LaunchFcInt8MathStream(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
+                                   static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o, bits, stream,
+                                   &op->last_kernel);
+      } else {
+        e = LaunchFcInt8Math(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
+                             static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o, bits, stream,
+                             &op->last_kernel);
+      }
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;

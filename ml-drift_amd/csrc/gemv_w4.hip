@@ -182,6 +182,16 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
 #pragma unroll
     for (int o = 0; o < 8; ++o) acc[m][o] = 0.0f;
 
+  // The per-channel scale and the bias of the output this thread writes at the end (output
+  // tid % STRIP of the strip, for every token it handles): fetched now, so that their latency
+  // does not follow the reduction.
+  // (Unconditional loads of the raw halfs at a clamped index: a branch, or a conversion, here
+  // would make the kernel wait for them before it issues the weight loads.)
+  const int n_out = min(strip * STRIP + tid % STRIP, sg.n_pad - 1);
+  const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(sg.bias ? sg.bias : sg.scale);
+  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(sg.scale)[n_out];
+  const unsigned short out_bias_raw = bias_src[n_out];
+
   int c = c_begin + row;
   u32x4 zv = {0u, 0u, 0u, 0u};  // zero points of this thread's 8 channels (halfs)
   if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(sg.zero_point + (size_t)2 * pcol * 4);
@@ -268,8 +278,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
     if (p.ksplit == 1) {
-      if (!GROUPED) v *= __half2float(sg.scale[n]);
-      StoreHalf(sg.dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, sg.bias, (size_t)n);
+      if (!GROUPED) v *= __half2float(__ushort_as_half(out_scale_raw));
+      __half h = __float2half_rn(v);
+      if (sg.bias) h = __hadd(h, __ushort_as_half(out_bias_raw));
+      sg.dst[((size_t)(n >> 2) * M + m) * 4 + (n & 3)] = h;
     } else {
       p.partial[((size_t)ky * M + m) * sg.n_pad + n] = v;
     }

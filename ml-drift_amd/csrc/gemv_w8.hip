@@ -111,8 +111,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
       const int ks = c * 8 + j;
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        Load4(act, ((size_t)min(ks, p.ks - 1) * M + m) * 4, a[j][m]);
-        if (ks >= p.ks) a[j][m][0] = a[j][m][1] = a[j][m][2] = a[j][m][3] = 0.0f;
+        // unconditional load at a clamped row, zeroed by selects: a branch here would make every
+        // wait of the chunk a wait for all loads
+        float v[4];
+        Load4(act, ((size_t)min(ks, p.ks - 1) * M + m) * 4, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[j][m][i] = ks < p.ks ? v[i] : 0.0f;
       }
     }
   };

@@ -51,6 +51,10 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
 // int8 activations x uint8/uint4 weights -> int32 (no scales).
 hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k,
                             int n, int weight_bits, hipStream_t stream, const char** kernel_name);
+// The same for 1..4 tokens as an HBM-streaming kernel.
+bool FcInt8MathStreamSupported(int m, int k, int n, int weight_bits);
+hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k, int n,
+                                  int weight_bits, hipStream_t stream, const char** kernel_name);
 
 struct QuantArgs {
   const void* src = nullptr;

@@ -223,7 +223,8 @@ def test_known_answers_on_gpu():
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("m,k,n", [(1, 112, 152), (5, 171, 533), (1, 2048, 2048), (16, 4096, 1024)])
+@pytest.mark.parametrize("m,k,n", [(1, 112, 152), (5, 171, 533), (1, 2048, 2048), (16, 4096, 1024),
+                                   (2, 171, 533), (3, 100, 8), (4, 1000, 4104), (1, 4096, 14336), (1, 36, 20)])
 def test_int8_math_bit_exact(oracle, bits, m, k, n):
     """int8 activations x packed weights -> int32, exact (fully_connected_test_util.cc:1446-1448)."""
     torch = torch_cuda()
@@ -245,6 +246,9 @@ def test_int8_math_bit_exact(oracle, bits, m, k, n):
     got = W.from_slices(out.cpu().numpy(), n)
     ref = oracle.fc_reference_i8(src, w)
     assert np.array_equal(got, ref)
+    # 1..4 tokens stream (uint4 rows with an odd number of slices keep the tiled kernel)
+    streams = m <= 4 and (bits == 8 or ((n + 3) // 4) % 2 == 0)
+    assert op.kernel_name == ("fc_i8math_stream_kernel" if streams else "fc_int8_math_kernel"), op.kernel_name
     if m * k * n <= 1 << 24:
         mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed, m, k, n, bits), n)
         assert np.array_equal(got, mimic)
