@@ -152,6 +152,53 @@ int mldhip_scale_to_tensor(const float* scale, int o, int groups, int dst_type, 
                            size_t dst_bytes);
 
 /* ------------------------------------------------------------------------------------ */
+/* Checkpoint files -> the buffers of a quantized FullyConnected (host side)              */
+/* ------------------------------------------------------------------------------------ */
+
+/* One linear layer as the LLM sample stores it on disk (samples/llm/extract_weights_hf.py writes
+ * these files, samples/llm/llm_file_tensor_loader.cc reads them): `<weights_name>` holds int8
+ * [o][i] values, or two's-complement nibbles with the low nibble first;
+ * `<base_name>.weight_quantized_scale` holds fp32 scales [o] or [o][i / group] (or an int32
+ * group-size header followed by int8 / int16 values of scale * 1024);
+ * `<base_name>.weight_quantized_zp`, if present, holds zero points in the same two formats,
+ * in units of the dequantized weight.  File names are appended to `directory` as they are
+ * (the directory string ends in a separator, as in the reference). */
+typedef struct {
+  mldhip_weights_desc weights; /* GetFullyConnectedInt4WeightsDesc / ...Int8WeightsDesc of (o, i) */
+  int o, i;
+  int weight_bits;             /* 4 or 8 */
+  int group_size;              /* input channels per scale; i for per-channel scales */
+  int scale_i;                 /* i / group_size: the scale / zero-point shape is OHWI(o, 1, 1, scale_i) */
+  int has_zero_point;          /* the zero-point file exists */
+  size_t weights_bytes;        /* bytes of the packed weight buffer */
+  size_t scale_elements;       /* elements of the scale (and zero-point) tensor: scale_i * ceil(o/4) * 4 */
+} mldhip_checkpoint_fc;
+
+/* What LlmWeightsLoader::GetWeightsInt4 / GetWeightsInt8 (samples/llm/llm_weights_loader.cc:29-117)
+ * find out before they load: the weights description, the quantization group size
+ * (LlmFileTensorLoader::GetQuantizationIGroupSize, llm_file_tensor_loader.cc:399-452: derived
+ * from the size of the scale file; a missing or unrecognised file means per-channel) and
+ * whether a zero-point file exists.  MLDHIP_NOT_FOUND when the weights file cannot be opened. */
+int mldhip_checkpoint_fc_probe(const char* directory, const char* weights_name,
+                               const char* base_name, int o, int i, int weight_bits,
+                               mldhip_checkpoint_fc* info);
+
+/* LoadInt4Weights (fast path, llm_file_tensor_loader.cc:350-395) / LoadInt8Weights (:262-302),
+ * LoadScale (:454-467) and LoadZeroPoint (:469-496) into caller-provided host buffers, ready to
+ * upload and bind as "weights", "weights_scale", "weights_zero_point" (and the weights_sum_i of
+ * the int8 x int8 route): packed weights in info->weights layout, scale and zero-point tensors
+ * of ScaleOrZeroPointToTensorDesc in `tensor_type` (FLOAT16 / FLOAT32), zero point = file value
+ * / scale (0 where the scale is 0), weights_sum_i[o] int32.  `swap_dims`: the weights file is
+ * [i][o].  `zero_point` may be null when info->has_zero_point is 0; `scale_bytes` is the size of
+ * each of the two tensor buffers.  As in the reference, a file shorter than the shape reads as
+ * zeros beyond its end. */
+int mldhip_checkpoint_fc_read(const char* directory, const char* weights_name,
+                              const char* base_name, const mldhip_checkpoint_fc* info,
+                              int swap_dims, int tensor_type, uint8_t* weights,
+                              size_t weights_bytes, void* scale, void* zero_point,
+                              size_t scale_bytes, int32_t* weights_sum_i);
+
+/* ------------------------------------------------------------------------------------ */
 /* Operations (node executors)                                                            */
 /* ------------------------------------------------------------------------------------ */
 

@@ -16,13 +16,19 @@
 using namespace mldhip;
 
 namespace {
-
 thread_local std::string g_error;
+}  // namespace
 
+namespace mldhip {
+// Records the calling thread's error message (mldhip_last_error) and returns `code`.
 int Fail(int code, const std::string& msg) {
   g_error = msg;
   return code;
 }
+}  // namespace mldhip
+
+namespace {
+using mldhip::Fail;
 
 int HipFail(hipError_t e, const char* what) {
   return Fail(MLDHIP_INTERNAL, std::string(what) + ": " + hipGetErrorString(e));

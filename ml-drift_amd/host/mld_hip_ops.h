@@ -197,6 +197,45 @@ inline Status AddToQueueFused(const std::vector<HipOperation*>& ops, void* hip_s
   return Status::FromCode(mldhip_fc_launch_fused(handles.data(), (int)handles.size(), hip_stream));
 }
 
+// One linear layer read from the LLM sample's checkpoint files, as host buffers ready to upload:
+// what LlmWeightsLoader::GetWeightsInt4 / GetWeightsInt8 (samples/llm/llm_weights_loader.cc:29-117)
+// assemble through LlmFileTensorLoader.  `weights` carries the description and shapes that
+// CreateFullyConnectedExternalWeights takes; the tensors are in the activation type.
+struct LoadedFcWeights {
+  ExternalWeights weights;
+  int quantization_i_group_size = 0;
+  std::vector<uint8_t> packed;          // "weights"
+  std::vector<uint8_t> scale;           // "weights_scale", tensor bytes
+  std::vector<uint8_t> zero_point;      // "weights_zero_point", empty without a zero-point file
+  std::vector<int32_t> weights_sum_i;   // for the int8 x int8 route
+};
+
+inline Status LoadFcWeights(const std::string& weights_directory, const std::string& w_name,
+                            const std::string& base_name, const OHWI& weights_shape, int weight_bits, bool swap_dims,
+                            DataType tensor_type, LoadedFcWeights* out) {
+  mldhip_checkpoint_fc info;
+  int rc = mldhip_checkpoint_fc_probe(weights_directory.c_str(), w_name.c_str(), base_name.c_str(), weights_shape.o,
+                                      weights_shape.i, weight_bits, &info);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  const size_t elem = tensor_type == DataType::kFloat16 ? 2 : 4;
+  out->packed.assign(info.weights_bytes, 0);
+  out->scale.assign(info.scale_elements * elem, 0);
+  out->zero_point.assign(info.has_zero_point ? info.scale_elements * elem : 0, 0);
+  out->weights_sum_i.assign(weights_shape.o, 0);
+  rc = mldhip_checkpoint_fc_read(weights_directory.c_str(), w_name.c_str(), base_name.c_str(), &info, swap_dims ? 1 : 0,
+                                 (int)tensor_type, out->packed.data(), out->packed.size(), out->scale.data(),
+                                 info.has_zero_point ? out->zero_point.data() : nullptr, out->scale.size(),
+                                 out->weights_sum_i.data());
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  out->quantization_i_group_size = info.group_size;
+  out->weights.desc = info.weights;
+  out->weights.shape = weights_shape;
+  out->weights.scale_zp_shape = OHWI{weights_shape.o, 1, 1, info.scale_i};
+  out->weights.has_scale_tensor = true;
+  out->weights.has_zero_point_tensor = info.has_zero_point != 0;
+  return Status{};
+}
+
 // One graph node: operation + the ids of its inputs/outputs in the caller's tensor table,
 // in the reference's order (common/gpu_model.h:38-60).
 struct GpuNode {

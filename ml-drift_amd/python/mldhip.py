@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libmldhip.so")
 
 OK, INVALID_ARGUMENT, FAILED_PRECONDITION, OUT_OF_RANGE, UNIMPLEMENTED, INTERNAL = 0, 3, 9, 11, 12, 13
+NOT_FOUND = 5
 FLOAT16, FLOAT32, UINT8, INT8, INT32, UINT4 = 1, 2, 5, 6, 10, 15
 PACKED_UINT8C4, PACKED_INT8C4, PACKED_INT8C16, PACKED_UINT8C16 = 1, 2, 5, 6
 LAYOUT_UNKNOWN, LAYOUT_I4O4, LAYOUT_O4I4, LAYOUT_2D_I4O4, LAYOUT_CUSTOM = 0, 1, 2, 6, 7
@@ -29,6 +30,7 @@ SYMBOLS = [
     "mldhip_op_src_count", "mldhip_op_dst_count", "mldhip_op_src_name", "mldhip_op_dst_name",
     "mldhip_op_set_src", "mldhip_op_set_dst", "mldhip_op_set_shape", "mldhip_op_launch",
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
+    "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read",
 ]
 
 
@@ -56,6 +58,12 @@ class ConvInt8Desc(C.Structure):
     _fields_ = [("src_packed_type", C.c_int32), ("dst_type", C.c_int32), ("o", C.c_int32),
                 ("i", C.c_int32), ("weights", WeightsDesc), ("has_zero_point", C.c_int32),
                 ("has_bias", C.c_int32), ("max_tokens", C.c_int32)]
+
+
+class CheckpointFc(C.Structure):
+    _fields_ = [("weights", WeightsDesc), ("o", C.c_int32), ("i", C.c_int32), ("weight_bits", C.c_int32),
+                ("group_size", C.c_int32), ("scale_i", C.c_int32), ("has_zero_point", C.c_int32),
+                ("weights_bytes", C.c_size_t), ("scale_elements", C.c_size_t)]
 
 
 class MldhipError(RuntimeError):
@@ -217,6 +225,30 @@ def scale_to_tensor(scale, dst_type):
     out = np.empty(groups * div_up(o, 4) * 4, dt)
     check(lib().mldhip_scale_to_tensor(_p(s), o, groups, dst_type, _p(out), C.c_size_t(out.nbytes)))
     return out
+
+
+# ---- checkpoint files (host) ----
+def checkpoint_fc_probe(directory, weights_name, base_name, o, i, weight_bits):
+    """-> CheckpointFc (weights description, group size, zero-point presence, buffer sizes)."""
+    info = CheckpointFc()
+    check(lib().mldhip_checkpoint_fc_probe(directory.encode(), weights_name.encode(), base_name.encode(),
+                                           o, i, weight_bits, C.byref(info)))
+    return info
+
+
+def checkpoint_fc_read(directory, weights_name, base_name, info, tensor_type, swap_dims=False):
+    """-> dict(weights=uint8 buffer, scale=tensor buffer, zero_point=tensor buffer or None,
+    weights_sum_i=int32[o])."""
+    dt = np.uint16 if tensor_type == FLOAT16 else np.float32
+    weights = np.empty(info.weights_bytes, np.uint8)
+    scale = np.empty(info.scale_elements, dt)
+    zp = np.empty(info.scale_elements, dt) if info.has_zero_point else None
+    sums = np.empty(info.o, np.int32)
+    check(lib().mldhip_checkpoint_fc_read(directory.encode(), weights_name.encode(), base_name.encode(),
+                                          C.byref(info), int(bool(swap_dims)), tensor_type, _p(weights),
+                                          C.c_size_t(weights.nbytes), _p(scale),
+                                          _p(zp) if zp is not None else None, C.c_size_t(scale.nbytes), _p(sums)))
+    return dict(weights=weights, scale=scale, zero_point=zp, weights_sum_i=sums)
 
 
 # ---- ops ----

@@ -3,6 +3,10 @@
 #include <cstdio>
 #include <cstring>
 
+#include <cstdlib>
+#include <cstdio>
+#include <string>
+
 #include "../ml-drift_amd/host/mld_hip_ops.h"
 
 using namespace mld_hip;
@@ -72,6 +76,37 @@ int main() {
                                           false, 2048, &conv)
              .ok());
   EXPECT(conv.GetSrcTensorsNames().size() == 5 && conv.GetSrcTensorsNames()[2] == "params_tensor");
+
+  // A layer from checkpoint files (samples/llm/llm_weights_loader.cc:29-71): int4 [4][8] with
+  // nibbles 0..7 per row pattern, two scale groups of 4 input channels, written here by hand.
+  {
+    const char* tmp = std::getenv("TMPDIR");
+    const std::string dir = std::string(tmp ? tmp : "/tmp") + "/";
+    const std::string base = "mldhip_adapter_layer";
+    std::vector<uint8_t> nib(4 * 8 / 2);
+    for (int e = 0; e < 32; e += 2) nib[e / 2] = (uint8_t)(((e % 8) & 15) | ((((e + 1) % 8) - 8) & 15) << 4);
+    std::vector<float> sc(4 * 2);
+    for (int k = 0; k < 8; ++k) sc[k] = 0.5f + 0.25f * k;
+    FILE* f = std::fopen((dir + base + ".weight").c_str(), "wb");
+    EXPECT(f && std::fwrite(nib.data(), 1, nib.size(), f) == nib.size());
+    std::fclose(f);
+    f = std::fopen((dir + base + ".weight_quantized_scale").c_str(), "wb");
+    EXPECT(f && std::fwrite(sc.data(), 4, sc.size(), f) == sc.size());
+    std::fclose(f);
+    LoadedFcWeights lw;
+    EXPECT(LoadFcWeights(dir, base + ".weight", base, OHWI{4, 1, 1, 8}, 4, false, DataType::kFloat32, &lw).ok());
+    EXPECT(lw.quantization_i_group_size == 4 && lw.weights.scale_zp_shape.i == 2 && !lw.weights.has_zero_point_tensor);
+    EXPECT(lw.packed.size() == 16 && lw.scale.size() == 2 * 4 * 4 && lw.zero_point.empty());
+    // row sums: elements e, e+1 of a row are (e % 8) and ((e+1) % 8) - 8: 0-7+2-5+4-3+6-1 = -4
+    EXPECT(lw.weights_sum_i[0] == -4 && lw.weights_sum_i[3] == -4);
+    // scale tensor [group][slice][4]: group 0 holds sc[o*2 + 0]
+    const float* st32 = reinterpret_cast<const float*>(lw.scale.data());
+    EXPECT(st32[0] == sc[0] && st32[1] == sc[2] && st32[4] == sc[1] && st32[7] == sc[7]);
+    EXPECT(LoadFcWeights(dir, "no_such_file", base, OHWI{4, 1, 1, 8}, 4, false, DataType::kFloat32, &lw).code ==
+           MLDHIP_NOT_FOUND);
+    std::remove((dir + base + ".weight").c_str());
+    std::remove((dir + base + ".weight_quantized_scale").c_str());
+  }
   std::printf("host adapter ok\n");
   return 0;
 }
