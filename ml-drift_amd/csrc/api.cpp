@@ -577,7 +577,11 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
       const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
-      if (!force_generic && FcW4StreamSupported(a)) {
+      // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
+      // on the vector-ALU kernel; MLDHIP_GEMV_MFMA=1 forces the matrix-core one there too)
+      if (!force_generic && (a.m >= 2 || EnvFlag("MLDHIP_GEMV_MFMA")) && FcW4MfmaStreamSupported(a)) {
+        e = LaunchFcW4MfmaStream(a, stream, &op->last_kernel);
+      } else if (!force_generic && FcW4StreamSupported(a)) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4MfmaSupported(a)) {
         e = LaunchFcW4Mfma(a, stream, &op->last_kernel);

@@ -45,6 +45,10 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 
 // Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
+// The same for 1..16 tokens on the matrix cores (per-channel scales, wide layers).
+bool FcW4MfmaStreamSupported(const FcArgs& a);
+hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+
 bool FcW8StreamSupported(const FcArgs& a);
 hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 

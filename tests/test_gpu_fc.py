@@ -222,6 +222,26 @@ def test_known_answers_on_gpu():
         assert np.allclose(dev.result(), np.full((1, 4), 8.0), atol=eps)
 
 
+@pytest.mark.parametrize("m,k,n,zp,bias", [(2, 4096, 14336, False, False), (16, 4096, 8192, True, True),
+                                            (3, 1000, 8200, False, True), (7, 171, 8200, True, False),
+                                            (5, 4104, 8228, False, False), (9, 16384, 8192, False, False)])
+def test_w4_mfma_stream_kernel(oracle, m, k, n, zp, bias):
+    """2..16 tokens on wide per-channel int4 layers run on the matrix-core GEMV: ragged K (the last
+    step, the last wave's share), ragged N, zero points, more than one chunk of steps per wave."""
+    case = W.make_fc_case(seed=m + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=1,
+                          with_zero_point=zp, with_bias=bias)
+    print("w4 mfma stream", m, k, n, zp, bias, flush=True)
+    dev = W.FcDevice(case)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_mfma_stream_kernel", dev.op.kernel_name
+    check_fp(got, textbook(case), case, "textbook")
+    if m * k * n <= 1 << 26:
+        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+    dev.run()
+    assert np.array_equal(got, dev.result())
+
+
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("m,k,n", [(1, 112, 152), (5, 171, 533), (1, 2048, 2048), (16, 4096, 1024),
                                    (2, 171, 533), (3, 100, 8), (4, 1000, 4104), (1, 4096, 14336), (1, 36, 20)])
