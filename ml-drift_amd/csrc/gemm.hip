@@ -832,7 +832,7 @@ __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) 
 }
 
 // Token tile of the int4 GEMM in blocks of 32 tokens.  64 tokens when that still yields a
-// work-group for half the CUs or M is large, else 32.  128 tokens (one wave per SIMD, every
+// work-group for half the CUs, else 32 (more work-groups beat a K split across them).  128 tokens (one wave per SIMD, every
 // dequantized weight feeds four MFMAs) when the launch fills the chip anyway and the rounds of
 // 256 work-groups come out cheaper: a 128-token tile takes about 1.85 x the time of a 64-token
 // one.
@@ -840,16 +840,17 @@ int W4TokenBlocks(int m, int n) {
   const long tiles_n = DivUp(n, 128);
   const long tiles64 = tiles_n * DivUp(m, 64), tiles128 = tiles_n * DivUp(m, 128);
   if (m % 2 == 0 && tiles128 >= 256 && 1.85 * DivUp(tiles128, 256L) < (double)DivUp(tiles64, 256L)) return 4;
-  return (m > 32 && (tiles64 >= 128 || m > 64)) ? 2 : 1;
+  return (m > 32 && tiles64 >= 128) ? 2 : 1;
 }
 // K split across work-groups: doubled while the grid stays within the CU count and every wave
-// keeps at least 4 steps of 16 channels.
+// keeps at least 24 steps of 16 channels (below that the partial sums and the second kernel
+// cost more than the idle CUs: 2048 x 2048 at 128 tokens 10.9 -> 8.5 us without a split).
 int W4KSplit(int m, int k, int n) {
   if (W4TokenBlocks(m, n) == 4) return 1;
   const long tiles = (long)DivUp(n, 128) * DivUp(m, W4TokenBlocks(m, n) * 32);
   const int steps = DivUp(k, 16);
   int s = 1;
-  while (s < 8 && tiles * s * 2 <= 256 && steps / (8 * s * 2) >= 4) s *= 2;
+  while (s < 8 && tiles * s * 2 <= 256 && steps / (8 * s * 2) >= 24) s *= 2;
   return s;
 }
 
