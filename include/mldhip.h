@@ -324,6 +324,20 @@ int mldhip_op_launch(mldhip_op* op, void* stream);
  * launches nothing) when the ops cannot share a launch; the caller then launches them singly. */
 int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream);
 
+/* The MLP step after the gate and up projections of a decoder layer,
+ * dst = activation(gate(x)) * up(x), in the same launch as the two projections
+ * (samples/llm/gemma3_model_builder.cc:1054-1090 CreateGeluTanhMulOp over the two Linear nodes of
+ * :1141-1147; samples/llm/qwen3_model_builder.cc:850-883 CreateSiluMulOp).  `gate` and `up` are
+ * FullyConnected ops bound to the same src_tensor with the same shape; their results are rounded
+ * to fp16 (+ biases) as the two nodes would store them and combined in fp32 in the operation
+ * order of the sample's elementwise kernel; their own dst tensors are not written.  dst:
+ * [ceil(o/4)][tokens][4] halfs.  Served for int4 weights, fp16 tensors, symmetric, 1..2 tokens;
+ * MLDHIP_FAILED_PRECONDITION otherwise: launch the two ops (mldhip_fc_launch_fused) and the
+ * host framework's elementwise node instead. */
+enum { MLDHIP_GATE_GELU_TANH = 1, MLDHIP_GATE_SILU = 2 };
+int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void* dst,
+                           size_t dst_bytes, void* stream);
+
 /* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
  * at the current shape (GPUOperation::flops_/read_size_/write_size_,
  * common/task/gpu_operation.h:190-195). */

@@ -657,6 +657,33 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
   return MLDHIP_OK;
 }
 
+int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void* dst, size_t dst_bytes,
+                           void* stream_ptr) {
+  if (!gate || !up || !dst) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
+  if (activation != MLDHIP_GATE_GELU_TANH && activation != MLDHIP_GATE_SILU)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "unknown gate activation");
+  mldhip_op* ops[2] = {gate, up};
+  FcArgs args[2];
+  for (int i = 0; i < 2; ++i) {
+    if (ops[i]->kind != mldhip_op::kFc || ops[i]->fc.src_type == MLDHIP_INT8)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "gated launch takes floating-point FullyConnected ops");
+    if (int rc = CheckBindings(ops[i])) return rc;
+    if (int rc = BuildFcArgs(ops[i], &args[i])) return rc;
+  }
+  if (!FcW4GatedSupported(args[0], args[1]))
+    return Fail(MLDHIP_FAILED_PRECONDITION,
+                "gate and up are not a pair of int4 fp16 FullyConnected ops over one tensor with one shape, "
+                "symmetric weights and at most 2 tokens");
+  const size_t need = (size_t)DivUp(args[0].n, 4) * 4 * args[0].m * sizeof(uint16_t);
+  if (dst_bytes < need) return Fail(MLDHIP_INVALID_ARGUMENT, "dst is too small for the gated output");
+  const char* name = nullptr;
+  hipError_t e = LaunchFcW4Gated(args[0], args[1], activation, dst,
+                                 static_cast<hipStream_t>(stream_ptr), &name);
+  if (e != hipSuccess) return HipFail(e, "gated launch");
+  gate->last_kernel = up->last_kernel = name;
+  return MLDHIP_OK;
+}
+
 const char* mldhip_op_kernel_name(const mldhip_op* op) { return op ? op->last_kernel : ""; }
 
 int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {

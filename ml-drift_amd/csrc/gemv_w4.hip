@@ -27,6 +27,7 @@
 
 #include <cstdlib>
 
+#include "../../include/mldhip.h"
 #include "kernels.h"
 
 namespace mldhip {
@@ -301,6 +302,169 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
   StoreHalf(sg.dst, ((size_t)(n >> 2) * p.m + m) * 4 + (n & 3), v, sg.bias, (size_t)n);
 }
 
+// ------------------------------------------------------------------------------------------
+// Gated pair: dst = activation(gate(x)) * up(x), the MLP step that follows the gate and up
+// projections in the decoder layers of the LLM sample (samples/llm/gemma3_model_builder.cc:
+// 1054-1090 CreateGeluTanhMulOp, samples/llm/qwen3_model_builder.cc:850-883 CreateSiluMulOp).
+// The two projections run as in the kernel above, in one work-group per strip (seg[0] = gate,
+// seg[1] = up, same shape); their sums are rounded to fp16 (+ bias) exactly as the two separate
+// FullyConnected nodes would store them, then combined in fp32 in the operation order of the
+// sample's elementwise kernel.  Only seg[0].dst is written.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float GatedActivation(int act, float g, float u) {
+  if (act == MLDHIP_GATE_GELU_TANH) {
+    const float gate_sq = g * g;
+    const float tanh_in = g * (0.7978845608f + 0.03567740813f * gate_sq);
+    const float clamped = fminf(fmaxf(tanh_in, -10.0f), 10.0f);
+    const float tanh_val = tanhf(clamped);
+    const float gate_up_half = 0.5f * g * u;
+    return fminf(fmaxf(gate_up_half * (1.0f + tanh_val), -65504.0f), 65504.0f);
+  }
+  const float sig = 1.0f / (1.0f + expf(-g));
+  const float silu = g * sig;
+  return fminf(fmaxf(silu * u, -65504.0f), 65504.0f);
+}
+
+template <int LPR, int WAVES, int M, bool GROUPED>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_gated_stream_kernel(StreamParams p, int activation) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int ROWS = THREADS / LPR;
+  constexpr int RPW = 64 / LPR;
+  constexpr int STRIP = LPR * 8;
+  constexpr int PARTS = THREADS / STRIP > ROWS ? ROWS : THREADS / STRIP;
+  constexpr int RPP = ROWS / PARTS;
+  __shared__ float red[ROWS][2 * M][STRIP];
+  __shared__ float red2[PARTS][2 * M][STRIP];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane % LPR;
+  const int row = wave * RPW + lane / LPR;
+  const int strip = blockIdx.x;
+  const int row_u4 = p.seg[0].row_u4;
+  const int pcol_raw = strip * LPR + col;
+  const int pcol = pcol_raw < row_u4 ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
+
+  // scales / biases of the output this thread finishes, fetched ahead (raw halfs, clamped index)
+  const int n_out = min(strip * STRIP + tid % STRIP, p.seg[0].n_pad - 1);
+  unsigned short scale_raw[2], bias_raw[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(p.seg[q].bias ? p.seg[q].bias : p.seg[q].scale);
+    scale_raw[q] = reinterpret_cast<const unsigned short*>(p.seg[q].scale)[n_out];
+    bias_raw[q] = bias_src[n_out];
+  }
+
+  float acc[2][M][8];
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int m = 0; m < M; ++m)
+#pragma unroll
+      for (int o = 0; o < 8; ++o) acc[q][m][o] = 0.0f;
+
+  for (int c = row; c < p.chunks; c += ROWS) {
+    u32x4 w[2][8];
+    u32x2 a[8][M];
+    LoadChunk<M>(p, p.seg[0].weights, row_u4, c, pcol, w[0], a);
+    {
+      const int ks0 = c * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        w[1][j] = __builtin_nontemporal_load(p.seg[1].weights + (size_t)min(ks0 + j, p.ks - 1) * row_u4 + pcol);
+    }
+    u32x4 sv[2];
+    if (GROUPED) {
+      int g = c / p.group_chunks;
+      if (g >= p.groups) g = p.groups - 1;
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+        sv[q] = *reinterpret_cast<const u32x4*>(p.seg[q].scale + ((size_t)g * p.seg[q].ns + 2 * pcol) * 4);
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      float t[M][8], asum[M];
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        asum[m] = 0.0f;
+#pragma unroll
+        for (int o = 0; o < 8; ++o) t[m][o] = 0.0f;
+      }
+      ComputeChunk<M>(p, w[q], a, t, asum);
+#pragma unroll
+      for (int m = 0; m < M; ++m)
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+          const float centered = fmaf((o & 1) ? -72.0f : -1032.0f, asum[m], t[m][o]);
+          if (GROUPED) {
+            const half2_t sp = AsHalf2(sv[q][o >> 1]);
+            acc[q][m][o] = fmaf((float)sp[o & 1], centered, acc[q][m][o]);
+          } else {
+            acc[q][m][o] += centered;
+          }
+        }
+    }
+  }
+
+#pragma unroll
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float4* dst4 = reinterpret_cast<float4*>(&red[row][q * M + m][col * 8]);
+      dst4[0] = make_float4(acc[q][m][0], acc[q][m][1], acc[q][m][2], acc[q][m][3]);
+      dst4[1] = make_float4(acc[q][m][4], acc[q][m][5], acc[q][m][6], acc[q][m][7]);
+    }
+  __syncthreads();
+  const int nl = tid % STRIP;
+  const int part = tid / STRIP;
+  if (part < PARTS) {
+#pragma unroll
+    for (int qm = 0; qm < 2 * M; ++qm) {
+      float v = 0.0f;
+#pragma unroll
+      for (int r = 0; r < RPP; ++r) v += red[part * RPP + r][qm][nl];
+      red2[part][qm][nl] = v;
+    }
+  }
+  __syncthreads();
+  const int n0 = strip * STRIP;
+  for (int idx = tid; idx < M * STRIP; idx += THREADS) {
+    const int m = idx / STRIP, ol = idx % STRIP;
+    const int n = n0 + ol;
+    if (n >= p.seg[0].n_pad) continue;
+    float gu[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      float v = 0.0f;
+#pragma unroll
+      for (int k = 0; k < PARTS; ++k) v += red2[k][q * M + m][ol];
+      if (!GROUPED) v *= __half2float(__ushort_as_half(scale_raw[q]));
+      __half h = __float2half_rn(v);
+      if (p.seg[q].bias) h = __hadd(h, __ushort_as_half(bias_raw[q]));
+      gu[q] = __half2float(h);
+    }
+    p.seg[0].dst[((size_t)(n >> 2) * M + m) * 4 + (n & 3)] = __float2half_rn(GatedActivation(activation, gu[0], gu[1]));
+  }
+}
+
+template <int LPR, int WAVES>
+hipError_t LaunchGatedM(const StreamParams& p, bool grouped, int activation, dim3 grid, hipStream_t stream) {
+  const dim3 block(WAVES * 64);
+#define MLD_GATED(MM)                                                                                             \
+  if (grouped)                                                                                                    \
+    hipLaunchKernelGGL((fc_w4_gated_stream_kernel<LPR, WAVES, MM, true>), grid, block, 0, stream, p, activation); \
+  else                                                                                                            \
+    hipLaunchKernelGGL((fc_w4_gated_stream_kernel<LPR, WAVES, MM, false>), grid, block, 0, stream, p, activation);
+  switch (p.m) {
+    case 1: MLD_GATED(1) break;
+    case 2: MLD_GATED(2) break;
+    default: return hipErrorInvalidValue;
+  }
+#undef MLD_GATED
+  return hipGetLastError();
+}
+
 template <int LPR, int WAVES, int M, bool GROUPED, bool ZP>
 hipError_t LaunchCfgS(const StreamParams& p, dim3 grid, hipStream_t stream) {
   if (p.segments > 1)
@@ -461,6 +625,53 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   else
     hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
   return hipGetLastError();
+}
+
+bool FcW4GatedSupported(const FcArgs& gate, const FcArgs& up) {
+  if (!FcW4StreamSupported(gate) || !FcW4StreamSupported(up)) return false;
+  if (gate.m > 2) return false;  // the paired accumulators of more tokens would spill
+  if (gate.has_zero_point || up.has_zero_point) return false;
+  return gate.act == up.act && gate.m == up.m && gate.k == up.k && gate.n == up.n && gate.scale_kind == up.scale_kind &&
+         gate.groups == up.groups;
+}
+
+hipError_t LaunchFcW4Gated(const FcArgs& gate, const FcArgs& up, int activation, void* dst, hipStream_t stream,
+                           const char** kernel_name) {
+  StreamParams p;
+  p.segments = 2;
+  p.act = static_cast<const __half*>(gate.act);
+  p.partial = nullptr;
+  p.m = gate.m;
+  p.ks = DivUp(gate.k, 4);
+  p.chunks = DivUp(p.ks, 8);
+  p.chunks_per_split = p.chunks;
+  p.ksplit = 1;
+  const bool grouped = gate.scale_kind == kScaleBlock;
+  p.groups = grouped ? gate.groups : 1;
+  p.group_chunks = grouped ? (p.ks / gate.groups) / 8 : p.chunks;
+  p.mask_lo = 0x000F000Fu;
+  p.mask_hi = 0x00F000F0u;
+  p.magic_lo = 0x64006400u;
+  p.magic_hi = 0x54005400u;
+  const FcArgs* both[2] = {&gate, &up};
+  for (int i = 0; i < 2; ++i) {
+    StreamSegment& sg = p.seg[i];
+    sg.weights = reinterpret_cast<const u32x4*>(both[i]->weights);
+    sg.scale = static_cast<const __half*>(both[i]->scale);
+    sg.zero_point = nullptr;
+    sg.bias = static_cast<const __half*>(both[i]->bias);
+    sg.dst = static_cast<__half*>(dst);
+    sg.ns = DivUp(both[i]->n, 4);
+    sg.n_pad = sg.ns * 4;
+    sg.row_u4 = sg.ns / 2;
+    sg.strip_end = 0;
+  }
+  p.seg[2] = p.seg[0];
+  if (kernel_name) *kernel_name = "fc_w4_gated_stream_kernel";
+  // 128-byte row segments, 8 waves: 64 rows of chunks per pass (one pass covers K = 2048); the
+  // 16-wave shape would spill with the two sets of accumulators
+  const dim3 grid(DivUp(p.seg[0].row_u4, 8));
+  return LaunchGatedM<8, 8>(p, grouped, activation, grid, stream);
 }
 
 hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {

@@ -45,6 +45,11 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 
 // Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
+// dst = activation(gate(x)) * up(x) for a pair of such layers of one shape (1..2 tokens).
+bool FcW4GatedSupported(const FcArgs& gate, const FcArgs& up);
+hipError_t LaunchFcW4Gated(const FcArgs& gate, const FcArgs& up, int activation, void* dst, hipStream_t stream,
+                           const char** kernel_name);
+
 // The same for 1..16 tokens on the matrix cores (per-channel scales, wide layers).
 bool FcW4MfmaStreamSupported(const FcArgs& a);
 hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char** kernel_name);

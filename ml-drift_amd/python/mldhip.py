@@ -30,7 +30,7 @@ SYMBOLS = [
     "mldhip_op_src_count", "mldhip_op_dst_count", "mldhip_op_src_name", "mldhip_op_dst_name",
     "mldhip_op_set_src", "mldhip_op_set_dst", "mldhip_op_set_shape", "mldhip_op_launch",
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
-    "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read",
+    "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
 ]
 
 
@@ -319,6 +319,17 @@ def fc_launch_fused(ops, stream=0):
     FAILED_PRECONDITION when they cannot share a launch."""
     arr = (C.c_void_p * len(ops))(*[op.handle for op in ops])
     check(lib().mldhip_fc_launch_fused(arr, len(ops), C.c_void_p(stream)))
+
+
+GATE_GELU_TANH, GATE_SILU = 1, 2
+
+
+def fc_launch_gated(gate, up, activation, dst, stream=0):
+    """dst = activation(gate(x)) * up(x) in one launch; MldhipError(FAILED_PRECONDITION) when the
+    pair is not served (launch the ops and the elementwise step separately then)."""
+    check(lib().mldhip_fc_launch_gated(gate.handle, up.handle, activation,
+                                       C.c_void_p(dst.data_ptr()), C.c_size_t(dst.numel() * dst.element_size()),
+                                       C.c_void_p(stream)))
 
 
 def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1, 1),

@@ -308,3 +308,27 @@ def dequantize_weights(weights, n, k, weight_bits, scale_bits, scale_kind=SCALE_
     lib().mldo_dequantize_weights(n, k, weight_bits, _p(w), scale_kind, groups, _p(sc), _p(zp),
                                   _p(out))
     return out
+
+
+# ---- gated MLP step (samples/llm/gemma3_model_builder.cc:1054-1075, qwen3_model_builder.cc:850-863) ----
+def gated_activation(gate_f16, up_f16, kind):
+    """The sample's elementwise kernels on fp16 tensors, in fp32, in their operation order.
+    kind: "gelu_tanh" or "silu".  Returns fp16.  (tanh / exp are numpy's float32 routines: the
+    result is pinned up to the accuracy of those, a few ulp of fp32.)"""
+    g = np.asarray(gate_f16, np.float16).astype(np.float32)
+    u = np.asarray(up_f16, np.float16).astype(np.float32)
+    f32 = np.float32
+    if kind == "gelu_tanh":
+        gate_sq = g * g
+        tanh_in = g * (f32(0.7978845608) + f32(0.03567740813) * gate_sq)
+        clamped = np.clip(tanh_in, f32(-10.0), f32(10.0))
+        tanh_val = np.tanh(clamped).astype(np.float32)
+        gate_up_half = f32(0.5) * g * u
+        res = np.clip(gate_up_half * (f32(1.0) + tanh_val), f32(-65504.0), f32(65504.0))
+    elif kind == "silu":
+        with np.errstate(over="ignore"):  # exp(-g) = inf for very negative g: sig = 0, as on the device
+            sig = f32(1.0) / (f32(1.0) + np.exp(-g).astype(np.float32))
+        res = np.clip((g * sig) * u, f32(-65504.0), f32(65504.0))
+    else:
+        raise ValueError(kind)
+    return res.astype(np.float16)

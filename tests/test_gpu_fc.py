@@ -272,3 +272,56 @@ def test_int8_math_bit_exact(oracle, bits, m, k, n):
     if m * k * n <= 1 << 24:
         mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed, m, k, n, bits), n)
         assert np.array_equal(got, mimic)
+
+
+@pytest.mark.parametrize("m,k,n,groups,bias", [(1, 2048, 16384, 64, False), (2, 2048, 16384, 64, True),
+                                               (1, 4096, 14336, 1, False), (2, 1000, 1032, 1, True),
+                                               (1, 512, 72, 16, False)])
+@pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
+def test_gated_pair(oracle, m, k, n, groups, bias, kind):
+    """dst = activation(gate(x)) * up(x) in one launch against the three separate steps: the two
+    FullyConnected launches on the GPU, then the oracle's restatement of the sample's elementwise
+    kernel on their fp16 outputs.  Bar: the FullyConnected bar, 2e-2 of the output RMS (the fused
+    kernel adds K in another order, so a gate value can differ by an fp16 ulp); besides, 99 % of
+    the elements must agree to 2 fp16 ulp."""
+    torch = torch_cuda()
+    gate_case = W.make_fc_case(seed=11 + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                               with_bias=bias)
+    up_case = W.make_fc_case(seed=12 + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                             with_bias=bias)
+    up_case["act"] = gate_case["act"]
+    # gate values of a few units so that the activation is in its curved range
+    gate_case["scale"] = gate_case["scale"] * np.float32(40.0)
+    gate = W.FcDevice(gate_case)
+    up = W.FcDevice(up_case)
+    srcs = [gate.act, up.weights, up.scale] + ([up.bias] if bias else [])
+    up.op.bind(srcs, [up.out])  # both read the same tensor
+    print("gated", m, k, n, groups, bias, kind, flush=True)
+    gate.run(); up.run()
+    torch.cuda.synchronize()
+    g16 = gate.out.cpu().numpy()
+    u16 = up.out.cpu().numpy()
+    ref = W.from_slices(oracle.gated_activation(g16, u16, kind).astype(np.float32), n).astype(np.float64)
+    dst = torch.zeros_like(gate.out)
+    M.fc_launch_gated(gate.op, up.op, M.GATE_GELU_TANH if kind == "gelu_tanh" else M.GATE_SILU, dst,
+                      torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert gate.op.kernel_name == "fc_w4_gated_stream_kernel"
+    got = W.from_slices(dst.cpu().numpy().astype(np.float32), n).astype(np.float64)
+    rms = np.sqrt(np.mean(ref ** 2))
+    assert rms > 0
+    assert np.abs(got - ref).max() <= 2e-2 * rms
+    close = np.abs(got - ref) <= 2 * np.maximum(np.abs(ref), 2.0 ** -14) * 2.0 ** -10
+    assert close.mean() >= 0.99, close.mean()
+    # the two ops' own outputs are untouched by the gated launch
+    assert np.array_equal(gate.out.cpu().numpy(), g16) and np.array_equal(up.out.cpu().numpy(), u16)
+
+
+def test_gated_pair_refused(oracle):
+    torch = torch_cuda()
+    a = W.FcDevice(W.make_fc_case(seed=1, m=3, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1))
+    b = W.FcDevice(W.make_fc_case(seed=2, m=3, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1))
+    dst = torch.zeros_like(a.out)
+    with pytest.raises(M.MldhipError) as e:   # 3 tokens, and two different source tensors
+        M.fc_launch_gated(a.op, b.op, M.GATE_SILU, dst, torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == M.FAILED_PRECONDITION

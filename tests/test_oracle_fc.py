@@ -177,3 +177,19 @@ def test_dequantize_weights_matches_make_weights(oracle):
     ref = o.make_weights_from_int8(w, scale)
     # fp16 rounding of (q-8)*s: relative error 2^-11
     assert np.abs(got - ref).max() <= np.abs(ref).max() * 2.0 ** -10
+
+
+def test_gated_activation_known_values(oracle):
+    """gelu_tanh(g) * u and silu(g) * u against closed forms: 0 at g = 0, ~g*u for large g,
+    ~0 for very negative g, silu(g) = g / (1 + e^-g), the tanh argument clamp at +-10, the
+    fp16 range clamp."""
+    g = np.array([0.0, 8.0, -8.0, 1.0, -1.0, 300.0], np.float16)
+    u = np.array([3.0, 2.0, 2.0, 1.0, 1.0, 300.0], np.float16)
+    gelu = oracle.gated_activation(g, u, "gelu_tanh").astype(np.float64)
+    assert gelu[0] == 0.0 and gelu[1] == 16.0 and abs(gelu[2]) < 1e-6
+    assert abs(gelu[3] - 0.5 * (1 + np.tanh(0.7978845608 * (1 + 0.044715)))) < 1e-3
+    assert abs(gelu[4] + 0.5 * (1 - np.tanh(0.7978845608 * (1 + 0.044715)))) < 1e-3
+    assert gelu[5] == 65504.0  # 300 * 300 clamps to the fp16 range
+    silu = oracle.gated_activation(g, u, "silu").astype(np.float64)
+    assert silu[0] == 0.0 and abs(silu[3] - 1 / (1 + np.exp(-1.0))) < 1e-3 and abs(silu[4] + 1 / (1 + np.exp(1.0))) < 1e-3
+    assert abs(silu[1] - 16.0) < 2e-2 and abs(silu[2]) < 1e-2 and silu[5] == 65504.0
