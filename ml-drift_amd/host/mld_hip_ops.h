@@ -197,6 +197,16 @@ inline Status AddToQueueFused(const std::vector<HipOperation*>& ops, void* hip_s
   return Status::FromCode(mldhip_fc_launch_fused(handles.data(), (int)handles.size(), hip_stream));
 }
 
+// gelu_tanh(gate(x)) * up(x) / silu(gate(x)) * up(x) in the launch of the two projections: the
+// Linear, Linear, GeluTanhMul / SiluMul nodes of the sample's FFLayer
+// (samples/llm/gemma3_model_builder.cc:1141-1147) as one.  kFailedPrecondition: keep the three nodes.
+enum class GateActivation { kGeluTanh = MLDHIP_GATE_GELU_TANH, kSilu = MLDHIP_GATE_SILU };
+inline Status AddToQueueGated(HipOperation* gate, HipOperation* up, GateActivation activation, void* dst_device_ptr,
+                              size_t dst_bytes, void* hip_stream) {
+  return Status::FromCode(
+      mldhip_fc_launch_gated(gate->handle(), up->handle(), (int)activation, dst_device_ptr, dst_bytes, hip_stream));
+}
+
 // One linear layer read from the LLM sample's checkpoint files, as host buffers ready to upload:
 // what LlmWeightsLoader::GetWeightsInt4 / GetWeightsInt8 (samples/llm/llm_weights_loader.cc:29-117)
 // assemble through LlmFileTensorLoader.  `weights` carries the description and shapes that

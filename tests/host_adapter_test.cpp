@@ -107,6 +107,8 @@ int main() {
     std::remove((dir + base + ".weight").c_str());
     std::remove((dir + base + ".weight_quantized_scale").c_str());
   }
+  // a gated launch over unbound ops is refused before anything reaches the GPU
+  EXPECT(AddToQueueGated(&fc, &fc, GateActivation::kSilu, nullptr, 0, nullptr).code == MLDHIP_INVALID_ARGUMENT);
   std::printf("host adapter ok\n");
   return 0;
 }
