@@ -554,8 +554,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
-  static_assert(WAVES == 4 || WAVES == 8 || WAVES == 16, "the reduction handles WAVES registers per phase");
-  __shared__ float4 red[WAVES][WAVES][64];  // [copy][register within the phase][lane]
+  static_assert(WAVES == 4 || WAVES == 8, "the reduction's LDS buffers are sized for 4 or 8 waves");
+  // K reduction buffers: [phase parity][copy][register within the phase][lane], 128 KB
+  constexpr int RPH = WAVES == 4 ? 16 : 8;  // accumulator registers (x 4 MFMAs) per phase
+  __shared__ float4 red[2][WAVES][RPH][64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -736,50 +738,58 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     }
   }
 
-  // K-split reduction, spread over all waves.  The tile goes through LDS in phases of WAVES
+  // K-split reduction, spread over all waves.  The tile goes through LDS in phases of RPH
   // accumulator registers per lane (x 4 MFMAs): every wave writes its copy, then wave w adds the
-  // WAVES copies of register w in a fixed order and stores that part of the output.  In the
-  // 32x32 result, register v of lane (g2, i32) belongs to output slice 8*(v/4) + 4*g2 + v%4 and
-  // token i32, and the four MFMAs hold the slice's four channels: one 8-byte store.
+  // WAVES copies of registers w, w + WAVES, ... in a fixed order and stores that part of the
+  // output.  Two buffers alternate, so one barrier per phase is enough: a wave that writes
+  // phase p + 2 has passed the barrier of phase p + 1, which every wave reaches only after its
+  // reads of phase p.  In the 32x32 result, register v of lane (g2, i32) belongs to output slice
+  // 8*(v/4) + 4*g2 + v%4 and token i32, and the four MFMAs hold the slice's four channels: one
+  // 8-byte store.
   const __half* bias = sg.bias;
   __half* dst = sg.dst;
+  static_assert(16 % RPH == 0 && RPH % WAVES == 0, "phases tile the 16 registers, waves tile a phase");
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
     const int mi = token(fm);
 #pragma unroll
-    for (int ph = 0; ph < 16 / WAVES; ++ph) {
+    for (int ph = 0; ph < 16 / RPH; ++ph) {
+      const int buf = (fm * (16 / RPH) + ph) & 1;
 #pragma unroll
-      for (int j = 0; j < WAVES; ++j) {
-        const int v = ph * WAVES + j;
-        red[wave][j][lane] = make_float4(acc[0][fm][v], acc[1][fm][v], acc[2][fm][v], acc[3][fm][v]);
+      for (int j = 0; j < RPH; ++j) {
+        const int v = ph * RPH + j;
+        red[buf][wave][j][lane] = make_float4(acc[0][fm][v], acc[1][fm][v], acc[2][fm][v], acc[3][fm][v]);
       }
       LdsBarrier();
-      float4 sum = red[0][wave][lane];
 #pragma unroll
-      for (int c = 1; c < WAVES; ++c) {
-        const float4 o = red[c][wave][lane];
-        sum.x += o.x;
-        sum.y += o.y;
-        sum.z += o.z;
-        sum.w += o.w;
-      }
-      const int v = ph * WAVES + wave;
-      const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-      if (mi < p.m && slice < sg.ns && p.ksplit > 1) {
-        // this work-group's share of K: fp32 sums for the second pass
-        *reinterpret_cast<float4*>(sg.partial + (((size_t)blockIdx.y * sg.ns + slice) * p.m + mi) * 4) = sum;
-      } else if (mi < p.m && slice < sg.ns) {
-        __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
-        if (bias) {
+      for (int q = 0; q < RPH / WAVES; ++q) {
+        const int j = q * WAVES + wave;
+        float4 sum = red[buf][0][j][lane];
 #pragma unroll
-          for (int t4 = 0; t4 < 4; ++t4) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
+        for (int c = 1; c < WAVES; ++c) {
+          const float4 o = red[buf][c][j][lane];
+          sum.x += o.x;
+          sum.y += o.y;
+          sum.z += o.z;
+          sum.w += o.w;
         }
-        u32x2 o;
-        o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
-        o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-        *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+        const int v = ph * RPH + j;
+        const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
+        if (mi < p.m && slice < sg.ns && p.ksplit > 1) {
+          // this work-group's share of K: fp32 sums for the second pass
+          *reinterpret_cast<float4*>(sg.partial + (((size_t)blockIdx.y * sg.ns + slice) * p.m + mi) * 4) = sum;
+        } else if (mi < p.m && slice < sg.ns) {
+          __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
+          if (bias) {
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
+          }
+          u32x2 o;
+          o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+          o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+          *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+        }
       }
-      if (fm + 1 < FM || ph + 1 < 16 / WAVES) LdsBarrier();
     }
   }
 }
