@@ -325,3 +325,35 @@ def test_gated_pair_refused(oracle):
     with pytest.raises(M.MldhipError) as e:   # 3 tokens, and two different source tensors
         M.fc_launch_gated(a.op, b.op, M.GATE_SILU, dst, torch.cuda.current_stream().cuda_stream)
     assert e.value.code == M.FAILED_PRECONDITION
+
+
+def test_random_shapes_sweep(oracle):
+    """Seeded sweep over token counts, ragged K / N and scale groupings, whatever kernel the
+    dispatcher picks: every result against the textbook reference at the fp16 bar.  Covers the
+    tile-plane edges of the kernels (odd tile counts per XCD rectangle, strips and K shares that
+    end inside a work-group, token counts at the kernel boundaries)."""
+    rng = np.random.default_rng(2024)
+    seen = {}
+    for it in range(48):
+        m = int(rng.choice([1, 2, 3, 4, 5, 7, 16, 17, 31, 33, 64, 65, 100, 128, 129, 200, 257, 300]))
+        bits = int(rng.choice([4, 4, 4, 8]))
+        k = int(rng.choice([64, 96, 171, 256, 512, 1000, 1024, 2048, 4096])) if m > 4 else int(
+            rng.choice([64, 171, 512, 1000, 2048, 4096, 8192]))
+        n = int(rng.choice([8, 20, 64, 152, 533, 1024, 2050, 4096, 8200, 8228]))
+        groups = 1
+        if k % 32 == 0 and rng.random() < 0.6:
+            groups = k // int(rng.choice([32, 64, k])) if k >= 64 else 1
+        zp = bool(rng.random() < 0.3)
+        bias = bool(rng.random() < 0.5)
+        if m * k * n > 300 * 1024 * 8228:
+            n = 1024
+        case = W.make_fc_case(seed=1000 + it, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                              with_zero_point=zp, with_bias=bias)
+        print("sweep", it, dict(m=m, k=k, n=n, bits=bits, groups=groups, zp=zp, bias=bias), flush=True)
+        dev = W.FcDevice(case)
+        dev.run()
+        got = dev.result()
+        seen[dev.op.kernel_name] = seen.get(dev.op.kernel_name, 0) + 1
+        check_fp(got, textbook(case), case, "sweep %d (%s)" % (it, dev.op.kernel_name))
+    print("kernels exercised:", seen)
+    assert len(seen) >= 4
