@@ -86,12 +86,6 @@ struct GemmParams {
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
 __device__ __forceinline__ uint32_t AsU32(half2_t v) { return __builtin_bit_cast(uint32_t, v); }
 
-__device__ __forceinline__ uint32_t AndOr(uint32_t x, uint32_t mask, uint32_t magic) {
-  uint32_t d;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "s"(mask), "v"(magic));
-  return d;
-}
-
 // The reference's rescale of an int32 accumulator: every product and sum is a separate
 // rounding, in this order.
 #pragma clang fp contract(off)
@@ -675,6 +669,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[t4][fm][v] = 0.0f;
 
+  // The exponent patterns are parked in vector registers: (x & mask) | magic then selects to one
+  // v_and_or_b32 (the instruction reads at most one scalar register), and the compiler, which
+  // sees the instruction, is free to schedule it among the MFMAs (an inline-asm form measured
+  // 7 % slower at 2048 tokens).
+  uint32_t magic_lo = p.magic_lo, magic_hi = p.magic_hi;
+  asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
   const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
 
@@ -718,7 +718,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
 #pragma unroll
         for (int wd = 0; wd < 4; ++wd) {
           const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
-          const uint32_t bits = (t4 & 1) ? AndOr(x, p.mask_hi, p.magic_hi) : AndOr(x, p.mask_lo, p.magic_lo);
+          const uint32_t bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
           aop[wd] = AsU32((AsHalf2(bits) + off) * s2);
         }
 #pragma unroll
