@@ -83,3 +83,34 @@ def test_fused_launch_matches_single_launches(stack):
                 print("tokens", tokens, case["name"], "fused vs single max|diff|/rms = %.2e" % (worst / rms), flush=True)
                 assert worst <= 2e-3 * rms
                 pos += 1
+
+
+def test_graph_replays_match_eager():
+    """A decode step and a prefill step captured into a graph: several replays, with eager work
+    and synchronisations in between, must reproduce the eager results bit for bit (launches
+    allocate nothing after the first eager pass and record no memset nodes)."""
+    import torch
+    from decoder_stack import DecoderStack
+    st = DecoderStack(layers=2, max_tokens=128)
+    for tokens in (1, 128):
+        st.set_tokens(tokens)
+        st.launch()
+        torch.cuda.synchronize()
+        eager = [o.clone() for o in st.outs]
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                st.launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for rep in range(3):
+            for o in st.outs:
+                o.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for idx, (a, b) in enumerate(zip(eager, st.outs)):
+                assert torch.equal(a, b), (tokens, rep, idx)
+            # eager work between replays
+            st.launch()
+            torch.cuda.synchronize()
