@@ -184,3 +184,18 @@ def test_int8_conv_shapes(oracle, m, k, n, symmetric):
 def test_config4_int8_gemm(oracle, symmetric):
     c = make_int8_case(0, 2048, 2048, 8192)
     check_int8(oracle, c, symmetric)
+
+
+def test_int8_pipeline_random_sweep(oracle):
+    """Seeded sweep of the quantize -> int8 MFMA pipeline over ragged token / channel counts, all
+    three token-tile sizes, both quantization modes, zero points and biases: codes, params and
+    int32 accumulators bit-exact, rescaled output at the fp16 bar (check_int8)."""
+    rng = np.random.default_rng(77)
+    for it in range(16):
+        m = int(rng.choice([1, 5, 33, 64, 65, 130, 257, 600, 1100]))
+        k = int(rng.choice([16, 40, 100, 256, 1000, 2048]))
+        n = int(rng.choice([4, 20, 100, 256, 260, 1000, 2100, 4096]))
+        if m * k * n > 1 << 29:
+            k = 256
+        c = make_int8_case(500 + it, m, k, n, with_zp=bool(rng.random() < 0.4), with_bias=bool(rng.random() < 0.5))
+        check_int8(oracle, c, symmetric=bool(rng.random() < 0.5))
