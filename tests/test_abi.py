@@ -128,3 +128,19 @@ def test_unsupported_pack_layout_is_unimplemented():
     with pytest.raises(M.MldhipError) as e:  # weights_conversion.cc:1617
         M.rearrange_uint4_packed(np.zeros(8, np.uint8), (4, 1, 1, 4), d)
     assert e.value.code == M.UNIMPLEMENTED and "Unsupported layout" in e.value.message
+
+
+def test_header_is_plain_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 on its own (what a cgo / JNI / ctypes
+    binding includes), with no C++ in it."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "mldhip.h"\n'
+                   "int main(void) { mldhip_checkpoint_fc c; (void)c; return MLDHIP_GATE_SILU == 2 ? 0 : 1; }\n")
+    r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only",
+                        "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
