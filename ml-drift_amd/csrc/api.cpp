@@ -546,8 +546,8 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
   a.scalar_scale = d.scalar_scale;
   a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
   a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
-  // split-K workspace of the int4 kernels: allocated once, on the first launch
-  if (a.weight_bits == 4 && a.act_f16)
+  // split-K workspace of the fp16 streaming and matrix-core kernels: allocated once, on the first launch
+  if ((a.weight_bits == 4 || a.weight_bits == 8) && a.act_f16)
     if (int rc = AllocWorkspace(op, d.o)) return rc;
   a.partial = op->partial;
   a.partial_floats = op->partial_floats;
@@ -644,11 +644,11 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
     stream_ok = stream_ok && FcW4StreamSupported(a);
     mfma_ok = mfma_ok && FcW4MfmaSupported(a);
     if (a.act != f.act || a.m != f.m || a.k != f.k || a.scale_kind != f.scale_kind || a.groups != f.groups ||
-        a.has_zero_point != f.has_zero_point)
-      return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " does not read the same tensor with the same K and scale groups as op 0");
+        a.has_zero_point != f.has_zero_point || a.weight_bits != f.weight_bits)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "op " + std::to_string(i) + " does not read the same tensor with the same K, weight type and scale groups as op 0");
   }
   if (!stream_ok && !mfma_ok)
-    return Fail(MLDHIP_FAILED_PRECONDITION, "the ops are not all served by the same int4 kernel at this shape");
+    return Fail(MLDHIP_FAILED_PRECONDITION, "the ops are not all served by the same kernel at this shape");
   const char* name = nullptr;
   hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
   hipError_t e = stream_ok ? LaunchFcW4StreamFused(args, count, stream, &name) : LaunchFcW4MfmaFused(args, count, stream, &name);

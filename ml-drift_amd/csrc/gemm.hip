@@ -1,9 +1,10 @@
 // Prefill-side kernels for gfx950: MFMA GEMMs.
 //
-//  fc_w4_mfma_gemm_kernel   multi-token FullyConnected over the packed int4 I4O4 buffer: every
+//  fc_w4_mfma_gemm_kernel   multi-token FullyConnected over the packed uint4 I4O4 buffer: every
 //                           wave dequantizes its weight operands in registers (one rounding per
 //                           weight: round((u-8)*s), like the reference's fma(u, s, -8s)), then
 //                           v_mfma_f32_32x32x16_f16 with fp32 accumulation; no LDS in the loop.
+//  fc_w8_mfma_gemm_kernel   the same kernel over the packed uint8 I4O4 buffer (u - 128).
 //  conv_int8_mfma_kernel    int8 codes x int8 weights with v_mfma_i32_32x32x32_i8 (int32
 //                           accumulators, exact), tiles streamed global -> LDS without passing
 //                           through registers, then the reference's rescale epilogue.
@@ -41,7 +42,7 @@ typedef float float2v_t __attribute__((ext_vector_type(2)));
 // belong to it.
 constexpr int kMaxW4Segments = 3;
 struct W4Segment {
-  const uint8_t* w4;    // [Ks][Ns] blocks of 8 bytes
+  const uint8_t* w4;    // [Ks][Ns] blocks of 8 bytes (uint4) or 16 bytes (uint8)
   const __half* scale;  // [groups][Ns][4]
   const __half* zp;     // zero points, same shape as scale, or null
   const __half* bias;
@@ -505,7 +506,8 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
 }
 
 // ------------------------------------------------------------------------------------------
-// int4 prefill GEMM without LDS in the main loop.
+// int4 / int8-weight prefill GEMM without LDS in the main loop (described for uint4; the uint8
+// differences are at the kernel).
 //
 // Work-group = WAVES waves on one output tile of 128 channels x (FM*32) tokens; the waves split
 // K WAVES ways and add their fp32 tiles through LDS at the end (fixed order).  Compiled shapes:
@@ -537,15 +539,22 @@ __device__ __forceinline__ void SwapRegisters(u32x4& a, u32x4& b) {
   b[1] = b1;
 }
 
-// ZP: the weights have a zero-point tensor (same shape as the scales); the centre of the codes
-// moves from 8 to 8 + zp (exact in fp16 for integral zero points).
+// ZP: the weights have a zero-point tensor (same shape as the scales): w = (u - shift) * s - zp * s,
+// one fused multiply-add per pair of weights (zp * s is formed once per channel and scale group).
 // PAIR (FM even, token count even): a lane's tokens for the MFMA pair (fm, fm+1) are neighbours
 // (2j, 2j+1 instead of j, j+32), so one 16-byte load brings both activation operands.
 // MULTI: the launch covers more than one matrix (the single-matrix instantiation reads its
 // arguments at fixed offsets instead of through a dependent scalar load).
-template <int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI>
+// WB: weight bits.  8: the packed buffer holds 16-byte blocks, word i = input channel i of the
+// K-slice, byte o = output channel o of the slice, u = w + 128.  A byte permute gathers byte o of
+// two words into the low bytes of two halfs, 0x6400 on top makes them 1024 + u, and
+// (1024 + u - 1152) * s is the weight.  Everything else is shared with the int4 form.
+template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
+  static_assert(WB == 4 || WB == 8, "uint4 or uint8 weights");
   static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
+  constexpr uint32_t kBlk = WB == 8 ? 16u : 8u;  // bytes of one (K-slice, output slice) block
+  typedef typename std::conditional<WB == 8, u32x4, u32x2>::type wblk_t;
   constexpr int BN = 128;
   constexpr int BM = FM * 32;
   static_assert(WAVES == 4 || WAVES == 8, "the reduction's LDS buffers are sized for 4 or 8 waves");
@@ -589,7 +598,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int shares = WAVES * p.ksplit;  // blockIdx.y selects the work-group's part of K
   const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
   const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * WAVES + wave) * per_wave);
-  const uint32_t row_w = (uint32_t)sg.ns * 8u;  // bytes per K-slice row of the weights
+  const uint32_t row_w = (uint32_t)sg.ns * kBlk;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
   const uint32_t w_end = min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w);
@@ -620,7 +629,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
   // address lives there.
   const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
-  uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * 8u : kOob;
+  uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * kBlk : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
   // token of this lane in MFMA token block fm
   auto token = [&](int fm) { return PAIR ? m0 + (fm / 2) * 64 + 2 * i32 + (fm & 1) : m0 + fm * 32 + i32; };
@@ -631,11 +640,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     const int mi = token(PAIR ? 2 * i : i);
     vx[i] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
   }
-  const uint32_t group_bytes = row_w;  // one scale group: [Ns][4] halfs
+  const uint32_t group_bytes = (uint32_t)sg.ns * 8u;  // one scale group: [Ns][4] halfs
 
-  u32x2 rw[U][2], rsc[U], rzp[U], rx[U][NX][2];
+  wblk_t rw[U][2];
+  u32x2 rsc[U], rzp[U], rx[U][NX][2];
   u32x4 rxp[U][NX][2];  // PAIR: {token 2j: 4 halfs, token 2j+1: 4 halfs} per K-slice row
-  auto load_step = [&](int t, bool with_scale, u32x2 (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[NX][2],
+  auto load_step = [&](int t, bool with_scale, wblk_t (&w)[2], u32x2& sc, u32x2& zpv, u32x2 (&x)[NX][2],
                        u32x4 (&xp)[NX][2]) {
     // The scales (and zero points) of a pair of steps (t - 1, t), t odd, which share a group
     // because a group holds an even number of steps.  They travel with the odd step: by then
@@ -645,8 +655,13 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       sc = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
       if (ZP) zpv = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, vs + (uint32_t)(t >> p.group_shift) * group_bytes, 0, 0);
     }
-    w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
-    w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w1, vw0, 0, 0);
+    if constexpr (WB == 8) {
+      w[0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, vw0, 0, 0);
+      w[1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w1, vw0, 0, 0);
+    } else {
+      w[0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw0, 0, 0);
+      w[1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w1, vw0, 0, 0);
+    }
     vw0 += step_w;
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
@@ -677,6 +692,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
   const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
   const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+  const half2_t off_w8 = {(_Float16)-1152.0f, (_Float16)-1152.0f};
 
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -689,8 +705,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     for (int u = 0; u < U; ++u) {
       const int t = t_begin + tt + u;
       // consume stage u
-      const u32x4 blk = {rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
-      const u32x4 blk8 = {blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
+      u32x4 blk = {0u, 0u, 0u, 0u}, blk8 = blk;
+      if constexpr (WB == 4) {
+        blk = u32x4{rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
+        blk8 = u32x4{blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
+      }
       const half2_t sc01 = AsHalf2(rsc[u & ~1][0]), sc23 = AsHalf2(rsc[u & ~1][1]);
       half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
       if (ZP) {
@@ -709,17 +728,28 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
       for (int t4 = 0; t4 < 4; ++t4) {
         const half2_t sp = (t4 & 2) ? sc23 : sc01;
         const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
-        half2_t off = (t4 & 1) ? off_hi : off_lo;
+        const half2_t off = WB == 8 ? off_w8 : ((t4 & 1) ? off_hi : off_lo);
+        // zero point: (u - shift) * s - zp * s in one fused step, so that a fractional zero point
+        // costs one extra rounding of zp * s and not a rounding of shift + zp to an integer
+        half2_t mzs = {(_Float16)0.0f, (_Float16)0.0f};
         if (ZP) {
           const half2_t zq = (t4 & 2) ? zp23 : zp01;
-          off -= (t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0);
+          mzs = -(((t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0)) * s2);
         }
         u32x4 aop;
 #pragma unroll
         for (int wd = 0; wd < 4; ++wd) {
-          const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
-          const uint32_t bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
-          aop[wd] = AsU32((AsHalf2(bits) + off) * s2);
+          uint32_t bits;
+          if constexpr (WB == 8) {
+            // bytes t4 of the words of input channels 2*wd, 2*wd + 1 -> the low bytes of two halfs
+            const uint32_t sel = 0x0c000c00u | (uint32_t)t4 | ((uint32_t)(4 + t4) << 16);
+            bits = __builtin_amdgcn_perm(rw[u][wd >> 1][2 * (wd & 1) + 1], rw[u][wd >> 1][2 * (wd & 1)], sel) | magic_lo;
+          } else {
+            const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
+            bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
+          }
+          const half2_t centred = AsHalf2(bits) + off;  // exact: u - shift
+          aop[wd] = AsU32(ZP ? __builtin_elementwise_fma(centred, s2, mzs) : centred * s2);
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -794,17 +824,24 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   }
 }
 
-template <int FM, int U, int WAVES, bool PAIR>
-void LaunchDirect(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
+template <int WB, int FM, int U, int WAVES, bool PAIR>
+void LaunchDirectW(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
   const dim3 block(WAVES * 64);
   if (zp && p.segments > 1)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, true>), grid, block, 0, stream, p);
   else if (zp)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, true, PAIR, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, false>), grid, block, 0, stream, p);
   else if (p.segments > 1)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, true>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<FM, U, WAVES, false, PAIR, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, false>), grid, block, 0, stream, p);
+}
+template <int FM, int U, int WAVES, bool PAIR>
+void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
+  if (weight_bits == 8)
+    LaunchDirectW<8, FM, U, WAVES, PAIR>(zp, grid, stream, p);
+  else
+    LaunchDirectW<4, FM, U, WAVES, PAIR>(zp, grid, stream, p);
 }
 
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
@@ -908,12 +945,13 @@ hipError_t LaunchConvInt8Tile(const GemmParams& p, hipStream_t stream) {
 }  // namespace
 
 bool FcW4MfmaSupported(const FcArgs& a) {
-  if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
+  if ((a.weight_bits != 4 && a.weight_bits != 8) || !a.act_f16 || !a.dst_f16) return false;
   if (a.scale_kind == kScaleScalar) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   if (a.m <= kGemvMaxTokens) return false;
   // 32-bit buffer offsets
-  if ((size_t)DivUp(a.k, 4) * DivUp(a.n, 4) * 8 >= 0x7FFFFFF0u || (size_t)DivUp(a.k, 4) * a.m * 8 >= 0x7FFFFFF0u)
+  const size_t block_bytes = a.weight_bits == 8 ? 16 : 8;
+  if ((size_t)DivUp(a.k, 4) * DivUp(a.n, 4) * block_bytes >= 0x7FFFFFF0u || (size_t)DivUp(a.k, 4) * a.m * 8 >= 0x7FFFFFF0u)
     return false;
   if (a.scale_kind == kScaleBlock) {
     // an MFMA step of 16 input channels must not straddle scale groups
@@ -961,14 +999,15 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
     sg.partial = args[i].partial;
     sg.n = args[i].n;
     sg.ns = DivUp(args[i].n, 4);
-    sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * 8);
+    if (args[i].weight_bits != a.weight_bits) return hipErrorInvalidValue;
+    sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * (a.weight_bits == 8 ? 16 : 8));
     sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8);
     tiles_n += DivUp(args[i].n, 128);
     sg.tile_end = tiles_n;
     n_total += args[i].n;
   }
   for (int i = count; i < kMaxW4Segments; ++i) p.seg[i] = p.seg[0];
-  if (kernel_name) *kernel_name = "fc_w4_mfma_gemm_kernel";
+  if (kernel_name) *kernel_name = a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel";
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 && a.m % 2 == 0 ? 4 : 2);
@@ -985,13 +1024,13 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   const bool zp = p.seg[0].zp != nullptr;
   const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
   if (fm == 4)
-    LaunchDirect<4, 4, 4, true>(zp, grid, stream, p);
+    LaunchDirect<4, 4, 4, true>(a.weight_bits, zp, grid, stream, p);
   else if (fm == 2 && pair)
-    LaunchDirect<2, 4, 8, true>(zp, grid, stream, p);
+    LaunchDirect<2, 4, 8, true>(a.weight_bits, zp, grid, stream, p);
   else if (fm == 2)
-    LaunchDirect<2, 4, 8, false>(zp, grid, stream, p);
+    LaunchDirect<2, 4, 8, false>(a.weight_bits, zp, grid, stream, p);
   else
-    LaunchDirect<1, 4, 8, false>(zp, grid, stream, p);
+    LaunchDirect<1, 4, 8, false>(a.weight_bits, zp, grid, stream, p);
   if (p.ksplit > 1) {
     size_t items = 0;
     for (int i = 0; i < count; ++i) items += (size_t)p.seg[i].ns * a.m;

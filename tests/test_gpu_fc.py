@@ -184,6 +184,8 @@ def test_generic_kernel_reference_test_shapes(oracle, bits, dtype, kind):
             expect = "fc_w4_stream_kernel" if m <= 4 else "fc_w4_mfma_gemm_kernel"
         if bits == 8 and kind == "linear" and m <= 4:  # per-channel int8, either tensor type
             expect = "fc_w8_stream_kernel"
+        if bits == 8 and kind == "linear" and m > 4 and dtype == np.float16:
+            expect = "fc_w8_mfma_gemm_kernel"
         run_case(oracle, case, expect)
 
 

@@ -18,11 +18,11 @@ FP16_TOL = 2e-2
 
 
 def run_w4(case):
-    print("w4 gemm", {k: case[k] for k in ("m", "k", "n", "groups")}, flush=True)
+    print("w%d gemm" % case["weight_bits"], {k: case[k] for k in ("m", "k", "n", "groups")}, flush=True)
     dev = W.FcDevice(case)
     dev.run()
     got = dev.result()
-    assert dev.op.kernel_name == "fc_w4_mfma_gemm_kernel", dev.op.kernel_name
+    assert dev.op.kernel_name == "fc_w%d_mfma_gemm_kernel" % case["weight_bits"], dev.op.kernel_name
     dev.run()
     assert np.array_equal(got, dev.result())
     return got
@@ -62,6 +62,74 @@ def test_w4_gemm_wide_token_tile(oracle, m, k, n, groups, zp):
     check_fp(got, textbook(case), case, "textbook")
     sub = dict(case, m=64, act=case["act"][:64])
     check_fp(got[:64], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement (first 64 tokens)")
+
+
+@pytest.mark.parametrize("m,k,n,groups,zp", [(16, 256, 128, 8, False), (5, 64, 8, 1, True), (128, 2048, 2048, 64, False),
+                                             (77, 352, 200, 11, True), (130, 96, 260, 1, False),
+                                             (64, 4096, 256, 128, True), (300, 1024, 1024, 8, False),
+                                             (2048, 64, 4096, 2, True), (2050, 96, 4000, 1, False)])
+def test_w8_gemm_shapes(oracle, m, k, n, groups, zp):
+    """uint8 weights (16-byte blocks, u = w + 128) through the same matrix-core kernel: every token
+    tile (32, 64, paired 64, 128), ragged edges, per-channel and group-wise scales, zero points."""
+    case = W.make_fc_case(seed=2 * m + n, m=m, k=k, n=n, weight_bits=8, tensor_dtype=np.float16, groups=groups,
+                          with_bias=(m % 2 == 1), with_zero_point=zp)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    small = min(m, 64)
+    sub = dict(case, m=small, act=case["act"][:small])
+    if small * k * n <= 1 << 26:
+        check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,k,n,groups", [(33, 512, 260, 4), (256, 1024, 512, 1)])
+def test_gemm_fractional_zero_points(oracle, bits, m, k, n, groups):
+    """Zero points that are not whole numbers (what `file / scale` of a checkpoint can give): the
+    kernel applies them as -(zp * s) inside a fused multiply-add, not by moving the integer centre."""
+    case = W.make_fc_case(seed=7 * m + bits, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True, with_zero_point=True)
+    rng = np.random.default_rng(m + bits)
+    spread = 3.0 if bits == 4 else 40.0
+    case["zero_point"] = rng.uniform(-spread, spread, size=(n, groups)).astype(np.float16).astype(np.float32)
+    # activations with a mean, so that an error in the centre does not average out
+    case["act"] = (case["act"].astype(np.float32) + 0.5).astype(np.float16)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    small = min(m, 64)
+    sub = dict(case, m=small, act=case["act"][:small])
+    check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+
+
+def test_w8_gemm_fused_launch():
+    """Three uint8 matrices over one activation tensor in one launch give the bytes of the three
+    single launches; a uint4 op cannot join them."""
+    import torch
+    m, k = 96, 512
+    cases = [W.make_fc_case(seed=40 + i, m=m, k=k, n=n, weight_bits=8, tensor_dtype=np.float16, groups=4, with_bias=True)
+             for i, n in enumerate((384, 128, 200))]
+    for c in cases[1:]:
+        c["act"] = cases[0]["act"]
+    devs = [W.FcDevice(c) for c in cases]
+    for d in devs[1:]:
+        d.op.set_src(0, devs[0].act)
+    single = []
+    for d in devs:
+        d.run()
+        single.append(d.result())
+        assert d.op.kernel_name == "fc_w8_mfma_gemm_kernel"
+        d.out.zero_()
+    M.fc_launch_fused([d.op for d in devs], torch.cuda.current_stream().cuda_stream)
+    for d, c, ref in zip(devs, cases, single):
+        got = d.result()
+        check_fp(got, textbook(c), c, "fused uint8")
+        assert np.array_equal(got, ref)
+    other = W.make_fc_case(seed=50, m=m, k=k, n=128, weight_bits=4, tensor_dtype=np.float16, groups=4)
+    other["act"] = cases[0]["act"]
+    d4 = W.FcDevice(other)
+    d4.op.set_src(0, devs[0].act)
+    with pytest.raises(M.MldhipError) as err:
+        M.fc_launch_fused([devs[0].op, d4.op])
+    assert err.value.code == M.FAILED_PRECONDITION
 
 
 def test_config3_prefill_gemm(oracle):
