@@ -670,15 +670,18 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
     if (int rc = CheckBindings(ops[i])) return rc;
     if (int rc = BuildFcArgs(ops[i], &args[i])) return rc;
   }
-  if (!FcW4GatedSupported(args[0], args[1]))
+  const bool gemv = FcW4GatedSupported(args[0], args[1]);
+  if (!gemv && !FcW4MfmaGatedSupported(args[0], args[1]))
     return Fail(MLDHIP_FAILED_PRECONDITION,
                 "gate and up are not a pair of int4 fp16 FullyConnected ops over one tensor with one shape, "
-                "symmetric weights and at most 2 tokens");
+                "symmetric weights and scale groups the int4 kernels serve");
   const size_t need = (size_t)DivUp(args[0].n, 4) * 4 * args[0].m * sizeof(uint16_t);
   if (dst_bytes < need) return Fail(MLDHIP_INVALID_ARGUMENT, "dst is too small for the gated output");
   const char* name = nullptr;
-  hipError_t e = LaunchFcW4Gated(args[0], args[1], activation, dst,
-                                 static_cast<hipStream_t>(stream_ptr), &name);
+  hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
+  // 1..2 tokens: the streaming GEMV pair; more: the matrix-core GEMM with the gated epilogue
+  hipError_t e = gemv ? LaunchFcW4Gated(args[0], args[1], activation, dst, stream, &name)
+                      : LaunchFcW4MfmaGated(args[0], args[1], activation, dst, stream, &name);
   if (e != hipSuccess) return HipFail(e, "gated launch");
   gate->last_kernel = up->last_kernel = name;
   return MLDHIP_OK;

@@ -22,6 +22,7 @@
 #include <type_traits>
 
 #include "../../include/mldhip.h"
+#include "gated.h"
 #include "kernels.h"
 
 namespace mldhip {
@@ -82,6 +83,7 @@ struct GemmParams {
   int ksplit;       // work-groups along K per output tile (fp16 path)
   int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
   int xcd_m;        // fp16 path: the 8 XCDs form an xcd_m x (8 / xcd_m) grid over (token tiles, channel tiles)
+  int gate_activation;  // gated fp16 launch: MLDHIP_GATE_*
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -549,9 +551,15 @@ __device__ __forceinline__ void SwapRegisters(u32x4& a, u32x4& b) {
 // K-slice, byte o = output channel o of the slice, u = w + 128.  A byte permute gathers byte o of
 // two words into the low bytes of two halfs, 0x6400 on top makes them 1024 + u, and
 // (1024 + u - 1152) * s is the weight.  Everything else is shared with the int4 form.
-template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI>
+// GATED: seg[0] = gate, seg[1] = up, two matrices of one shape; the launch writes
+// activation(gate(x)) * up(x) to seg[0].dst.  The first half of the waves works on gate, the
+// second half on up, each half splitting K among its waves; the main loop is the same.  In the
+// reduction the wave that adds the copies of a register adds the two halves separately and so
+// holds the gate and the up value of the same slice and token.
+template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI, bool GATED = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   static_assert(WB == 4 || WB == 8, "uint4 or uint8 weights");
+  static_assert(!GATED || (!ZP && !MULTI), "the gated pair is symmetric and is the whole launch");
   static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
   constexpr uint32_t kBlk = WB == 8 ? 16u : 8u;  // bytes of one (K-slice, output slice) block
   typedef typename std::conditional<WB == 8, u32x4, u32x2>::type wblk_t;
@@ -584,10 +592,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     si = (p.segments > 2 && tn >= p.seg[1].tile_end) ? 2 : 1;
     tn -= p.seg[si - 1].tile_end;
   }
-  const W4Segment& sg = p.seg[MULTI ? si : 0];
-  const int n0 = tn * BN;
+  constexpr int KW = GATED ? WAVES / 2 : WAVES;  // waves that share one matrix's K
+  const int half = GATED ? __builtin_amdgcn_readfirstlane(wave / KW) : 0;
+  const W4Segment& sg = p.seg[GATED ? half : (MULTI ? si : 0)];
+  const int slice0 = tn * (BN / 4);  // first output slice of the tile
   const int m0 = tm * BM;
-  const int nsi = n0 / 4 + i32;
+  const int nsi = slice0 + i32;
   const bool n_ok = nsi < sg.ns;
 
   // This wave's range of 16-channel steps.  The buffer descriptors of the weights and the
@@ -595,9 +605,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // past K itself) read zeros without a test in the loop; a lane without an output slice or
   // a token gets an offset beyond every buffer.
   const int steps_total = (p.k + 15) / 16;
-  const int shares = WAVES * p.ksplit;  // blockIdx.y selects the work-group's part of K
+  const int shares = KW * p.ksplit;  // blockIdx.y selects the work-group's part of K
   const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
-  const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * WAVES + wave) * per_wave);
+  const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * KW + wave % KW) * per_wave);
   const uint32_t row_w = (uint32_t)sg.ns * kBlk;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
@@ -705,12 +715,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     for (int u = 0; u < U; ++u) {
       const int t = t_begin + tt + u;
       // consume stage u
+      const wblk_t wr[2] = {rw[u][0], rw[u][1]};
+      const u32x2 scr = rsc[u & ~1];
       u32x4 blk = {0u, 0u, 0u, 0u}, blk8 = blk;
       if constexpr (WB == 4) {
-        blk = u32x4{rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
+        blk = u32x4{wr[0][0], wr[0][1], wr[1][0], wr[1][1]};
         blk8 = u32x4{blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
       }
-      const half2_t sc01 = AsHalf2(rsc[u & ~1][0]), sc23 = AsHalf2(rsc[u & ~1][1]);
+      const half2_t sc01 = AsHalf2(scr[0]), sc23 = AsHalf2(scr[1]);
       half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
       if (ZP) {
         zp01 = AsHalf2(rzp[u & ~1][0]);
@@ -743,7 +755,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
           if constexpr (WB == 8) {
             // bytes t4 of the words of input channels 2*wd, 2*wd + 1 -> the low bytes of two halfs
             const uint32_t sel = 0x0c000c00u | (uint32_t)t4 | ((uint32_t)(4 + t4) << 16);
-            bits = __builtin_amdgcn_perm(rw[u][wd >> 1][2 * (wd & 1) + 1], rw[u][wd >> 1][2 * (wd & 1)], sel) | magic_lo;
+            bits = __builtin_amdgcn_perm(wr[wd >> 1][2 * (wd & 1) + 1], wr[wd >> 1][2 * (wd & 1)], sel) | magic_lo;
           } else {
             const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
             bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
@@ -776,8 +788,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // reads of phase p.  In the 32x32 result, register v of lane (g2, i32) belongs to output slice
   // 8*(v/4) + 4*g2 + v%4 and token i32, and the four MFMAs hold the slice's four channels: one
   // 8-byte store.
-  const __half* bias = sg.bias;
-  __half* dst = sg.dst;
+  // GATED: copies 0 .. KW-1 are gate's, the others up's; the two sums are rounded to fp16 (+ bias)
+  // as the two FullyConnected nodes would store them, then combined in fp32.
+  const __half* bias = GATED ? p.seg[0].bias : sg.bias;
+  const __half* bias_up = p.seg[GATED ? 1 : 0].bias;
+  __half* dst = GATED ? p.seg[0].dst : sg.dst;
   static_assert(16 % RPH == 0 && RPH % WAVES == 0, "phases tile the 16 registers, waves tile a phase");
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
@@ -796,7 +811,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
         const int j = q * WAVES + wave;
         float4 sum = red[buf][0][j][lane];
 #pragma unroll
-        for (int c = 1; c < WAVES; ++c) {
+        for (int c = 1; c < KW; ++c) {
           const float4 o = red[buf][c][j][lane];
           sum.x += o.x;
           sum.y += o.y;
@@ -804,11 +819,37 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
           sum.w += o.w;
         }
         const int v = ph * RPH + j;
-        const int slice = n0 / 4 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-        if (mi < p.m && slice < sg.ns && p.ksplit > 1) {
+        const int slice = slice0 + 8 * (v >> 2) + 4 * g2 + (v & 3);
+        const bool in_range = mi < p.m && slice < sg.ns;
+        if constexpr (GATED) {
+          float4 sum_up = red[buf][KW][j][lane];
+#pragma unroll
+          for (int c = KW + 1; c < WAVES; ++c) {
+            const float4 o = red[buf][c][j][lane];
+            sum_up.x += o.x;
+            sum_up.y += o.y;
+            sum_up.z += o.z;
+            sum_up.w += o.w;
+          }
+          if (in_range) {
+            const float g[4] = {sum.x, sum.y, sum.z, sum.w}, up[4] = {sum_up.x, sum_up.y, sum_up.z, sum_up.w};
+            __half h[4];
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4) {
+              __half hg = __float2half_rn(g[t4]), hu = __float2half_rn(up[t4]);
+              if (bias) hg = __hadd(hg, bias[slice * 4 + t4]);
+              if (bias_up) hu = __hadd(hu, bias_up[slice * 4 + t4]);
+              h[t4] = __float2half_rn(GatedActivation(p.gate_activation, __half2float(hg), __half2float(hu)));
+            }
+            u32x2 o;
+            o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+            o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+            *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+          }
+        } else if (in_range && p.ksplit > 1) {
           // this work-group's share of K: fp32 sums for the second pass
           *reinterpret_cast<float4*>(sg.partial + (((size_t)blockIdx.y * sg.ns + slice) * p.m + mi) * 4) = sum;
-        } else if (mi < p.m && slice < sg.ns) {
+        } else if (in_range) {
           __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
           if (bias) {
 #pragma unroll
@@ -838,6 +879,11 @@ void LaunchDirectW(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) 
 }
 template <int FM, int U, int WAVES, bool PAIR>
 void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
+  if (p.gate_activation != 0) {  // gated pair: uint4, symmetric
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<4, FM, U, WAVES, false, PAIR, false, true>), grid, dim3(WAVES * 64), 0,
+                       stream, p);
+    return;
+  }
   if (weight_bits == 8)
     LaunchDirectW<8, FM, U, WAVES, PAIR>(zp, grid, stream, p);
   else
@@ -942,13 +988,12 @@ hipError_t LaunchConvInt8Tile(const GemmParams& p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-}  // namespace
-
-bool FcW4MfmaSupported(const FcArgs& a) {
+// What the matrix-core kernel can run at all (any token count).
+bool DirectGemmShapeOk(const FcArgs& a) {
   if ((a.weight_bits != 4 && a.weight_bits != 8) || !a.act_f16 || !a.dst_f16) return false;
   if (a.scale_kind == kScaleScalar) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
-  if (a.m <= kGemvMaxTokens) return false;
+  if (a.m < 1) return false;
   // 32-bit buffer offsets
   const size_t block_bytes = a.weight_bits == 8 ? 16 : 8;
   if ((size_t)DivUp(a.k, 4) * DivUp(a.n, 4) * block_bytes >= 0x7FFFFFF0u || (size_t)DivUp(a.k, 4) * a.m * 8 >= 0x7FFFFFF0u)
@@ -963,10 +1008,15 @@ bool FcW4MfmaSupported(const FcArgs& a) {
   return true;
 }
 
-hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name) {
+// gate_activation != 0: args = {gate, up}, one output (gated_dst) of activation(gate) * up.
+hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, void* gated_dst, hipStream_t stream,
+                            const char** kernel_name) {
   if (count < 1 || count > kMaxW4Segments) return hipErrorInvalidValue;
+  const bool gated = gate_activation != 0;
+  if (gated && count != 2) return hipErrorInvalidValue;
   const FcArgs& a = args[0];
   GemmParams p = {};
+  p.gate_activation = gate_activation;
   p.segments = count;
   p.m = a.m;
   p.k = a.k;
@@ -995,25 +1045,33 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
     sg.scale = static_cast<const __half*>(args[i].scale);
     sg.zp = args[i].has_zero_point ? static_cast<const __half*>(args[i].zero_point) : nullptr;
     sg.bias = static_cast<const __half*>(args[i].bias);
-    sg.dst = static_cast<__half*>(args[i].dst);
+    sg.dst = static_cast<__half*>(gated ? gated_dst : args[i].dst);
     sg.partial = args[i].partial;
     sg.n = args[i].n;
     sg.ns = DivUp(args[i].n, 4);
     if (args[i].weight_bits != a.weight_bits) return hipErrorInvalidValue;
     sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * (a.weight_bits == 8 ? 16 : 8));
     sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8);
-    tiles_n += DivUp(args[i].n, 128);
+    if (gated) {
+      tiles_n = DivUp(args[i].n, 128);  // a tile holds the same 128 channels of both matrices
+      if (args[i].n != a.n) return hipErrorInvalidValue;
+    } else {
+      tiles_n += DivUp(args[i].n, 128);
+    }
     sg.tile_end = tiles_n;
     n_total += args[i].n;
   }
+  if (gated) n_total = a.n;  // one set of channel tiles, each with twice the work
   for (int i = count; i < kMaxW4Segments; ++i) p.seg[i] = p.seg[0];
-  if (kernel_name) *kernel_name = a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel";
+  if (kernel_name)
+    *kernel_name = gated ? "fc_w4_gated_mfma_gemm_kernel" : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 && a.m % 2 == 0 ? 4 : 2);
   p.ksplit = 1;
   if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) p.ksplit = std::max(1, std::atoi(e));
+  if (gated) p.ksplit = 1;  // the epilogue needs whole sums
   for (int i = 0; i < count; ++i)
     while (p.ksplit > 1 && (size_t)p.ksplit * p.seg[i].ns * 4 * a.m > args[i].partial_floats) p.ksplit /= 2;
   const int tiles_m = DivUp(a.m, fm * 32);
@@ -1039,8 +1097,30 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
   return hipGetLastError();
 }
 
+}  // namespace
+
+bool FcW4MfmaSupported(const FcArgs& a) { return a.m > kGemvMaxTokens && DirectGemmShapeOk(a); }
+
+hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name) {
+  return LaunchDirectGemm(args, count, 0, nullptr, stream, kernel_name);
+}
+
 hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
   return LaunchFcW4MfmaFused(&a, 1, stream, kernel_name);
+}
+
+bool FcW4MfmaGatedSupported(const FcArgs& gate, const FcArgs& up) {
+  if (!DirectGemmShapeOk(gate) || !DirectGemmShapeOk(up)) return false;
+  if (gate.weight_bits != 4 || up.weight_bits != 4) return false;
+  if (gate.has_zero_point || up.has_zero_point) return false;
+  return gate.act == up.act && gate.m == up.m && gate.k == up.k && gate.n == up.n && gate.scale_kind == up.scale_kind &&
+         gate.groups == up.groups;
+}
+
+hipError_t LaunchFcW4MfmaGated(const FcArgs& gate, const FcArgs& up, int activation, void* dst, hipStream_t stream,
+                               const char** kernel_name) {
+  const FcArgs both[2] = {gate, up};
+  return LaunchDirectGemm(both, 2, activation, dst, stream, kernel_name);
 }
 
 size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n) {

@@ -28,6 +28,7 @@
 #include <cstdlib>
 
 #include "../../include/mldhip.h"
+#include "gated.h"
 #include "kernels.h"
 
 namespace mldhip {
@@ -311,20 +312,6 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
 // FullyConnected nodes would store them, then combined in fp32 in the operation order of the
 // sample's elementwise kernel.  Only seg[0].dst is written.
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ float GatedActivation(int act, float g, float u) {
-  if (act == MLDHIP_GATE_GELU_TANH) {
-    const float gate_sq = g * g;
-    const float tanh_in = g * (0.7978845608f + 0.03567740813f * gate_sq);
-    const float clamped = fminf(fmaxf(tanh_in, -10.0f), 10.0f);
-    const float tanh_val = tanhf(clamped);
-    const float gate_up_half = 0.5f * g * u;
-    return fminf(fmaxf(gate_up_half * (1.0f + tanh_val), -65504.0f), 65504.0f);
-  }
-  const float sig = 1.0f / (1.0f + expf(-g));
-  const float silu = g * sig;
-  return fminf(fmaxf(silu * u, -65504.0f), 65504.0f);
-}
-
 template <int LPR, int WAVES, int M, bool GROUPED>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_gated_stream_kernel(StreamParams p, int activation) {
   constexpr int THREADS = WAVES * 64;

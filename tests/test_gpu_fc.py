@@ -281,6 +281,10 @@ def test_int8_math_bit_exact(oracle, bits, m, k, n):
                                                (1, 512, 72, 16, False)])
 @pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
 def test_gated_pair(oracle, m, k, n, groups, bias, kind):
+    run_gated_pair(oracle, m, k, n, groups, bias, kind, "fc_w4_gated_stream_kernel")
+
+
+def run_gated_pair(oracle, m, k, n, groups, bias, kind, expect_kernel, ulp_check=True):
     """dst = activation(gate(x)) * up(x) in one launch against the three separate steps: the two
     FullyConnected launches on the GPU, then the oracle's restatement of the sample's elementwise
     kernel on their fp16 outputs.  Bar: the FullyConnected bar, 2e-2 of the output RMS (the fused
@@ -308,15 +312,30 @@ def test_gated_pair(oracle, m, k, n, groups, bias, kind):
     M.fc_launch_gated(gate.op, up.op, M.GATE_GELU_TANH if kind == "gelu_tanh" else M.GATE_SILU, dst,
                       torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert gate.op.kernel_name == "fc_w4_gated_stream_kernel"
+    assert gate.op.kernel_name == expect_kernel, gate.op.kernel_name
     got = W.from_slices(dst.cpu().numpy().astype(np.float32), n).astype(np.float64)
     rms = np.sqrt(np.mean(ref ** 2))
     assert rms > 0
     assert np.abs(got - ref).max() <= 2e-2 * rms
-    close = np.abs(got - ref) <= 2 * np.maximum(np.abs(ref), 2.0 ** -14) * 2.0 ** -10
-    assert close.mean() >= 0.99, close.mean()
+    if ulp_check:
+        close = np.abs(got - ref) <= 2 * np.maximum(np.abs(ref), 2.0 ** -14) * 2.0 ** -10
+        assert close.mean() >= 0.99, close.mean()
     # the two ops' own outputs are untouched by the gated launch
     assert np.array_equal(gate.out.cpu().numpy(), g16) and np.array_equal(up.out.cpu().numpy(), u16)
+
+
+@pytest.mark.parametrize("m,k,n,groups,bias", [(3, 512, 72, 16, False), (16, 2048, 2048, 1, True),
+                                               (64, 1024, 1032, 32, True), (77, 352, 200, 11, False),
+                                               (128, 2048, 16384, 64, False), (130, 96, 260, 1, True),
+                                               (2048, 256, 4096, 1, True)])
+@pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
+def test_gated_pair_prefill(oracle, m, k, n, groups, bias, kind):
+    """The same step at prefill token counts: the matrix-core GEMM with the gated epilogue (tiles of
+    64 channels of both matrices), every token tile, ragged channel and token edges."""
+    # Up to 4 tokens the separate launches run the streaming GEMV, which keeps the weights in fp32
+    # where the matrix-core kernel rounds them to fp16: gate values then differ by a few fp16 ulp
+    # (inside the FullyConnected bar) and the ulp-level comparison says nothing there.
+    run_gated_pair(oracle, m, k, n, groups, bias, kind, "fc_w4_gated_mfma_gemm_kernel", ulp_check=m > 4)
 
 
 def test_gated_pair_refused(oracle):
@@ -324,9 +343,24 @@ def test_gated_pair_refused(oracle):
     a = W.FcDevice(W.make_fc_case(seed=1, m=3, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1))
     b = W.FcDevice(W.make_fc_case(seed=2, m=3, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1))
     dst = torch.zeros_like(a.out)
-    with pytest.raises(M.MldhipError) as e:   # 3 tokens, and two different source tensors
+    with pytest.raises(M.MldhipError) as e:   # two different source tensors
         M.fc_launch_gated(a.op, b.op, M.GATE_SILU, dst, torch.cuda.current_stream().cuda_stream)
     assert e.value.code == M.FAILED_PRECONDITION
+    # uint8 weights: not served by the gated kernels
+    c8 = W.make_fc_case(seed=3, m=8, k=256, n=64, weight_bits=8, tensor_dtype=np.float16, groups=1)
+    g8, u8 = W.FcDevice(c8), W.FcDevice(c8)
+    u8.op.set_src(0, g8.act)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_launch_gated(g8.op, u8.op, M.GATE_SILU, torch.zeros_like(g8.out), torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == M.FAILED_PRECONDITION
+    # a destination that is too small
+    c4 = W.make_fc_case(seed=4, m=8, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1)
+    g4, u4 = W.FcDevice(c4), W.FcDevice(c4)
+    u4.op.set_src(0, g4.act)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_launch_gated(g4.op, u4.op, M.GATE_SILU, torch.zeros(16, dtype=torch.float16, device="cuda"),
+                          torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == M.INVALID_ARGUMENT
 
 
 def test_random_shapes_sweep(oracle):
