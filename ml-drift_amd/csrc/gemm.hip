@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdlib>
 #include <type_traits>
 
@@ -84,6 +85,7 @@ struct GemmParams {
   int group_shift;  // log2(group_size / 16) when that is a power of two, else -1 (not supported by the direct kernel)
   int xcd_m;        // fp16 path: the 8 XCDs form an xcd_m x (8 / xcd_m) grid over (token tiles, channel tiles)
   int gate_activation;  // gated fp16 launch: MLDHIP_GATE_*
+  int dual;             // fp16 path: a work-group owns two neighbouring channel tiles
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -556,8 +558,14 @@ __device__ __forceinline__ void SwapRegisters(u32x4& a, u32x4& b) {
 // second half on up, each half splitting K among its waves; the main loop is the same.  In the
 // reduction the wave that adds the copies of a register adds the two halves separately and so
 // holds the gate and the up value of the same slice and token.
-template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI, bool GATED = false>
+// DUAL: the same split of the waves for an ordinary launch: the work-group owns two neighbouring
+// channel tiles (2j, 2j + 1 of the launch), one per half.  The two halves read the same
+// activations, so every activation tile is fetched from L2 once for 256 channels, and there are
+// half as many work-groups and reduction rounds; for launches with many tiles.
+enum { kModePlain = 0, kModeGated = 1, kModeDual = 2 };
+template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI, int MODE = kModePlain>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
+  constexpr bool GATED = MODE == kModeGated, DUAL = MODE == kModeDual;
   static_assert(WB == 4 || WB == 8, "uint4 or uint8 weights");
   static_assert(!GATED || (!ZP && !MULTI), "the gated pair is symmetric and is the whole launch");
   static_assert(!PAIR || FM % 2 == 0, "pairs of token blocks");
@@ -580,25 +588,35 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // tiles and the weight tiles of that rectangle, and the L2 fetches each of them once.  Inside
   // the rectangle the token tile runs fastest, so that the tiles in flight at any time reuse the
   // same few activation tiles while the weights stream through.
-  const int tiles_n = p.seg[MULTI ? p.segments - 1 : 0].tile_end;  // channel tiles of all matrices of the launch
+  const int tiles_n_all = p.seg[MULTI ? p.segments - 1 : 0].tile_end;  // channel tiles of all matrices of the launch
+  const int tiles_n = DUAL ? (tiles_n_all + 1) / 2 : tiles_n_all;        // channel tiles of the grid
   const int tiles_m = (p.m + BM - 1) / BM;
   const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
   const int xm = p.xcd_m, xn = 8 / xm;
   const int rect_m = (tiles_m + xm - 1) / xm, rect_n = (tiles_n + xn - 1) / xn;
   const int tm = (xcd % xm) * rect_m + local % rect_m;
-  int tn = (xcd / xm) * rect_n + local / rect_m, si = 0;
-  if (tm >= tiles_m || tn >= tiles_n) return;
-  if (MULTI && p.segments > 1 && tn >= p.seg[0].tile_end) {
-    si = (p.segments > 2 && tn >= p.seg[1].tile_end) ? 2 : 1;
-    tn -= p.seg[si - 1].tile_end;
-  }
-  constexpr int KW = GATED ? WAVES / 2 : WAVES;  // waves that share one matrix's K
-  const int half = GATED ? __builtin_amdgcn_readfirstlane(wave / KW) : 0;
+  const int tn_grid = (xcd / xm) * rect_n + local / rect_m;
+  if (tm >= tiles_m || tn_grid >= tiles_n) return;
+  // channel tile of the launch -> matrix of the launch (return value) and tile inside it
+  auto locate = [&](int& tile) {
+    int seg_index = 0;
+    if (MULTI && p.segments > 1 && tile >= p.seg[0].tile_end) {
+      seg_index = (p.segments > 2 && tile >= p.seg[1].tile_end) ? 2 : 1;
+      tile -= p.seg[seg_index - 1].tile_end;
+    }
+    return seg_index;
+  };
+  constexpr int KW = MODE != kModePlain ? WAVES / 2 : WAVES;  // waves that share one tile's K
+  const int half = MODE != kModePlain ? __builtin_amdgcn_readfirstlane(wave / KW) : 0;
+  int tn = DUAL ? 2 * tn_grid + half : tn_grid;
+  const bool tile_ok = !DUAL || tn < tiles_n_all;  // the last pair of an odd count has one tile
+  if (!tile_ok) tn = 0;
+  const int si = locate(tn);
   const W4Segment& sg = p.seg[GATED ? half : (MULTI ? si : 0)];
   const int slice0 = tn * (BN / 4);  // first output slice of the tile
   const int m0 = tm * BM;
   const int nsi = slice0 + i32;
-  const bool n_ok = nsi < sg.ns;
+  const bool n_ok = tile_ok && nsi < sg.ns;
 
   // This wave's range of 16-channel steps.  The buffer descriptors of the weights and the
   // activations end where the wave's share of K ends, so the prefetches that run past it (and
@@ -789,10 +807,33 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // 8*(v/4) + 4*g2 + v%4 and token i32, and the four MFMAs hold the slice's four channels: one
   // 8-byte store.
   // GATED: copies 0 .. KW-1 are gate's, the others up's; the two sums are rounded to fp16 (+ bias)
-  // as the two FullyConnected nodes would store them, then combined in fp32.
-  const __half* bias = GATED ? p.seg[0].bias : sg.bias;
-  const __half* bias_up = p.seg[GATED ? 1 : 0].bias;
-  __half* dst = GATED ? p.seg[0].dst : sg.dst;
+  // as the two FullyConnected nodes would store them, then combined in fp32.  DUAL: the two sums
+  // belong to the two tiles of the work-group.
+  int tile_b = 2 * tn_grid + 1;  // DUAL: the second tile
+  const bool tile_b_ok = DUAL && tile_b < tiles_n_all;
+  if (!tile_b_ok) tile_b = 0;
+  int tile_a = DUAL ? 2 * tn_grid : tn;
+  const int seg_a = DUAL ? locate(tile_a) : si, seg_b = DUAL ? locate(tile_b) : 0;
+  const W4Segment& sga = p.seg[GATED ? 0 : (MULTI ? seg_a : 0)];
+  const W4Segment& sgb = p.seg[GATED ? 1 : (MULTI ? seg_b : 0)];
+  const int slice0_a = DUAL ? tile_a * (BN / 4) : slice0, slice0_b = tile_b * (BN / 4);
+  // one slice of four channels of one token: the K-split partial sums, or the fp16 result
+  auto store = [&](const W4Segment& sgx, int slice, int mi, const float4& sum) {
+    if (p.ksplit > 1) {
+      // this work-group's share of K: fp32 sums for the second pass
+      *reinterpret_cast<float4*>(sgx.partial + (((size_t)blockIdx.y * sgx.ns + slice) * p.m + mi) * 4) = sum;
+      return;
+    }
+    __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
+    if (sgx.bias) {
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) h[t4] = __hadd(h[t4], sgx.bias[slice * 4 + t4]);
+    }
+    u32x2 o;
+    o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+    o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+    *reinterpret_cast<u32x2*>(sgx.dst + ((size_t)slice * p.m + mi) * 4) = o;
+  };
   static_assert(16 % RPH == 0 && RPH % WAVES == 0, "phases tile the 16 registers, waves tile a phase");
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
@@ -819,75 +860,77 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
           sum.w += o.w;
         }
         const int v = ph * RPH + j;
-        const int slice = slice0 + 8 * (v >> 2) + 4 * g2 + (v & 3);
-        const bool in_range = mi < p.m && slice < sg.ns;
-        if constexpr (GATED) {
-          float4 sum_up = red[buf][KW][j][lane];
+        const int slice_l = 8 * (v >> 2) + 4 * g2 + (v & 3);  // slice inside the tile
+        if constexpr (MODE != kModePlain) {
+          float4 sum_b = red[buf][KW][j][lane];
 #pragma unroll
           for (int c = KW + 1; c < WAVES; ++c) {
             const float4 o = red[buf][c][j][lane];
-            sum_up.x += o.x;
-            sum_up.y += o.y;
-            sum_up.z += o.z;
-            sum_up.w += o.w;
+            sum_b.x += o.x;
+            sum_b.y += o.y;
+            sum_b.z += o.z;
+            sum_b.w += o.w;
           }
-          if (in_range) {
-            const float g[4] = {sum.x, sum.y, sum.z, sum.w}, up[4] = {sum_up.x, sum_up.y, sum_up.z, sum_up.w};
+          if (DUAL) {
+            if (mi < p.m && slice0_a + slice_l < sga.ns) store(sga, slice0_a + slice_l, mi, sum);
+            if (mi < p.m && tile_b_ok && slice0_b + slice_l < sgb.ns) store(sgb, slice0_b + slice_l, mi, sum_b);
+          } else if (mi < p.m && slice0 + slice_l < sga.ns) {
+            const int slice = slice0 + slice_l;
+            const float g[4] = {sum.x, sum.y, sum.z, sum.w}, up[4] = {sum_b.x, sum_b.y, sum_b.z, sum_b.w};
             __half h[4];
 #pragma unroll
             for (int t4 = 0; t4 < 4; ++t4) {
               __half hg = __float2half_rn(g[t4]), hu = __float2half_rn(up[t4]);
-              if (bias) hg = __hadd(hg, bias[slice * 4 + t4]);
-              if (bias_up) hu = __hadd(hu, bias_up[slice * 4 + t4]);
+              if (sga.bias) hg = __hadd(hg, sga.bias[slice * 4 + t4]);
+              if (sgb.bias) hu = __hadd(hu, sgb.bias[slice * 4 + t4]);
               h[t4] = __float2half_rn(GatedActivation(p.gate_activation, __half2float(hg), __half2float(hu)));
             }
             u32x2 o;
             o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
             o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-            *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+            *reinterpret_cast<u32x2*>(sga.dst + ((size_t)slice * p.m + mi) * 4) = o;
           }
-        } else if (in_range && p.ksplit > 1) {
-          // this work-group's share of K: fp32 sums for the second pass
-          *reinterpret_cast<float4*>(sg.partial + (((size_t)blockIdx.y * sg.ns + slice) * p.m + mi) * 4) = sum;
-        } else if (in_range) {
-          __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
-          if (bias) {
-#pragma unroll
-            for (int t4 = 0; t4 < 4; ++t4) h[t4] = __hadd(h[t4], bias[slice * 4 + t4]);
-          }
-          u32x2 o;
-          o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
-          o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-          *reinterpret_cast<u32x2*>(dst + ((size_t)slice * p.m + mi) * 4) = o;
+        } else if (mi < p.m && slice0 + slice_l < sg.ns) {
+          store(sg, slice0 + slice_l, mi, sum);
         }
       }
     }
   }
 }
 
-template <int WB, int FM, int U, int WAVES, bool PAIR>
+template <int WB, int FM, int U, int WAVES, bool PAIR, int MODE>
 void LaunchDirectW(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
   const dim3 block(WAVES * 64);
   if (zp && p.segments > 1)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, true, MODE>), grid, block, 0, stream, p);
   else if (zp)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, true, PAIR, false, MODE>), grid, block, 0, stream, p);
   else if (p.segments > 1)
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, true, MODE>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<WB, FM, U, WAVES, false, PAIR, false, MODE>), grid, block, 0, stream, p);
 }
-template <int FM, int U, int WAVES, bool PAIR>
+// DUAL_OK: the two-tile mode is compiled for this shape.
+template <int FM, int U, int WAVES, bool PAIR, bool DUAL_OK>
 void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
   if (p.gate_activation != 0) {  // gated pair: uint4, symmetric
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<4, FM, U, WAVES, false, PAIR, false, true>), grid, dim3(WAVES * 64), 0,
-                       stream, p);
+    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<4, FM, U, WAVES, false, PAIR, false, kModeGated>), grid,
+                       dim3(WAVES * 64), 0, stream, p);
     return;
   }
+  if constexpr (DUAL_OK) {
+    if (p.dual) {
+      if (weight_bits == 8)
+        LaunchDirectW<8, FM, U, WAVES, PAIR, kModeDual>(zp, grid, stream, p);
+      else
+        LaunchDirectW<4, FM, U, WAVES, PAIR, kModeDual>(zp, grid, stream, p);
+      return;
+    }
+  }
   if (weight_bits == 8)
-    LaunchDirectW<8, FM, U, WAVES, PAIR>(zp, grid, stream, p);
+    LaunchDirectW<8, FM, U, WAVES, PAIR, kModePlain>(zp, grid, stream, p);
   else
-    LaunchDirectW<4, FM, U, WAVES, PAIR>(zp, grid, stream, p);
+    LaunchDirectW<4, FM, U, WAVES, PAIR, kModePlain>(zp, grid, stream, p);
 }
 
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
@@ -1075,20 +1118,31 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
   for (int i = 0; i < count; ++i)
     while (p.ksplit > 1 && (size_t)p.ksplit * p.seg[i].ns * 4 * a.m > args[i].partial_floats) p.ksplit /= 2;
   const int tiles_m = DivUp(a.m, fm * 32);
+  const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
+  // Two channel tiles per work-group when the rounds of 256 work-groups come out cheaper: a
+  // two-tile work-group takes 1.87 x the time of a one-tile one, and a last round filled to the
+  // fraction f costs 0.45 + 0.55 f of a full one (fitted to same-box timings of 14 shapes).
+  const bool dual_ok = !gated && pair && fm >= 2 && p.ksplit == 1;
+  auto rounds = [](long work_groups) {
+    const double r = work_groups / 256.0, whole = std::floor(r), f = r - whole;
+    return whole + (f > 0.0 ? 0.45 + 0.55 * f : 0.0);
+  };
+  p.dual = dual_ok && 1.87 * rounds((long)DivUp(tiles_n, 2) * tiles_m) < 0.97 * rounds((long)tiles_n * tiles_m);
+  if (const char* e = std::getenv("MLDHIP_GEMM_DUAL")) p.dual = dual_ok && std::atoi(e) != 0;
+  if (p.dual) tiles_n = DivUp(tiles_n, 2);
   p.xcd_m = W4XcdGrid(tiles_m, tiles_n, fm * 32, a.k, p.groups);
   if (const char* e = std::getenv("MLDHIP_GEMM_XCD_M")) p.xcd_m = std::atoi(e);
   if (p.xcd_m != 1 && p.xcd_m != 2 && p.xcd_m != 4 && p.xcd_m != 8) p.xcd_m = 8;
   const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
   const bool zp = p.seg[0].zp != nullptr;
-  const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
   if (fm == 4)
-    LaunchDirect<4, 4, 4, true>(a.weight_bits, zp, grid, stream, p);
+    LaunchDirect<4, 4, 4, true, true>(a.weight_bits, zp, grid, stream, p);
   else if (fm == 2 && pair)
-    LaunchDirect<2, 4, 8, true>(a.weight_bits, zp, grid, stream, p);
+    LaunchDirect<2, 4, 8, true, true>(a.weight_bits, zp, grid, stream, p);
   else if (fm == 2)
-    LaunchDirect<2, 4, 8, false>(a.weight_bits, zp, grid, stream, p);
+    LaunchDirect<2, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);
   else
-    LaunchDirect<1, 4, 8, false>(a.weight_bits, zp, grid, stream, p);
+    LaunchDirect<1, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);
   if (p.ksplit > 1) {
     size_t items = 0;
     for (int i = 0; i < count; ++i) items += (size_t)p.seg[i].ns * a.m;

@@ -100,6 +100,62 @@ def test_gemm_fractional_zero_points(oracle, bits, m, k, n, groups):
     check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
 
 
+@pytest.mark.parametrize("bits,m,k,n,groups,zp", [(4, 64, 512, 384, 4, False),    # 3 channel tiles: the last pair holds one
+                                                  (4, 130, 352, 1000, 11, True),   # ragged channels and tokens, 64-token tile
+                                                  (4, 256, 96, 260, 1, False),
+                                                  (8, 128, 1024, 640, 8, True),
+                                                  (4, 4096, 64, 2048, 2, True),    # 128-token tile
+                                                  (8, 2050, 96, 1100, 1, False)])
+def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp, monkeypatch):
+    """The two-tile mode (half of a work-group's waves per channel tile), forced on shapes of test
+    size: odd tile counts, ragged edges, zero points, both weight types, both token tiles; and
+    the same bytes as the one-tile mode where the K shares coincide is not required - the bar is
+    the FullyConnected one."""
+    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "1")
+    case = W.make_fc_case(seed=m + n + bits, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True, with_zero_point=zp)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+    small = min(m, 64)
+    sub = dict(case, m=small, act=case["act"][:small])
+    if small * k * n <= 1 << 26:
+        check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+
+
+def test_gemm_two_tiles_fused_launch(monkeypatch):
+    """Three matrices in one two-tile launch: pairs of tiles that straddle two matrices (3 + 1 + 2
+    channel tiles) against the single one-tile launches."""
+    import torch
+    m, k = 128, 512
+    cases = [W.make_fc_case(seed=60 + i, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=4, with_bias=True)
+             for i, n in enumerate((384, 100, 256))]
+    for c in cases[1:]:
+        c["act"] = cases[0]["act"]
+    devs = [W.FcDevice(c) for c in cases]
+    for d in devs[1:]:
+        d.op.set_src(0, devs[0].act)
+    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "0")
+    single = []
+    for d in devs:
+        d.run()
+        single.append(d.result())
+        d.out.zero_()
+    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "1")
+    M.fc_launch_fused([d.op for d in devs], torch.cuda.current_stream().cuda_stream)
+    for d, c, ref in zip(devs, cases, single):
+        got = d.result()
+        check_fp(got, textbook(c), c, "two-tile fused")
+        rms = np.sqrt(np.mean(textbook(c) ** 2))
+        assert np.abs(got - ref).max() <= 2e-3 * rms  # another K split among the waves: fp32 summation order
+
+
+def test_gemm_two_tiles_chosen_for_large_launches():
+    """4096 x 4096 x 4096 (1024 tiles) runs in the two-tile mode by default and meets the bar."""
+    case = W.make_fc_case(seed=5, m=4096, k=4096, n=4096, weight_bits=4, tensor_dtype=np.float16, groups=1)
+    got = run_w4(case)
+    check_fp(got, textbook(case), case, "textbook")
+
+
 def test_w8_gemm_fused_launch():
     """Three uint8 matrices over one activation tensor in one launch give the bytes of the three
     single launches; a uint4 op cannot join them."""
