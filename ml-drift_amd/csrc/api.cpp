@@ -93,6 +93,10 @@ struct mldhip_op {
   mldhip_quant_desc q{};
   mldhip_conv_int8_desc cv{};
   int idx_scale = -1, idx_zp = -1, idx_bias = -1;
+  // FullyConnected with batched weights selected by a runtime tensor of ids
+  int idx_weights = 1, idx_ids = -1;
+  int weights_batch = 1;  // ExternalWeights::shape.h
+  int shared_src = 0;     // the source tensor has one row that every dst row reads
   float* partial = nullptr;
   size_t partial_floats = 0;
   const char* last_kernel = "";
@@ -257,24 +261,30 @@ static uint16_t FloatToHalfBits(float f) {
   return (uint16_t)(sign | q);
 }
 
-int mldhip_scale_to_tensor(const float* scale, int o, int groups, int dst_type, void* dst, size_t dst_bytes) {
+int mldhip_scale_to_tensor_batched(const float* scale, int o, int batch, int groups, int dst_type, void* dst,
+                                   size_t dst_bytes) {
   if (!scale || !dst) return Fail(MLDHIP_INVALID_ARGUMENT, "null buffer");
-  if (o <= 0 || groups <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad scale shape");
+  if (o <= 0 || groups <= 0 || batch <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad scale shape");
   if (dst_type != MLDHIP_FLOAT16 && dst_type != MLDHIP_FLOAT32)
     return Fail(MLDHIP_INVALID_ARGUMENT, "scale tensor type must be FLOAT16 or FLOAT32");
   const int os = DivUp(o, 4);
-  const size_t count = (size_t)groups * os * 4;
+  const size_t count = (size_t)groups * batch * os * 4;
   if (dst_bytes < count * TypeBytes(dst_type)) return Fail(MLDHIP_INVALID_ARGUMENT, "destination too small");
   for (int g = 0; g < groups; ++g)
-    for (int oc = 0; oc < os * 4; ++oc) {
-      const float v = oc < o ? scale[(size_t)oc * groups + g] : 0.0f;
-      const size_t idx = (size_t)g * os * 4 + oc;
-      if (dst_type == MLDHIP_FLOAT32)
-        static_cast<float*>(dst)[idx] = v;
-      else
-        static_cast<uint16_t*>(dst)[idx] = FloatToHalfBits(v);
-    }
+    for (int b = 0; b < batch; ++b)
+      for (int oc = 0; oc < os * 4; ++oc) {
+        const float v = oc < o ? scale[((size_t)oc * batch + b) * groups + g] : 0.0f;
+        const size_t idx = ((size_t)g * batch + b) * os * 4 + oc;
+        if (dst_type == MLDHIP_FLOAT32)
+          static_cast<float*>(dst)[idx] = v;
+        else
+          static_cast<uint16_t*>(dst)[idx] = FloatToHalfBits(v);
+      }
   return MLDHIP_OK;
+}
+
+int mldhip_scale_to_tensor(const float* scale, int o, int groups, int dst_type, void* dst, size_t dst_bytes) {
+  return mldhip_scale_to_tensor_batched(scale, o, 1, groups, dst_type, dst, dst_bytes);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -296,9 +306,12 @@ static int AllocWorkspace(mldhip_op* op, int n) {
   return MLDHIP_OK;
 }
 
-int mldhip_fc_create(const mldhip_fc_desc* d, mldhip_op** out) {
+static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, int shared_src, mldhip_op** out) {
   if (!d || !out) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
   *out = nullptr;
+  if (batch_ids && weights_batch < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "weights_batch must be positive");
+  if (batch_ids && d->src_type == MLDHIP_INT8)
+    return Fail(MLDHIP_UNIMPLEMENTED, "batched weights are served for floating-point tensors");
   if (d->o <= 0 || d->i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
   if (d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "max_tokens must be positive");
   const mldhip_weights_desc& wd = d->weights;
@@ -341,6 +354,13 @@ int mldhip_fc_create(const mldhip_fc_desc* d, mldhip_op** out) {
   op->fc = *d;
   op->max_tokens = d->max_tokens;
   op->AddSrc("src_tensor");
+  if (batch_ids) {  // registered before the weights objects (fully_connected.cc:1203-1208)
+    op->idx_ids = (int)op->src_names.size();
+    op->AddSrc("batch_ids");
+    op->weights_batch = weights_batch;
+    op->shared_src = shared_src ? 1 : 0;
+  }
+  op->idx_weights = (int)op->src_names.size();
   op->AddSrc("weights");
   if (!int8_math && d->scale_o * d->scale_i > 1) {
     op->idx_scale = (int)op->src_names.size();
@@ -357,6 +377,12 @@ int mldhip_fc_create(const mldhip_fc_desc* d, mldhip_op** out) {
   op->AddDst("dst_tensor");
   *out = op;
   return MLDHIP_OK;
+}
+
+int mldhip_fc_create(const mldhip_fc_desc* d, mldhip_op** out) { return CreateFc(d, false, 1, 0, out); }
+
+int mldhip_fc_batch_ids_create(const mldhip_fc_desc* d, int weights_batch, int shared_src, mldhip_op** out) {
+  return CreateFc(d, true, weights_batch, shared_src, out);
 }
 
 int mldhip_quantization_create(const mldhip_quant_desc* d, mldhip_op** out) {
@@ -457,6 +483,7 @@ int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w) {
   if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
   if (b <= 0 || h <= 0 || w <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "shape must be positive");
   if ((long long)b * h * w > op->max_tokens) return Fail(MLDHIP_OUT_OF_RANGE, "b*h*w exceeds max_tokens");
+  if (op->idx_ids >= 0 && b != 1) return Fail(MLDHIP_UNIMPLEMENTED, "batched weights: the tensors have batch 1");
   op->b = b;
   op->h = h;
   op->w = w;
@@ -471,11 +498,14 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
   if (op->kind == mldhip_op::kFc) {
     const mldhip_fc_desc& d = op->fc;
     const size_t ks = DivUp(d.i, 4), ns = DivUp(d.o, 4);
-    (*src)[0] = ks * m * 4 * TypeBytes(d.src_type);
-    (*src)[1] = ks * ns * 16 * WeightBits(d.weights.type) / 8;
+    const size_t wbatch = (size_t)op->weights_batch;
+    // batched weights: h rows of w tokens; a shared source has one row
+    (*src)[0] = ks * (op->shared_src ? (size_t)op->w : m) * 4 * TypeBytes(d.src_type);
+    if (op->idx_ids >= 0) (*src)[op->idx_ids] = (size_t)op->h * sizeof(int32_t);
+    (*src)[op->idx_weights] = wbatch * ks * ns * 16 * WeightBits(d.weights.type) / 8;
     const size_t tb = TypeBytes(d.src_type);
-    if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * ns * 4 * tb;
-    if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * ns * 4 * tb;
+    if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
+    if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
     (*dst)[0] = ns * m * 4 * TypeBytes(d.dst_type);
   } else if (op->kind == mldhip_op::kQuant) {
@@ -530,12 +560,19 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
   const mldhip_fc_desc& d = op->fc;
   FcArgs a;
   a.act = op->src_ptr[0];
-  a.weights = static_cast<const uint8_t*>(op->src_ptr[1]);
+  a.weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
   a.scale = op->idx_scale >= 0 ? op->src_ptr[op->idx_scale] : nullptr;
   a.zero_point = op->idx_zp >= 0 ? op->src_ptr[op->idx_zp] : nullptr;
   a.bias = op->idx_bias >= 0 ? op->src_ptr[op->idx_bias] : nullptr;
   a.dst = op->dst_ptr[0];
   a.m = op->Tokens();
+  if (op->idx_ids >= 0) {
+    a.batch_ids = static_cast<const int32_t*>(op->src_ptr[op->idx_ids]);
+    a.rows = op->h;
+    a.src_rows = op->shared_src ? 1 : op->h;
+    a.weights_batch = op->weights_batch;
+    a.m = op->w;  // tokens per row
+  }
   a.k = d.i;
   a.n = d.o;
   a.act_f16 = d.src_type == MLDHIP_FLOAT16;
@@ -576,7 +613,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
-      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
+      // (batched weights by runtime ids: the unspecialised kernel)
+      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC") || a.batch_ids != nullptr;
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
       // on the vector-ALU kernel; MLDHIP_GEMV_MFMA=1 forces the matrix-core one there too)
       if (!force_generic && (a.m >= 2 || EnvFlag("MLDHIP_GEMV_MFMA")) && FcW4MfmaStreamSupported(a)) {
@@ -636,8 +674,8 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
   for (int i = 0; i < count; ++i) {
     mldhip_op* op = ops[i];
     if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
-    if (op->kind != mldhip_op::kFc || op->fc.src_type == MLDHIP_INT8)
-      return Fail(MLDHIP_FAILED_PRECONDITION, "fused launch takes floating-point FullyConnected ops");
+    if (op->kind != mldhip_op::kFc || op->fc.src_type == MLDHIP_INT8 || op->idx_ids >= 0)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "fused launch takes floating-point FullyConnected ops without batched weights");
     if (int rc = CheckBindings(op)) return rc;
     if (int rc = BuildFcArgs(op, &args[i])) return rc;
     const FcArgs &a = args[i], &f = args[0];
@@ -665,8 +703,8 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
   mldhip_op* ops[2] = {gate, up};
   FcArgs args[2];
   for (int i = 0; i < 2; ++i) {
-    if (ops[i]->kind != mldhip_op::kFc || ops[i]->fc.src_type == MLDHIP_INT8)
-      return Fail(MLDHIP_FAILED_PRECONDITION, "gated launch takes floating-point FullyConnected ops");
+    if (ops[i]->kind != mldhip_op::kFc || ops[i]->fc.src_type == MLDHIP_INT8 || ops[i]->idx_ids >= 0)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "gated launch takes floating-point FullyConnected ops without batched weights");
     if (int rc = CheckBindings(ops[i])) return rc;
     if (int rc = BuildFcArgs(ops[i], &args[i])) return rc;
   }

@@ -49,6 +49,10 @@ struct GenericParams {
   int scale_kind, groups, group_slices;
   float scalar_scale, scalar_zero_point;
   int has_zero_point;
+  // batched weights by runtime ids (fully_connected.cc:654-665, 804-822; fully_connected_util.cc:
+  // 279-290): blockIdx.z = dst row; m = tokens per row
+  const int32_t* batch_ids;
+  int rows, src_rows, weights_batch;
 };
 
 template <typename ActT, typename DstT, int WBITS, int TB>
@@ -61,6 +65,15 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
   const ActT* scale = static_cast<const ActT*>(p.scale);
   const ActT* zp = static_cast<const ActT*>(p.zero_point);
   const float shift = WBITS == 8 ? 128.0f : 8.0f;
+  // Row of the launch: its weight matrix, its source row (one shared row is broadcast) and the
+  // token strides of the two tensors.  An id outside the batch is clamped into it (the reference
+  // reads whatever lies there).
+  const int row = blockIdx.z;
+  int wb = p.batch_ids ? p.batch_ids[row] : 0;
+  wb = min(max(wb, 0), p.weights_batch - 1);
+  const size_t act_stride = (size_t)p.src_rows * p.m, dst_stride = (size_t)p.rows * p.m;
+  const size_t act_tok0 = (size_t)min(row, p.src_rows - 1) * p.m, dst_tok0 = (size_t)row * p.m;
+  const uint8_t* weights = p.weights + (size_t)wb * p.ks * p.ns * (WBITS == 8 ? 16 : 8);
 
   float acc[TB][4];
 #pragma unroll
@@ -78,8 +91,8 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
     if (p.scale_kind == kScaleLinear) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        s[c] = LoadF(scale, (size_t)ds * 4 + c);
-        if (zp) z[c] = LoadF(zp, (size_t)ds * 4 + c);
+        s[c] = LoadF(scale, ((size_t)wb * p.ns + ds) * 4 + c);
+        if (zp) z[c] = LoadF(zp, ((size_t)wb * p.ns + ds) * 4 + c);
       }
     }
 #pragma unroll 4
@@ -87,7 +100,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
       if (p.scale_kind == kScaleBlock) {
         int g = ks / p.group_slices;
         if (g >= p.groups) g = p.groups - 1;
-        const size_t sidx = ((size_t)g * p.ns + ds) * 4;
+        const size_t sidx = (((size_t)g * p.weights_batch + wb) * p.ns + ds) * 4;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           s[c] = LoadF(scale, sidx + c);
@@ -97,14 +110,14 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
       const size_t blk = (size_t)ks * p.ns + ds;
       float wf[4][4];
       if (WBITS == 8) {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(p.weights + blk * 16);
+        const u32x4 w = *reinterpret_cast<const u32x4*>(weights + blk * 16);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int c = 0; c < 4; ++c)
             wf[i][c] = ((float)((w[i] >> (8 * c)) & 0xFFu) - (shift + z[c])) * s[c];
       } else {
-        const u32x2 w = *reinterpret_cast<const u32x2*>(p.weights + blk * 8);
+        const u32x2 w = *reinterpret_cast<const u32x2*>(weights + blk * 8);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -117,7 +130,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
         if (tok < p.m) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float a = LoadF(act, ((size_t)ks * p.m + tok) * 4 + i);
+            const float a = LoadF(act, ((size_t)ks * act_stride + act_tok0 + tok) * 4 + i);
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[t][c] = fmaf(a, wf[i][c], acc[t][c]);
           }
@@ -142,7 +155,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
         float r = 0.0f;
 #pragma unroll
         for (int q = 0; q < kKl; ++q) r += red[q][tx][t * 4 + c];
-        StoreOut(dst, ((size_t)ds * p.m + tok) * 4 + c, r, bias, (size_t)ds * 4 + c);
+        StoreOut(dst, ((size_t)ds * dst_stride + dst_tok0 + tok) * 4 + c, r, bias, (size_t)ds * 4 + c);
       }
     }
   }
@@ -151,7 +164,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 template <typename ActT, typename DstT, int WBITS>
 hipError_t LaunchGenericT(const GenericParams& p, hipStream_t stream) {
   constexpr int TB = 4;
-  dim3 grid(DivUp(p.ns, kSl), DivUp(p.m, TB));
+  dim3 grid(DivUp(p.ns, kSl), DivUp(p.m, TB), p.rows);
   dim3 block(kSl, kKl);
   hipLaunchKernelGGL((fc_generic_kernel<ActT, DstT, WBITS, TB>), grid, block, 0, stream, p);
   return hipGetLastError();
@@ -273,6 +286,10 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
   p.scalar_scale = a.scalar_scale;
   p.scalar_zero_point = a.scalar_zero_point;
   p.has_zero_point = a.has_zero_point;
+  p.batch_ids = a.batch_ids;
+  p.rows = a.rows;
+  p.src_rows = a.src_rows;
+  p.weights_batch = a.weights_batch;
   if (kernel_name) *kernel_name = "fc_generic_kernel";
   const bool w8 = a.weight_bits == 8;
   if (a.act_f16 && a.dst_f16)

@@ -32,6 +32,13 @@ struct FcArgs {
   // private workspace of the op (split-K partial sums)
   float* partial = nullptr;
   size_t partial_floats = 0;
+  // Batched weights selected by a runtime tensor of ids (the reference's
+  // CreateFullyConnectedWeightsBatchIds): dst row y (of `rows`, m tokens each) = FC of src row
+  // min(y, src_rows - 1) with weight matrix batch_ids[y] of `weights_batch`.  The packed buffer
+  // holds the matrices one after the other, scales are [groups][weights_batch][Ns][4].
+  // Plain launches: batch_ids = nullptr, rows = src_rows = weights_batch = 1.
+  const int32_t* batch_ids = nullptr;
+  int rows = 1, src_rows = 1, weights_batch = 1;
 };
 
 // Split-K workspace sizing for the streaming GEMV.

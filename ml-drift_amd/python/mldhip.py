@@ -31,6 +31,7 @@ SYMBOLS = [
     "mldhip_op_set_src", "mldhip_op_set_dst", "mldhip_op_set_shape", "mldhip_op_launch",
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
+    "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
 ]
 
 
@@ -227,6 +228,16 @@ def scale_to_tensor(scale, dst_type):
     return out
 
 
+def scale_to_tensor_batched(scale, dst_type):
+    """scale: (o, batch, groups) float32 -> [groups][batch][ceil(o/4)][4] tensor buffer."""
+    s = np.ascontiguousarray(scale, np.float32)
+    o, batch, groups = s.shape
+    dt = np.uint16 if dst_type == FLOAT16 else np.float32
+    out = np.empty(groups * batch * div_up(o, 4) * 4, dt)
+    check(lib().mldhip_scale_to_tensor_batched(_p(s), o, batch, groups, dst_type, _p(out), C.c_size_t(out.nbytes)))
+    return out
+
+
 # ---- checkpoint files (host) ----
 def checkpoint_fc_probe(directory, weights_name, base_name, o, i, weight_bits):
     """-> CheckpointFc (weights description, group size, zero-point presence, buffer sizes)."""
@@ -334,7 +345,8 @@ def fc_launch_gated(gate, up, activation, dst, stream=0):
 
 def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1, 1),
               scalar_scale=1.0, has_zero_point_tensor=False, scalar_zero_point=None,
-              has_bias=False, max_tokens=1):
+              has_bias=False, max_tokens=1, weights_batch=None, shared_src=False):
+    """weights_batch: number of weight matrices of a batch-ids op (mldhip_fc_batch_ids_create)."""
     d = FcDesc()
     d.precision, d.src_type, d.dst_type, d.o, d.i = precision, src_type, dst_type, o, i
     d.weights = weights_desc
@@ -346,7 +358,10 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
     d.has_bias = int(has_bias)
     d.max_tokens = max_tokens
     h = C.c_void_p()
-    check(lib().mldhip_fc_create(C.byref(d), C.byref(h)))
+    if weights_batch is not None:
+        check(lib().mldhip_fc_batch_ids_create(C.byref(d), weights_batch, int(shared_src), C.byref(h)))
+    else:
+        check(lib().mldhip_fc_create(C.byref(d), C.byref(h)))
     return Op(h)
 
 

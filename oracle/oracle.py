@@ -194,6 +194,17 @@ def scale_to_hoio4(scale_ohi):
     return np.ascontiguousarray(out.reshape(div_up(o, 4), i, 4).transpose(1, 0, 2))
 
 
+def scale_to_hoio4_batched(scale_obi):
+    """(O, batch, I) float scales -> [I groups][batch][ceil(O/4)][4] float, zero padded: the HWC
+    tensor (h = batch, w = O slices, c = 4*I) of OHIToHOIO4 (common/task/tensor_desc.cc:267-292) in
+    the buffer order [slice of c][h][w][4] (task/tensor_desc.cc:1841-1873)."""
+    s = _c(scale_obi, np.float32)
+    o, b, i = s.shape
+    out = np.empty((b, div_up(o, 4), 4 * i), np.float32)
+    lib().mldo_scale_to_hoio4(_p(s), o, b, i, _p(out))
+    return np.ascontiguousarray(out.reshape(b, div_up(o, 4), i, 4).transpose(2, 0, 1, 3))
+
+
 # ---- FullyConnected ----
 def fc_kernel(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=SCALE_LINEAR,
               scale=None, zero_point=None, bias=None, groups=1, use_fma=True, wg_y=1,
@@ -213,6 +224,55 @@ def fc_kernel(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=S
     bi = None if bias is None else _c(bias, tdt)
     out = np.empty((div_up(n, 4), m, 4), tdt)
     lib().mldo_fc_kernel(C.byref(p), _p(act), _p(w), _p(sc), _p(zp), _p(bi), _p(out))
+    return out
+
+
+def fc_batch_ids_kernel(act_slices, ids, weights, rows, row_tokens, src_rows, weights_batch, k, n, precision,
+                        weight_bits, scale_kind=SCALE_LINEAR, scale=None, zero_point=None, bias=None, groups=1):
+    """The generated kernel with batched weights and runtime batch ids
+    (common/kernels/fully_connected.cc:654-665 w_batch_id, :482-560 the weight address offset
+    w_batch_id * Ks * Ns, :804-822 source row min(dst_h, Height - 1);
+    fully_connected_util.cc:80-125 scale / zero point read at (o_slice, w_batch_id, group),
+    :279-290 GetWeightsBatchId): every dst row is the plain kernel on that row's source tokens with
+    the selected matrix, so this restatement runs `fc_kernel` per row on views of the buffers.
+    act_slices [Ks][src_rows * row_tokens][4], result [Ns][rows * row_tokens][4];
+    weights: `weights_batch` packed matrices one after the other; scale / zero_point:
+    [groups][weights_batch][Ns][4]."""
+    tdt = np.float32 if precision == PREC_F32 else np.uint16
+    ks, ns = div_up(k, 4), div_up(n, 4)
+    act = _c(act_slices, tdt).reshape(ks, src_rows * row_tokens, 4)
+    w = _c(weights, np.uint8).reshape(weights_batch, -1)
+    sc = None if scale is None else _c(scale, tdt).reshape(groups, weights_batch, ns * 4)
+    zp = None if zero_point is None else _c(zero_point, tdt).reshape(groups, weights_batch, ns * 4)
+    out = np.empty((ns, rows * row_tokens, 4), tdt)
+    for y in range(rows):
+        e = int(ids[y])
+        sy = min(y, src_rows - 1)
+        a = np.ascontiguousarray(act[:, sy * row_tokens:(sy + 1) * row_tokens, :])
+        r = fc_kernel(a, w[e], row_tokens, k, n, precision, weight_bits, scale_kind,
+                      None if sc is None else np.ascontiguousarray(sc[:, e, :]),
+                      None if zp is None else np.ascontiguousarray(zp[:, e, :]), bias, groups)
+        out[:, y * row_tokens:(y + 1) * row_tokens, :] = r
+    return out
+
+
+def fc_batch_ids_reference_f32(src, weights_obi, ids):
+    """FullyConnectedWeightsBatchIdsReference (common/task/testing_ref_ops.cc:1042-1067): src
+    (src_rows, tokens, K) float, weights (O, batch, K) float -> (rows, tokens, O); a source with one
+    row is read by every dst row."""
+    src = np.asarray(src, np.float32)
+    w = np.asarray(weights_obi, np.float32)
+    rows = len(ids)
+    out = np.zeros((rows, src.shape[1], w.shape[0]), np.float32)
+    for y in range(rows):
+        sy = 0 if src.shape[0] == 1 else y
+        wm = w[:, int(ids[y]), :]
+        for x in range(src.shape[1]):
+            for d in range(w.shape[0]):
+                acc = np.float32(0.0)
+                for c in range(w.shape[2]):
+                    acc = np.float32(acc + src[sy, x, c] * wm[d, c])
+                out[y, x, d] = acc
     return out
 
 

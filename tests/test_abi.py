@@ -144,3 +144,34 @@ def test_header_is_plain_c(tmp_path):
     r = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only",
                         "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr
+
+
+def test_fc_batch_ids_object_order_and_validation():
+    # fully_connected.cc:1203-1213: batch_ids is registered before the weights objects
+    wd = M.fc_int8_weights_desc(32, 64)
+    op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 32, 64, wd, scale_shape=(32, 1), has_bias=True,
+                     max_tokens=128, weights_batch=16)
+    assert op.src_names == ["src_tensor", "batch_ids", "weights", "weights_scale", "biases"]
+    assert op.dst_names == ["dst_tensor"]
+    op.set_shape(1, 8, 2)
+    with pytest.raises(M.MldhipError) as e:   # tensors of a batch-ids op have batch 1
+        op.set_shape(2, 4, 1)
+    assert e.value.code == M.UNIMPLEMENTED
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 32, 64, wd, scale_shape=(32, 1), weights_batch=0)
+    assert e.value.code == M.INVALID_ARGUMENT
+    with pytest.raises(M.MldhipError) as e:   # the integer-math variant has no batched form here
+        M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 32, 64, wd, weights_batch=4)
+    assert e.value.code == M.UNIMPLEMENTED
+
+
+def test_scale_to_tensor_batched_matches_oracle(oracle):
+    import numpy as np
+    rng = np.random.default_rng(1)
+    s = rng.normal(size=(10, 3, 2)).astype(np.float32)
+    got = M.scale_to_tensor_batched(s, M.FLOAT32)
+    assert np.array_equal(got, oracle.scale_to_hoio4_batched(s).reshape(-1))
+    got16 = M.scale_to_tensor_batched(s, M.FLOAT16)
+    assert np.array_equal(got16, oracle.f32_to_f16_bits(oracle.scale_to_hoio4_batched(s).reshape(-1)))
+    # one matrix: the unbatched conversion
+    assert np.array_equal(M.scale_to_tensor_batched(s[:, :1, :], M.FLOAT32), M.scale_to_tensor(s[:, 0, :], M.FLOAT32))

@@ -1,0 +1,128 @@
+"""GPU parity of the FullyConnected with batched weights selected by runtime ids (the
+mixture-of-experts projection, CreateFullyConnectedWeightsBatchIds), through the C-ABI: against
+the oracle's restatement of the generated kernel and against the reference's float reference
+over dequantized weights.  fp32 tensors: 1.2e-7 * (K + 1) relative; fp16: 2e-2 of the output RMS."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mldhip as M
+import workloads as W
+from test_oracle_fc import batch_ids_float_weights, make_batch_ids_case, run_batch_ids_oracle
+
+FP16_TOL = 2e-2
+
+
+def run_device(c, td, bias=None, max_tokens=None):
+    import torch
+    tt = torch.float16 if td == np.float16 else torch.float32
+    mt = M.FLOAT16 if td == np.float16 else M.FLOAT32
+    n, k, batch = c["n"], c["k"], c["batch"]
+    ns = W.div_up(n, 4)
+    desc = (M.fc_int8_weights_desc if c["bits"] == 8 else M.fc_int4_weights_desc)(n, k)
+    packed = (M.rearrange_int8_as_uint8 if c["bits"] == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
+    src2 = c["src"].reshape(c["src_rows"] * c["row_tokens"], k)
+    act = torch.from_numpy(W.to_slices(src2).astype(td)).cuda()
+    ids = torch.from_numpy(c["ids"]).cuda()
+    weights = torch.from_numpy(packed).cuda()
+
+    def tensor(v):
+        t = M.scale_to_tensor_batched(v, mt)
+        return torch.from_numpy(t.view(td) if td == np.float16 else t).cuda()
+    srcs = [act, ids, weights, tensor(c["scale"])]
+    if c["zp"] is not None:
+        srcs.append(tensor(c["zp"]))
+    if bias is not None:
+        b = np.zeros(ns * 4, td)
+        b[:n] = bias
+        srcs.append(torch.from_numpy(b).cuda())
+    out = torch.zeros((ns, c["rows"] * c["row_tokens"], 4), dtype=tt, device="cuda")
+    precision = M.PRECISION_F32 if td == np.float32 else M.PRECISION_F32_F16
+    op = M.fc_create(precision, mt, mt, n, k, desc, scale_shape=(n, c["groups"]),
+                     has_zero_point_tensor=c["zp"] is not None, has_bias=bias is not None,
+                     max_tokens=max_tokens or c["rows"] * c["row_tokens"], weights_batch=batch,
+                     shared_src=c["src_rows"] == 1 and c["rows"] > 1)
+    op.bind(srcs, [out])
+    op.set_shape(1, c["rows"], c["row_tokens"])
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    got = W.from_slices(out.cpu().numpy().astype(np.float32), n).reshape(c["rows"], c["row_tokens"], n)
+    return got, op.kernel_name
+
+
+def check(c, td, got, oracle, bias=None):
+    ref = oracle.fc_batch_ids_reference_f32(c["src"].astype(td).astype(np.float32), batch_ids_float_weights(oracle, c),
+                                            c["ids"]).astype(np.float64)
+    if bias is not None:
+        ref = ref + np.asarray(bias, np.float64)
+    err = np.abs(got - ref).max()
+    if td == np.float16:
+        rms = np.sqrt(np.mean(ref ** 2))
+        assert err <= FP16_TOL * rms, (err, rms)
+    else:
+        tol = 1.1920929e-7 * (c["k"] + 1) * max(1.0, np.abs(ref).max())
+        assert err <= tol, (err, tol)
+
+
+@pytest.mark.parametrize("src_shape,ids_count", [((1, 1, 32), 1), ((8, 1, 32), 8), ((128, 1, 64), 128),
+                                                 ((1, 1, 32), 4)])
+@pytest.mark.parametrize("td", [np.float32, np.float16])
+def test_reference_test_shapes(oracle, src_shape, ids_count, td):
+    """fully_connected_test.cc:227-250 (32 channels, 16 int8 matrices; the last case broadcasts
+    one source row to 4 ids)."""
+    src_rows, row_tokens, k = src_shape
+    c = make_batch_ids_case(ids_count + k, ids_count, row_tokens, src_rows, k, 32, 16)
+    print("batch ids", src_shape, ids_count, td.__name__, flush=True)
+    got, name = run_device(c, td)
+    check(c, td, got, oracle)
+    if td == np.float32:  # and against the kernel restatement
+        ref = run_batch_ids_oracle(oracle, c, 0)
+        assert np.abs(got - ref).max() <= 1.1920929e-7 * (k + 1) * max(1.0, np.abs(ref).max())
+
+
+@pytest.mark.parametrize("bits,rows,row_tokens,src_rows,k,n,batch,groups,zp", [
+    (4, 8, 1, 1, 2048, 768, 8, 64, False),     # decode step of a mixture layer: one token, 8 of 8 experts, shared input
+    (4, 8, 1, 8, 768, 2048, 8, 24, False),     # its down projections: one input row per expert
+    (4, 5, 3, 5, 64, 20, 4, 2, True),          # several tokens per row, zero points, ragged channels
+    (8, 6, 2, 1, 171, 533, 3, 1, True),        # the reference's odd sizes
+    (4, 4, 7, 4, 352, 200, 128, 11, False),    # many matrices, few used
+])
+@pytest.mark.parametrize("td", [np.float16, np.float32])
+def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td):
+    c = make_batch_ids_case(rows * 7 + n, rows, row_tokens, src_rows, k, n, batch, bits, groups, zp)
+    rng = np.random.default_rng(n)
+    bias = (rng.uniform(-1, 1, size=n) * 0.1).astype(td).astype(np.float32)
+    print("batch ids", bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td.__name__, flush=True)
+    got, name = run_device(c, td, bias=bias)
+    check(c, td, got, oracle, bias=bias)
+
+
+def test_repeated_and_out_of_range_ids(oracle):
+    """The same matrix for several rows; an id outside the batch is clamped into it."""
+    c = make_batch_ids_case(1, rows=6, row_tokens=2, src_rows=6, k=64, n=32, batch=4)
+    c["ids"] = np.array([2, 2, 0, 3, 2, 0], np.int32)
+    got, _ = run_device(c, np.float32)
+    check(c, np.float32, got, oracle)
+    bad = dict(c, ids=np.array([7, -1, 0, 3, 2, 0], np.int32))
+    got_bad, _ = run_device(bad, np.float32)
+    clamped = dict(c, ids=np.array([3, 0, 0, 3, 2, 0], np.int32))
+    check(clamped, np.float32, got_bad, oracle)
+
+
+def test_bindings_are_checked():
+    import torch
+    c = make_batch_ids_case(2, rows=4, row_tokens=1, src_rows=4, k=64, n=32, batch=4)
+    desc = M.fc_int8_weights_desc(32, 64)
+    op = M.fc_create(M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 32, 64, desc, scale_shape=(32, 1), max_tokens=8,
+                     weights_batch=4)
+    op.set_shape(1, 4, 1)
+    small = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    big = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    op.bind([big, big, small, big], [big])   # weights of one matrix only
+    with pytest.raises(M.MldhipError) as e:
+        op.launch(torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == M.INVALID_ARGUMENT and "weights" in str(e.value)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_launch_fused([op])
+    assert e.value.code == M.FAILED_PRECONDITION

@@ -193,3 +193,104 @@ def test_gated_activation_known_values(oracle):
     silu = oracle.gated_activation(g, u, "silu").astype(np.float64)
     assert silu[0] == 0.0 and abs(silu[3] - 1 / (1 + np.exp(-1.0))) < 1e-3 and abs(silu[4] + 1 / (1 + np.exp(1.0))) < 1e-3
     assert abs(silu[1] - 16.0) < 2e-2 and abs(silu[2]) < 1e-2 and silu[5] == 65504.0
+
+
+# ---- batched weights selected by runtime ids (mixture-of-experts FullyConnected) ----
+def make_batch_ids_case(seed, rows, row_tokens, src_rows, k, n, batch, bits=8, groups=1, with_zp=False):
+    """Shapes of FullyConnectedInt8BatchedWeightsIdsBigTest (fully_connected_test_util.cc:1338-1380):
+    weights OHWI(n, batch, 1, k), scales OHWI(n, batch, 1, groups), ids random in [0, batch)."""
+    rng = np.random.default_rng(seed)
+    lim = 127 if bits == 8 else 7
+    w = rng.integers(-lim - (bits == 4), lim + 1, size=(n, batch, 1, k), dtype=np.int8)
+    scale = (np.abs(rng.normal(0.0, 1.0, size=(n, batch, groups))) / 128.0 + 1e-3).astype(np.float32)
+    zp = rng.integers(-3, 4, size=(n, batch, groups)).astype(np.float32) if with_zp else None
+    src = rng.uniform(-1, 1, size=(src_rows, row_tokens, k)).astype(np.float32)
+    ids = rng.integers(0, batch, size=rows).astype(np.int32)
+    return dict(w=w, scale=scale, zp=zp, src=src, ids=ids, rows=rows, row_tokens=row_tokens, src_rows=src_rows,
+                k=k, n=n, batch=batch, bits=bits, groups=groups)
+
+
+def batch_ids_float_weights(o, c):
+    """(n, batch, k) dequantized weights (MakeWeightsFromInt8 per matrix)."""
+    out = np.empty((c["n"], c["batch"], c["k"]), np.float32)
+    for e in range(c["batch"]):
+        zp = None if c["zp"] is None else c["zp"][:, e, :]
+        out[:, e, :] = o.make_weights_from_int8(c["w"][:, e, 0, :], c["scale"][:, e, :], zp)
+    return out
+
+
+def run_batch_ids_oracle(o, c, precision):
+    ns = (c["n"] + 3) // 4
+    pack = o.int8_as_uint8 if c["bits"] == 8 else o.int8_as_uint4
+    packed = pack(c["w"], I4O4, ns)
+    src2 = c["src"].reshape(c["src_rows"] * c["row_tokens"], c["k"])
+    act = tensor(o, o.to_slices(src2), precision)
+    kind = o.SCALE_LINEAR if c["groups"] == 1 else o.SCALE_BLOCK
+    sc = tensor(o, o.scale_to_hoio4_batched(c["scale"]), precision)
+    zp = None if c["zp"] is None else tensor(o, o.scale_to_hoio4_batched(c["zp"]), precision)
+    out = o.fc_batch_ids_kernel(act, c["ids"], packed, c["rows"], c["row_tokens"], c["src_rows"], c["batch"], c["k"],
+                                c["n"], precision, c["bits"], kind, sc, zp, None, c["groups"])
+    return o.from_slices(to_f32(o, out, precision), c["n"]).reshape(c["rows"], c["row_tokens"], c["n"])
+
+
+def test_batched_packing_is_one_matrix_after_the_other(oracle):
+    """kOSpatialIOGroupI4O4 with one output group: the spatial index (the weights batch) is the
+    outermost, so a batched buffer is the single-matrix buffers concatenated - what the kernel's
+    address offset w_batch_id * Ks * Ns (fully_connected.cc:493-496) assumes."""
+    rng = np.random.default_rng(5)
+    for bits, n, k, batch in ((8, 32, 64, 16), (4, 20, 40, 3), (8, 7, 12, 2)):
+        lim = 127 if bits == 8 else 7
+        w = rng.integers(-lim, lim + 1, size=(n, batch, 1, k), dtype=np.int8)
+        ns = (n + 3) // 4
+        pack = oracle.int8_as_uint8 if bits == 8 else oracle.int8_as_uint4
+        whole = pack(w, I4O4, ns)
+        parts = np.concatenate([pack(np.ascontiguousarray(w[:, e, 0, :]), I4O4, ns) for e in range(batch)])
+        assert np.array_equal(whole, parts)
+
+
+def test_batched_scale_tensor_layout(oracle):
+    """[group][batch][slice][4], zero padded: element (o, b, g) found where the kernel reads it
+    (weights_scale.Read(o_slice, w_batch_id, group), fully_connected_util.cc:80-98)."""
+    o_ch, batch, groups = 10, 3, 2
+    s = np.arange(o_ch * batch * groups, dtype=np.float32).reshape(o_ch, batch, groups) + 1
+    t = oracle.scale_to_hoio4_batched(s)
+    assert t.shape == (groups, batch, 3, 4)
+    for oc in range(o_ch):
+        for b in range(batch):
+            for g in range(groups):
+                assert t[g, b, oc // 4, oc % 4] == s[oc, b, g]
+    assert np.all(t[:, :, 2, 2:] == 0)
+    # one matrix: the same bytes as the unbatched conversion
+    assert np.array_equal(oracle.scale_to_hoio4_batched(s[:, :1, :])[:, 0], oracle.scale_to_hoio4(s[:, 0, :]))
+
+
+@pytest.mark.parametrize("src_shape,ids_count", [((1, 1, 32), 1), ((8, 1, 32), 8), ((128, 1, 64), 128),
+                                                 ((1, 1, 32), 4)])
+@pytest.mark.parametrize("precision", [0, 1])
+def test_batch_ids_reference_test_shapes(oracle, src_shape, ids_count, precision):
+    """fully_connected_test.cc:227-250: 32 output channels, a batch of 16 int8 matrices, sources
+    (1,1,1,32), (1,8,1,32), (1,128,1,64) with as many ids as rows, and the broadcast case of one
+    source row read by 4 ids.  Checked like the reference does: kernel against the float
+    reference over dequantized weights."""
+    src_rows, row_tokens, k = src_shape
+    c = make_batch_ids_case(ids_count + k, ids_count, row_tokens, src_rows, k, 32, 16)
+    got = run_batch_ids_oracle(oracle, c, precision)
+    ref = oracle.fc_batch_ids_reference_f32(c["src"], batch_ids_float_weights(oracle, c), c["ids"])
+    eps = 2e-5 * k if precision == 0 else 2e-2
+    assert np.abs(got - ref).max() <= eps * max(1.0, np.abs(ref).max())
+    # a row's result depends on its id: permuting two different ids changes those rows
+    if ids_count >= 8:
+        c2 = dict(c, ids=c["ids"].copy())
+        a, b = 0, int(np.argmax(c["ids"] != c["ids"][0]))
+        c2["ids"][[a, b]] = c["ids"][[b, a]]
+        got2 = run_batch_ids_oracle(oracle, c2, precision)
+        assert not np.array_equal(got2[a], got[a])
+        others = [y for y in range(ids_count) if y not in (a, b)]
+        assert np.array_equal(got2[others], got[others])
+
+
+def test_batch_ids_int4_groups_zero_points(oracle):
+    c = make_batch_ids_case(3, rows=5, row_tokens=3, src_rows=5, k=64, n=20, batch=4, bits=4, groups=2, with_zp=True)
+    got = run_batch_ids_oracle(oracle, c, 0)
+    ref = oracle.fc_batch_ids_reference_f32(c["src"], batch_ids_float_weights(oracle, c), c["ids"])
+    assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
