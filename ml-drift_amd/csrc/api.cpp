@@ -613,8 +613,12 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
-      // (batched weights by runtime ids: the unspecialised kernel)
-      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC") || a.batch_ids != nullptr;
+      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
+      // batched weights by runtime ids: the int4 streaming GEMV, else the unspecialised kernel
+      if (a.batch_ids != nullptr) {
+        e = !force_generic && FcW4StreamSupported(a) ? LaunchFcW4Stream(a, stream, &op->last_kernel)
+                                                     : LaunchFcGeneric(a, stream, &op->last_kernel);
+      } else
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
       // on the vector-ALU kernel; MLDHIP_GEMV_MFMA=1 forces the matrix-core one there too)
       if (!force_generic && (a.m >= 2 || EnvFlag("MLDHIP_GEMV_MFMA")) && FcW4MfmaStreamSupported(a)) {

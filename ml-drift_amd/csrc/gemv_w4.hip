@@ -78,6 +78,11 @@ struct StreamParams {
   // nibble masks and fp16 exponent patterns, passed as run-time values so that the compiler
   // keeps them in registers and forms single v_and_or_b32 instructions
   uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+  // Batched weights selected by runtime ids (fully_connected.cc:654-665, 804-822;
+  // fully_connected_util.cc:279-290): blockIdx.z = dst row, m tokens per row.  seg[0].weights
+  // holds weights_batch matrices one after the other, scales are [group][weights_batch][Ns][4].
+  const int32_t* batch_ids;
+  int rows, src_rows, weights_batch;
 };
 
 __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const __half* bias, size_t bi) {
@@ -89,9 +94,11 @@ __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const 
 // Branch-free: a K-slice past the end re-reads the last row of weights against zeroed
 // activations, so the eight loads of a chunk are issued back to back and the waits for them can
 // be counted down one by one while the arithmetic of the earlier slices runs.
+// act_stride / act_tok0: tokens per K-slice row of the activation tensor and the first token of
+// this launch row in it (M and 0 unless the launch has batched weights).
 template <int M>
 __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* weights, int row_u4, int c, int pcol,
-                                          u32x4 w[8], u32x2 a[8][M]) {
+                                          u32x4 w[8], u32x2 a[8][M], int act_stride = M, int act_tok0 = 0) {
   const int ks0 = c * 8;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -100,7 +107,7 @@ __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* we
     w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * row_u4 + pcol);
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      const u32x2 v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksc * M + m) * 4);
+      const u32x2 v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksc * act_stride + act_tok0 + m) * 4);
       a[j][m] = u32x2{ks < p.ks ? v[0] : 0u, ks < p.ks ? v[1] : 0u};
     }
   }
@@ -148,8 +155,11 @@ __device__ __forceinline__ void ComputeChunk(const StreamParams& p, const u32x4 
 // MULTI: the launch covers more than one matrix (the single-matrix instantiation reads its
 // arguments at fixed offsets, which saves a dependent scalar load in front of the first weight
 // load: 0.2 us on a 29 MB matrix).
-template <int LPR, int WAVES, int M, bool GROUPED, bool ZP, bool MULTI>
+// BATCHED: batched weights selected by runtime ids, one dst row per blockIdx.z (no K split, one
+// matrix list entry).
+template <int LPR, int WAVES, int M, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p) {
+  static_assert(!BATCHED || !MULTI, "a batched launch has one matrix list entry");
   constexpr int THREADS = WAVES * 64;
   constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
   constexpr int RPW = 64 / LPR;        // rows per wave
@@ -169,8 +179,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
     strip -= p.seg[si - 1].strip_end;
   }
   const StreamSegment& sg = p.seg[MULTI ? si : 0];
-  const u32x4* weights = sg.weights;
   const int row_u4 = sg.row_u4;
+  // BATCHED: this row's matrix (an id outside the batch is clamped into it), its source row
+  // (one shared row is broadcast) and the token strides of the two tensors
+  const int brow = BATCHED ? (int)blockIdx.z : 0;
+  int wb = BATCHED ? p.batch_ids[brow] : 0;
+  if (BATCHED) wb = __builtin_amdgcn_readfirstlane(min(max(wb, 0), p.weights_batch - 1));
+  const u32x4* weights = sg.weights + (BATCHED ? (size_t)wb * p.ks * row_u4 : 0);
+  const __half* scale_base = sg.scale + (BATCHED ? (size_t)wb * sg.n_pad : 0);
+  const __half* zp_base = ZP ? sg.zero_point + (BATCHED ? (size_t)wb * sg.n_pad : 0) : nullptr;
+  const size_t group_stride = (size_t)sg.n_pad * (BATCHED ? p.weights_batch : 1);  // elements per scale group
+  const int act_stride = BATCHED ? p.src_rows * M : M, act_tok0 = BATCHED ? min(brow, p.src_rows - 1) * M : 0;
+  const int dst_stride = BATCHED ? p.rows * M : M, dst_tok0 = BATCHED ? brow * M : 0;
   const int pcol_raw = strip * LPR + col;  // uint4 column = output channels 8*pcol .. +7
   const bool col_ok = pcol_raw < row_u4;
   const int pcol = col_ok ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
@@ -191,28 +211,28 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   // would make the kernel wait for them before it issues the weight loads.)
   const int n_out = min(strip * STRIP + tid % STRIP, sg.n_pad - 1);
   const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(sg.bias ? sg.bias : sg.scale);
-  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(sg.scale)[n_out];
+  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(scale_base)[n_out];
   const unsigned short out_bias_raw = bias_src[n_out];
 
   int c = c_begin + row;
   u32x4 zv = {0u, 0u, 0u, 0u};  // zero points of this thread's 8 channels (halfs)
-  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(sg.zero_point + (size_t)2 * pcol * 4);
+  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(zp_base + (size_t)2 * pcol * 4);
   if (c < c_end) {
     u32x4 w[8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, weights, row_u4, c, pcol, w, a);
+    LoadChunk<M>(p, weights, row_u4, c, pcol, w, a, act_stride, act_tok0);
     while (true) {
       const int cn = c + ROWS;
       const bool more = cn < c_end;
       u32x4 wn[8];
       u32x2 an[8][M];
-      if (more) LoadChunk<M>(p, weights, row_u4, cn, pcol, wn, an);
+      if (more) LoadChunk<M>(p, weights, row_u4, cn, pcol, wn, an, act_stride, act_tok0);
       u32x4 sv;
       if (GROUPED) {
         int g = c / p.group_chunks;
         if (g >= p.groups) g = p.groups - 1;
-        sv = *reinterpret_cast<const u32x4*>(sg.scale + ((size_t)g * sg.ns + 2 * pcol) * 4);
-        if (ZP) zv = *reinterpret_cast<const u32x4*>(sg.zero_point + ((size_t)g * sg.ns + 2 * pcol) * 4);
+        sv = *reinterpret_cast<const u32x4*>(scale_base + (size_t)g * group_stride + (size_t)2 * pcol * 4);
+        if (ZP) zv = *reinterpret_cast<const u32x4*>(zp_base + (size_t)g * group_stride + (size_t)2 * pcol * 4);
       }
       float t[M][8], asum[M];
 #pragma unroll
@@ -283,7 +303,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
       if (!GROUPED) v *= __half2float(__ushort_as_half(out_scale_raw));
       __half h = __float2half_rn(v);
       if (sg.bias) h = __hadd(h, __ushort_as_half(out_bias_raw));
-      sg.dst[((size_t)(n >> 2) * M + m) * 4 + (n & 3)] = h;
+      sg.dst[((size_t)(n >> 2) * dst_stride + dst_tok0 + m) * 4 + (n & 3)] = h;
     } else {
       p.partial[((size_t)ky * M + m) * sg.n_pad + n] = v;
     }
@@ -492,6 +512,32 @@ hipError_t LaunchShape(const StreamParams& p, int lpr, int waves, bool grouped, 
   return LaunchCfgM<8, 16>(p, grouped, grid, stream);
 }
 
+// Batched weights: two launch shapes (128-byte row segments with 8 waves, 64-byte ones with 4).
+template <int LPR, int WAVES, int M>
+hipError_t LaunchBatchedCfg(const StreamParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  const bool zp = p.seg[0].zero_point != nullptr;
+  const dim3 block(WAVES * 64);
+  if (grouped && zp)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true, true, false, true>), grid, block, 0, stream, p);
+  else if (grouped)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, true, false, false, true>), grid, block, 0, stream, p);
+  else if (zp)
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false, true, false, true>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((fc_w4_stream_kernel<LPR, WAVES, M, false, false, false, true>), grid, block, 0, stream, p);
+  return hipGetLastError();
+}
+template <int LPR, int WAVES>
+hipError_t LaunchBatchedM(const StreamParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  switch (p.m) {
+    case 1: return LaunchBatchedCfg<LPR, WAVES, 1>(p, grouped, grid, stream);
+    case 2: return LaunchBatchedCfg<LPR, WAVES, 2>(p, grouped, grid, stream);
+    case 3: return LaunchBatchedCfg<LPR, WAVES, 3>(p, grouped, grid, stream);
+    case 4: return LaunchBatchedCfg<LPR, WAVES, 4>(p, grouped, grid, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 int EnvInt(const char* name, int fallback) {
   const char* v = std::getenv(name);
   return v ? std::atoi(v) : fallback;
@@ -546,6 +592,23 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     weight_bytes += (size_t)p.ks * sg.ns * 8;
   }
   for (int i = count; i < kMaxSegments; ++i) p.seg[i] = p.seg[0];
+  p.batch_ids = a.batch_ids;
+  p.rows = a.rows;
+  p.src_rows = a.src_rows;
+  p.weights_batch = a.weights_batch;
+  if (a.batch_ids) {
+    // One dst row per blockIdx.z, K inside the work-group.  128-byte row segments when the rows
+    // together still give most CUs a work-group, else 64-byte ones.
+    if (count != 1) return hipErrorInvalidValue;
+    p.ksplit = 1;
+    if (kernel_name) *kernel_name = "fc_w4_stream_kernel";
+    const bool wide = (long)DivUp(p.seg[0].row_u4, 8) * a.rows >= 192;
+    const int lpr_b = wide ? 8 : 4, rows_b = wide ? 64 : 64;
+    p.chunks_per_split = DivUp(p.chunks, rows_b) * rows_b;
+    p.seg[0].strip_end = DivUp(p.seg[0].row_u4, lpr_b);
+    const dim3 grid_b(p.seg[0].strip_end, 1, a.rows);
+    return wide ? LaunchBatchedM<8, 8>(p, grouped, grid_b, stream) : LaunchBatchedM<4, 4>(p, grouped, grid_b, stream);
+  }
 
   // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the
   // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous

@@ -87,6 +87,8 @@ def test_reference_test_shapes(oracle, src_shape, ids_count, td):
     (4, 5, 3, 5, 64, 20, 4, 2, True),          # several tokens per row, zero points, ragged channels
     (8, 6, 2, 1, 171, 533, 3, 1, True),        # the reference's odd sizes
     (4, 4, 7, 4, 352, 200, 128, 11, False),    # many matrices, few used
+    (4, 3, 4, 3, 1000, 1032, 5, 1, True),      # per-channel scales + zero points, 4 tokens per row, ragged K
+    (4, 16, 2, 1, 512, 72, 6, 16, True),       # narrow matrices (64-byte row segments), group-wise zero points
 ])
 @pytest.mark.parametrize("td", [np.float16, np.float32])
 def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td):
@@ -96,6 +98,11 @@ def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, g
     print("batch ids", bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td.__name__, flush=True)
     got, name = run_device(c, td, bias=bias)
     check(c, td, got, oracle, bias=bias)
+    # fp16 int4 rows of up to 4 tokens with whole 32-channel chunks per scale group stream through
+    # the int4 GEMV; everything else takes the unspecialised kernel
+    fast = (td == np.float16 and bits == 4 and row_tokens <= 4 and (n + 3) // 4 % 2 == 0 and
+            (groups == 1 or (k // 4 // groups) % 8 == 0))
+    assert name == ("fc_w4_stream_kernel" if fast else "fc_generic_kernel"), name
 
 
 def test_repeated_and_out_of_range_ids(oracle):
