@@ -32,9 +32,9 @@ HBM_PEAK_GBS = 8000.0
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=None, help="default 4000 (c2), 200 (c3, c4), 20 (c5-*)")
+    p.add_argument("--steps", type=int, default=None, help="default 4000 (c2, c1, f2), 2000 (moe), 200 (c3, c4), 20 (c5-*)")
     p.add_argument("--warmup", type=int, default=None, help="default steps / 10")
-    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2"],
+    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe"],
                    help="c2 (default) is the headline line; the others time the remaining configurations "
                         "the same way (one JSON line each, no CPU baseline)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
@@ -46,7 +46,7 @@ def parse():
                         "reference dispatch) followed by 64 launches over the weight ring, then exit")
     a = p.parse_args()
     if a.steps is None:
-        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "c3": 200, "c4": 200}.get(a.workload, 20)
+        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "moe": 2000, "c3": 200, "c4": 200}.get(a.workload, 20)
     if a.warmup is None:
         a.warmup = max(1, a.steps // 10)
     return a
@@ -129,6 +129,41 @@ def run_other(args, torch, M, W):
         out = dict(base, metric=metric, value=round(nbytes * args.steps / wall / 1e9, 1), unit="GB/s",
                    ms_per_step=round(wall * 1e3 / args.steps, 6), dtype=dtype,
                    config={"workload": label, "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes},
+                   roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "traffic": None, "avg_launch_us": round(us, 3)})
+    elif args.workload == "moe":
+        # FullyConnected with batched weights selected by runtime ids: one token, 2 of 8 expert
+        # matrices of the c2 shape per step.  Successive steps take other pairs of experts and the
+        # weights exist twice, so a matrix comes back after 470 MB of other weights.
+        m, k, n, experts, top = 1, 4096, 14336, 8, 2
+        ns = (n + 3) // 4
+        desc = M.fc_int4_weights_desc(n, k)
+        rng = np.random.default_rng(0)
+        act = torch.from_numpy(W.to_slices(rng.standard_normal((m, k)).astype(np.float16))).cuda()
+        scale = torch.from_numpy(M.scale_to_tensor_batched(
+            (np.abs(rng.normal(0.0, 0.02, size=(n, experts, 1))) / 7.0).astype(np.float32), M.FLOAT16).view(np.float16)).cuda()
+        out_t = torch.zeros((ns, top * m, 4), dtype=torch.float16, device="cuda")
+        ops, keep = [], []
+        for copy in range(2):
+            wt = torch.randint(0, 256, (experts * (k // 4) * ns * 8,), dtype=torch.uint8, device="cuda")
+            for pair in range(experts // top):
+                ids = torch.tensor([pair * top + j for j in range(top)], dtype=torch.int32, device="cuda")
+                op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, n, k, desc, scale_shape=(n, 1),
+                                 max_tokens=top * m, weights_batch=experts, shared_src=True)
+                op.bind([act, ids, wt, scale], [out_t])
+                op.set_shape(1, top, m)
+                ops.append(op)
+                keep += [ids, wt]
+        nbytes = top * (n * k // 2 + n * 2 + n * 2 * m) + k * 2 * m + top * 4  # W + scale + out per row, act, ids
+        wall, ev_ms = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup)
+        us = ev_ms * 1e3 / args.steps
+        out = dict(base, metric="int4_moe_decode_gemv_hbm_bandwidth", value=round(nbytes * args.steps / wall / 1e9, 1),
+                   unit="GB/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+                   dtype="u4 weights x f16 activations, f32 accumulate",
+                   config={"workload": "moe: FullyConnected with batched weights by runtime ids, 1 token, 2 of 8 matrices "
+                                       "K=4096 N=14336 int4 per-channel, fp16 act/out",
+                           "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes},
                    roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})

@@ -6,6 +6,7 @@
 //   WeightsDescription, OHWI, BHWC            common/task/weights_layout.h, common/shape.h
 //   ExternalWeights                            common/task/gpu_operation.h:354-363
 //   CreateFullyConnectedExternalWeights        common/kernels/fully_connected.h:155-161
+//   CreateFullyConnectedWeightsBatchIds        common/kernels/fully_connected.cc:1174-1216
 //   CreateQuantization                         common/kernels/quantize_and_dequantize.h:68-73
 //   ClOperation::{SetSrcTensor, SetDstTensor, UpdateParams, AddToQueue}   cl/cl_operation.h:44-129
 //   GpuModelBuilder::FullyConnectedInt4/8ExternalWeights (dispatcher)     common/gpu_model_builder.cc:1548-1725
@@ -135,9 +136,40 @@ class HipOperation {
   std::unique_ptr<mldhip_op, void (*)(mldhip_op*)> op_{nullptr, &mldhip_op_destroy};
 };
 
+namespace detail {
+inline mldhip_fc_desc FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
+                               const ExternalWeights& weights, bool has_bias, int max_tokens);
+}  // namespace detail
+
+// CreateFullyConnectedWeightsBatchIds (common/kernels/fully_connected.h, .cc:1174-1216): the
+// FullyConnected of a mixture-of-experts layer.  weights.shape.h = number of weight matrices;
+// src objects: src_tensor, batch_ids, weights, [weights_scale, weights_zero_point,] [biases].
+// UpdateParams(BHWC(1, ids, tokens per id, c)) sets the dst shape; `shared_src`: the source tensor
+// has one row that every id reads (its H is 1), else one row per id.
+inline Status CreateFullyConnectedWeightsBatchIds(CalculationsPrecision precision, DataType src_type,
+                                                  DataType dst_type, const ExternalWeights& weights, bool has_bias,
+                                                  bool shared_src, int max_tokens, HipOperation* result) {
+  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens);
+  mldhip_op* op = nullptr;
+  const int rc = mldhip_fc_batch_ids_create(&d, weights.shape.h, shared_src ? 1 : 0, &op);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  *result = HipOperation(op);
+  return {};
+}
+
 inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precision, DataType src_type,
                                                   DataType dst_type, const ExternalWeights& weights, bool has_bias,
                                                   int max_tokens, HipOperation* result) {
+  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens);
+  mldhip_op* op = nullptr;
+  const int rc = mldhip_fc_create(&d, &op);
+  if (rc != MLDHIP_OK) return Status::FromCode(rc);
+  *result = HipOperation(op);
+  return {};
+}
+
+inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
+                                       const ExternalWeights& weights, bool has_bias, int max_tokens) {
   mldhip_fc_desc d{};
   d.precision = (int)precision;
   d.src_type = (int)src_type;
@@ -153,11 +185,7 @@ inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precisio
   d.scalar_zero_point = weights.scalar_zero_point;
   d.has_bias = has_bias;
   d.max_tokens = max_tokens;
-  mldhip_op* op = nullptr;
-  const int rc = mldhip_fc_create(&d, &op);
-  if (rc != MLDHIP_OK) return Status::FromCode(rc);
-  *result = HipOperation(op);
-  return {};
+  return d;
 }
 
 inline Status CreateQuantization(DataType src_type, PackedType dst_type, const BHWC& shape, bool calculate_sum,

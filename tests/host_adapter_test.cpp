@@ -59,6 +59,22 @@ int main() {
                                            false, 1, &bad);
   EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !bad.valid());
 
+  // the mixture-of-experts FullyConnected: fully_connected.cc:1203-1213 registers batch_ids before the weights
+  ExternalWeights we;
+  we.shape = OHWI{768, 128, 1, 2048};
+  we.desc = GetFullyConnectedInt4WeightsDesc(we.shape);
+  we.scale_zp_shape = OHWI{768, 128, 1, 64};
+  we.has_scale_tensor = true;
+  HipOperation moe;
+  EXPECT(CreateFullyConnectedWeightsBatchIds(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, we,
+                                             /*has_bias=*/false, /*shared_src=*/true, 32, &moe)
+             .ok());
+  names = moe.GetSrcTensorsNames();
+  EXPECT(names.size() == 4 && names[0] == "src_tensor" && names[1] == "batch_ids" && names[2] == "weights" &&
+         names[3] == "weights_scale");
+  EXPECT(moe.UpdateParams(BHWC{1, 8, 1, 2048}).ok());
+  EXPECT(moe.UpdateParams(BHWC{2, 8, 1, 2048}).code == MLDHIP_UNIMPLEMENTED);
+
   HipOperation q;
   EXPECT(CreateQuantization(DataType::kFloat16, PackedType::kInt8C16, BHWC{1, 1, 2048, 2048}, false, true, &q).ok());
   EXPECT(q.GetDstTensorsNames().size() == 2 && q.GetDstTensorsNames()[1] == "dst_params");
