@@ -614,10 +614,14 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
       const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
-      // batched weights by runtime ids: the int4 streaming GEMV, else the unspecialised kernel
+      // batched weights by runtime ids: the streaming GEMVs, else the unspecialised kernel
       if (a.batch_ids != nullptr) {
-        e = !force_generic && FcW4StreamSupported(a) ? LaunchFcW4Stream(a, stream, &op->last_kernel)
-                                                     : LaunchFcGeneric(a, stream, &op->last_kernel);
+        if (!force_generic && FcW4StreamSupported(a))
+          e = LaunchFcW4Stream(a, stream, &op->last_kernel);
+        else if (!force_generic && FcW8StreamSupported(a))
+          e = LaunchFcW8Stream(a, stream, &op->last_kernel);
+        else
+          e = LaunchFcGeneric(a, stream, &op->last_kernel);
       } else
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
       // on the vector-ALU kernel; MLDHIP_GEMV_MFMA=1 forces the matrix-core one there too)

@@ -36,6 +36,11 @@ struct W8Params {
   int group_chunks;  // chunks per scale group (grouped only)
   int groups;
   int grouped;
+  // Batched weights selected by runtime ids (fully_connected.cc:654-665, 804-822;
+  // fully_connected_util.cc:279-290): blockIdx.z = dst row, m tokens per row; the matrices lie one
+  // after the other, scales are [group][weights_batch][Ns][4].
+  const int32_t* batch_ids;
+  int rows, src_rows, weights_batch;
 };
 
 __device__ __forceinline__ void Load4(const float* p, size_t i, float v[4]) {
@@ -63,7 +68,7 @@ __device__ __forceinline__ void Store1(__half* dst, size_t i, float r, const __h
   dst[i] = h;
 }
 
-template <typename T, int LPR, int WAVES, int M>
+template <typename T, int LPR, int WAVES, int M, bool BATCHED>
 __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
   constexpr int THREADS = WAVES * 64;
   constexpr int ROWS = THREADS / LPR;  // chunks the work-group covers per step
@@ -74,9 +79,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
   __shared__ float red[ROWS][M][STRIP];
   __shared__ float red2[PARTS][M][STRIP];
 
+  // BATCHED: this row's matrix (an id outside the batch is clamped into it), its source row (one
+  // shared row is broadcast) and the token strides of the two tensors
+  const int brow = BATCHED ? (int)blockIdx.z : 0;
+  int wb = BATCHED ? p.batch_ids[brow] : 0;
+  if (BATCHED) wb = min(max(wb, 0), p.weights_batch - 1);
+  const u32x4* weights = p.weights + (BATCHED ? (size_t)wb * p.ks * p.ns : 0);
   const T* act = static_cast<const T*>(p.act);
-  const T* scale = static_cast<const T*>(p.scale);
-  const T* zero_point = static_cast<const T*>(p.zero_point);
+  const T* scale = static_cast<const T*>(p.scale) + (BATCHED ? (size_t)wb * p.ns * 4 : 0);
+  const T* zero_point = p.zero_point ? static_cast<const T*>(p.zero_point) + (BATCHED ? (size_t)wb * p.ns * 4 : 0) : nullptr;
+  const size_t group_stride = (size_t)p.ns * 4 * (BATCHED ? p.weights_batch : 1);
+  const int act_stride = BATCHED ? p.src_rows * M : M, act_tok0 = BATCHED ? min(brow, p.src_rows - 1) * M : 0;
+  const int dst_stride = BATCHED ? p.rows * M : M, dst_tok0 = BATCHED ? brow * M : 0;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -102,7 +116,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int ks = min(c * 8 + j, p.ks - 1);  // rows past K re-read the last one; their activations are zero
-      w[j] = __builtin_nontemporal_load(p.weights + (size_t)ks * p.ns + slice);
+      w[j] = __builtin_nontemporal_load(weights + (size_t)ks * p.ns + slice);
     }
   };
   auto load_acts = [&](int c, float (&a)[8][M][4]) {
@@ -114,7 +128,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
         // unconditional load at a clamped row, zeroed by selects: a branch here would make every
         // wait of the chunk a wait for all loads
         float v[4];
-        Load4(act, ((size_t)min(ks, p.ks - 1) * M + m) * 4, v);
+        Load4(act, ((size_t)min(ks, p.ks - 1) * act_stride + act_tok0 + m) * 4, v);
 #pragma unroll
         for (int i = 0; i < 4; ++i) a[j][m][i] = ks < p.ks ? v[i] : 0.0f;
       }
@@ -135,8 +149,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
     if (p.grouped) {
       int g = c / p.group_chunks;
       if (g >= p.groups) g = p.groups - 1;
-      Load4(scale, ((size_t)g * p.ns + slice) * 4, s);
-      if (zero_point) Load4(zero_point, ((size_t)g * p.ns + slice) * 4, z);
+      Load4(scale, (size_t)g * group_stride + (size_t)slice * 4, s);
+      if (zero_point) Load4(zero_point, (size_t)g * group_stride + (size_t)slice * 4, z);
     }
     float t[M][4], asum[M];
 #pragma unroll
@@ -196,26 +210,30 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
     float v = 0.0f;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
-    Store1(dst, ((size_t)(n >> 2) * M + m) * 4 + (n & 3), v, bias, (size_t)n);
+    Store1(dst, ((size_t)(n >> 2) * dst_stride + dst_tok0 + m) * 4 + (n & 3), v, bias, (size_t)n);
   }
 }
 
-template <typename T, int LPR, int WAVES>
-hipError_t LaunchM(const W8Params& p, dim3 grid, hipStream_t stream) {
+template <typename T, int LPR, int WAVES, bool BATCHED>
+hipError_t LaunchMB(const W8Params& p, dim3 grid, hipStream_t stream) {
   const dim3 block(WAVES * 64);
   switch (p.m) {
-    case 1: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 2>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 3>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 4>), grid, block, 0, stream, p); break;
+    case 1: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1, BATCHED>), grid, block, 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 2, BATCHED>), grid, block, 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 3, BATCHED>), grid, block, 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 4, BATCHED>), grid, block, 0, stream, p); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
+template <typename T, int LPR, int WAVES>
+hipError_t LaunchM(const W8Params& p, dim3 grid, hipStream_t stream) {
+  return p.batch_ids ? LaunchMB<T, LPR, WAVES, true>(p, grid, stream) : LaunchMB<T, LPR, WAVES, false>(p, grid, stream);
+}
 
 template <typename T>
 hipError_t LaunchT(const W8Params& p, int lpr, int waves, hipStream_t stream) {
-  const dim3 grid(DivUp(p.ns, lpr));
+  const dim3 grid(DivUp(p.ns, lpr), 1, p.batch_ids ? p.rows : 1);
   if (lpr == 4) return waves == 4 ? LaunchM<T, 4, 4>(p, grid, stream) : LaunchM<T, 4, 16>(p, grid, stream);
   return waves == 4 ? LaunchM<T, 8, 4>(p, grid, stream) : LaunchM<T, 8, 16>(p, grid, stream);
 }
@@ -250,9 +268,13 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
   p.grouped = a.scale_kind == kScaleBlock;
   p.groups = p.grouped ? a.groups : 1;
   p.group_chunks = p.grouped ? (p.ks / a.groups) / 8 : p.chunks;
+  p.batch_ids = a.batch_ids;
+  p.rows = a.rows;
+  p.src_rows = a.src_rows;
+  p.weights_batch = a.weights_batch;
   // 128-byte row segments (8 slices) when that still gives a work-group to half the CUs, else
   // 64-byte ones; small work-groups when K is covered by 64 / 128 rows of chunks
-  const int lpr = DivUp(p.ns, 8) >= 128 ? 8 : 4;
+  const int lpr = (long)DivUp(p.ns, 8) * (a.batch_ids ? a.rows : 1) >= 128 ? 8 : 4;
   const int waves = p.chunks <= 4 * 64 / lpr ? 4 : 16;
   if (kernel_name) *kernel_name = "fc_w8_stream_kernel";
   return a.act_f16 ? LaunchT<__half>(p, lpr, waves, stream) : LaunchT<float>(p, lpr, waves, stream);

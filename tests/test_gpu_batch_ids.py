@@ -89,6 +89,8 @@ def test_reference_test_shapes(oracle, src_shape, ids_count, td):
     (4, 4, 7, 4, 352, 200, 128, 11, False),    # many matrices, few used
     (4, 3, 4, 3, 1000, 1032, 5, 1, True),      # per-channel scales + zero points, 4 tokens per row, ragged K
     (4, 16, 2, 1, 512, 72, 6, 16, True),       # narrow matrices (64-byte row segments), group-wise zero points
+    (8, 8, 1, 1, 2048, 768, 16, 64, True),     # int8 matrices, group-wise, shared input
+    (8, 4, 3, 4, 1000, 2048, 5, 1, False),     # int8 per-channel, 3 tokens per row, ragged K
 ])
 @pytest.mark.parametrize("td", [np.float16, np.float32])
 def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td):
@@ -98,11 +100,17 @@ def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, g
     print("batch ids", bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, td.__name__, flush=True)
     got, name = run_device(c, td, bias=bias)
     check(c, td, got, oracle, bias=bias)
-    # fp16 int4 rows of up to 4 tokens with whole 32-channel chunks per scale group stream through
-    # the int4 GEMV; everything else takes the unspecialised kernel
-    fast = (td == np.float16 and bits == 4 and row_tokens <= 4 and (n + 3) // 4 % 2 == 0 and
-            (groups == 1 or (k // 4 // groups) % 8 == 0))
-    assert name == ("fc_w4_stream_kernel" if fast else "fc_generic_kernel"), name
+    # rows of up to 4 tokens with whole 32-channel chunks per scale group stream through the GEMV
+    # kernels (int4: fp16 tensors and an even slice count); everything else takes the
+    # unspecialised kernel
+    chunks_ok = groups == 1 or (k // 4 // groups) % 8 == 0
+    expect = "fc_generic_kernel"
+    if row_tokens <= 4 and chunks_ok:
+        if bits == 4 and td == np.float16 and (n + 3) // 4 % 2 == 0:
+            expect = "fc_w4_stream_kernel"
+        elif bits == 8:
+            expect = "fc_w8_stream_kernel"
+    assert name == expect, (name, expect)
 
 
 def test_repeated_and_out_of_range_ids(oracle):
