@@ -739,6 +739,13 @@ int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {
   if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
   std::vector<size_t> need_src, need_dst;
   RequiredSizes(op, &need_src, &need_dst);
+  // batched weights: only the matrices the ids select are read
+  // (common/gpu_model_builder_moe_util.cc:268-283)
+  if (op->kind == mldhip_op::kFc && op->idx_ids >= 0 && op->h < op->weights_batch) {
+    const int objects[3] = {op->idx_weights, op->idx_scale, op->idx_zp};
+    for (int idx : objects)
+      if (idx >= 0) need_src[idx] = need_src[idx] / op->weights_batch * op->h;
+  }
   uint64_t total = 0;
   for (size_t v : need_src) total += v;
   for (size_t v : need_dst) total += v;

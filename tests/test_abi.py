@@ -154,6 +154,10 @@ def test_fc_batch_ids_object_order_and_validation():
     assert op.src_names == ["src_tensor", "batch_ids", "weights", "weights_scale", "biases"]
     assert op.dst_names == ["dst_tensor"]
     op.set_shape(1, 8, 2)
+    # cost: 8 of the 16 matrices are read (gpu_model_builder_moe_util.cc:268-283), fp16 tensors
+    nbytes, flops = op.cost()
+    assert flops == 2 * 16 * 64 * 32
+    assert nbytes == 16 * 64 * 2 + 8 * 4 + 8 * (64 * 32 + 32 * 2) + 32 * 2 + 16 * 32 * 2
     with pytest.raises(M.MldhipError) as e:   # tensors of a batch-ids op have batch 1
         op.set_shape(2, 4, 1)
     assert e.value.code == M.UNIMPLEMENTED
