@@ -52,8 +52,11 @@ def run_device(c, td, bias=None, max_tokens=None):
 
 
 def check(c, td, got, oracle, bias=None):
-    ref = oracle.fc_batch_ids_reference_f32(c["src"].astype(td).astype(np.float32), batch_ids_float_weights(oracle, c),
-                                            c["ids"]).astype(np.float64)
+    # FullyConnectedWeightsBatchIdsReference (common/task/testing_ref_ops.cc:1042-1067) in float64, vectorised:
+    # the oracle's loop form of it is pinned in tests/test_oracle_fc.py and is too slow for these sizes
+    src = c["src"].astype(td).astype(np.float64)
+    wf = batch_ids_float_weights(oracle, c).astype(np.float64)
+    ref = np.stack([src[0 if src.shape[0] == 1 else y] @ wf[:, int(c["ids"][y]), :].T for y in range(c["rows"])])
     if bias is not None:
         ref = ref + np.asarray(bias, np.float64)
     err = np.abs(got - ref).max()
@@ -141,3 +144,32 @@ def test_bindings_are_checked():
     with pytest.raises(M.MldhipError) as e:
         M.fc_launch_fused([op])
     assert e.value.code == M.FAILED_PRECONDITION
+
+
+def test_random_sweep(oracle):
+    """Seeded sweep over rows, tokens per row, shared / per-row sources, weight types, ragged K / N
+    and scale groupings, whatever kernel the dispatcher picks."""
+    rng = np.random.default_rng(77)
+    seen = {}
+    for it in range(30):
+        bits = int(rng.choice([4, 8]))
+        rows = int(rng.choice([1, 2, 3, 8, 17]))
+        row_tokens = int(rng.choice([1, 1, 2, 4, 5]))
+        shared = bool(rng.random() < 0.5)
+        k = int(rng.choice([64, 96, 171, 256, 1000, 2048]))
+        n = int(rng.choice([8, 20, 64, 152, 533, 1024, 2056]))
+        batch = int(rng.choice([1, 2, 5, 32]))
+        groups = 1
+        gs = int(rng.choice([32, 64]))
+        if k % gs == 0 and rng.random() < 0.6:
+            groups = k // gs
+        zp = bool(rng.random() < 0.3)
+        td = np.float16 if rng.random() < 0.7 else np.float32
+        c = make_batch_ids_case(500 + it, rows, row_tokens, 1 if shared else rows, k, n, batch, bits, groups, zp)
+        print("sweep", it, dict(bits=bits, rows=rows, tok=row_tokens, shared=shared, k=k, n=n, batch=batch, groups=groups,
+                                zp=zp, td=td.__name__), flush=True)
+        got, name = run_device(c, td)
+        seen[name] = seen.get(name, 0) + 1
+        check(c, td, got, oracle)
+    print("kernels exercised:", seen)
+    assert len(seen) >= 3

@@ -122,6 +122,28 @@ def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp, monkey
         check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
 
 
+def test_gemm_modes_random_sweep(monkeypatch):
+    """Seeded sweep over shapes with the two-tile mode forced on and off and every token tile
+    forced in turn: all against the textbook reference at the fp16 bar."""
+    rng = np.random.default_rng(31)
+    for it in range(24):
+        bits = int(rng.choice([4, 8]))
+        m = int(rng.choice([6, 33, 64, 66, 128, 130, 258, 300]))
+        k = int(rng.choice([64, 96, 352, 512, 1024]))
+        n = int(rng.choice([8, 100, 128, 260, 384, 1000]))
+        groups = 1
+        gs = int(rng.choice([32, 64]))
+        if k % gs == 0 and rng.random() < 0.6:
+            groups = k // gs
+        zp = bool(rng.random() < 0.4)
+        monkeypatch.setenv("MLDHIP_GEMM_DUAL", str(it % 2))
+        monkeypatch.setenv("MLDHIP_GEMM_FM", str([1, 2, 4][it % 3]))
+        case = W.make_fc_case(seed=900 + it, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                              with_bias=bool(it % 2), with_zero_point=zp)
+        got = run_w4(case)
+        check_fp(got, textbook(case), case, "sweep %d" % it)
+
+
 def test_gemm_two_tiles_fused_launch(monkeypatch):
     """Three matrices in one two-tile launch: pairs of tiles that straddle two matrices (3 + 1 + 2
     channel tiles) against the single one-tile launches."""
