@@ -51,16 +51,17 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 
-// Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
-// dst = activation(gate(x)) * up(x) for a pair of such layers of one shape (1..2 tokens).
+// dst = activation(gate(x)) * up(x) for a pair of int4 layers of one shape on the streaming GEMV
+// (1..2 tokens).
 bool FcW4GatedSupported(const FcArgs& gate, const FcArgs& up);
 hipError_t LaunchFcW4Gated(const FcArgs& gate, const FcArgs& up, int activation, void* dst, hipStream_t stream,
                            const char** kernel_name);
 
-// The same for 1..16 tokens on the matrix cores (per-channel scales, wide layers).
+// The int4 streaming GEMV for 1..16 tokens on the matrix cores (per-channel scales, wide layers).
 bool FcW4MfmaStreamSupported(const FcArgs& a);
 hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 
+// Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
 bool FcW8StreamSupported(const FcArgs& a);
 hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 
@@ -98,7 +99,7 @@ struct ConvInt8Args {
 };
 hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char** kernel_name);
 
-// Multi-token FullyConnected with int4 weights on the MFMA units (fp16 tensors).
+// Multi-token FullyConnected with uint4 or uint8 weights on the MFMA units (fp16 tensors).
 bool FcW4MfmaSupported(const FcArgs& a);
 hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
