@@ -171,6 +171,24 @@ def test_gemm_two_tiles_fused_launch(monkeypatch):
         assert np.abs(got - ref).max() <= 2e-3 * rms  # another K split among the waves: fp32 summation order
 
 
+def test_fused_prefill_2048_tokens_default_modes():
+    """q / k / v of the decoder stack (2048 -> 2048, 256, 256, group 32) at 2048 tokens in one launch with
+    the dispatcher's own choices (128-token tiles, two channel tiles per work-group, pairs that
+    straddle matrices): every output against the textbook reference."""
+    import torch
+    m, k = 2048, 2048
+    cases = [W.make_fc_case(seed=70 + i, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=64)
+             for i, n in enumerate((2048, 256, 256))]
+    for c in cases[1:]:
+        c["act"] = cases[0]["act"]
+    devs = [W.FcDevice(c) for c in cases]
+    for d in devs[1:]:
+        d.op.set_src(0, devs[0].act)
+    M.fc_launch_fused([d.op for d in devs], torch.cuda.current_stream().cuda_stream)
+    for d, c in zip(devs, cases):
+        check_fp(d.result(), textbook(c), c, "fused prefill n=%d" % c["n"])
+
+
 def test_gemm_two_tiles_chosen_for_large_launches():
     """4096 x 4096 x 4096 (1024 tiles) runs in the two-tile mode by default and meets the bar."""
     case = W.make_fc_case(seed=5, m=4096, k=4096, n=4096, weight_bits=4, tensor_dtype=np.float16, groups=1)
