@@ -37,6 +37,9 @@ def parse():
     p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe"],
                    help="c2 (default) is the headline line; the others time the remaining configurations "
                         "the same way (one JSON line each, no CPU baseline)")
+    p.add_argument("--tokens", type=int, default=128,
+                   help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
+                        "kernels away from the launch-bound regime)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
@@ -221,8 +224,8 @@ def run_other(args, torch, M, W):
                              "traffic": None, "avg_launch_us": round(us, 3)})
     else:
         from decoder_stack import DecoderStack
-        tokens = 1 if args.workload == "c5-decode" else 128
-        st = DecoderStack(max_tokens=128)
+        tokens = 1 if args.workload == "c5-decode" else max(5, args.tokens)
+        st = DecoderStack(max_tokens=max(128, tokens))
         st.set_tokens(tokens)
         wall, ev_ms = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
         us = ev_ms * 1e3 / args.steps
