@@ -327,7 +327,8 @@ def run_gated_pair(oracle, m, k, n, groups, bias, kind, expect_kernel, ulp_check
 @pytest.mark.parametrize("m,k,n,groups,bias", [(3, 512, 72, 16, False), (16, 2048, 2048, 1, True),
                                                (64, 1024, 1032, 32, True), (77, 352, 200, 11, False),
                                                (128, 2048, 16384, 64, False), (130, 96, 260, 1, True),
-                                               (2048, 256, 4096, 1, True)])
+                                               (2048, 256, 4096, 1, True),
+                                               (129, 128, 8192, 4, True)])  # odd token count on the 64-token tile
 @pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
 def test_gated_pair_prefill(oracle, m, k, n, groups, bias, kind):
     """The same step at prefill token counts: the matrix-core GEMM with the gated epilogue (tiles of
