@@ -353,9 +353,10 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream);
  * FullyConnected ops bound to the same src_tensor with the same shape; their results are rounded
  * to fp16 (+ biases) as the two nodes would store them and combined in fp32 in the operation
  * order of the sample's elementwise kernel; their own dst tensors are not written.  dst:
- * [ceil(o/4)][tokens][4] halfs.  Served for int4 weights, fp16 tensors, symmetric: 1..2 tokens by
- * the streaming GEMV pair, more tokens by the matrix-core GEMM (half of a work-group's waves on
- * gate, half on up, combined where the K reduction ends).  MLDHIP_FAILED_PRECONDITION otherwise:
+ * [ceil(o/4)][tokens][4] halfs.  Served for fp16 tensors and symmetric weights: int4 at 1..2
+ * tokens by the streaming GEMV pair, int4 at more tokens and int8 above 4 tokens by the
+ * matrix-core GEMM (half of a work-group's waves on gate, half on up, combined where the K
+ * reduction ends).  MLDHIP_FAILED_PRECONDITION otherwise:
  * launch the two ops (mldhip_fc_launch_fused) and the host framework's elementwise node
  * instead. */
 enum { MLDHIP_GATE_GELU_TANH = 1, MLDHIP_GATE_SILU = 2 };

@@ -719,8 +719,8 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
   const bool gemv = FcW4GatedSupported(args[0], args[1]);
   if (!gemv && !FcW4MfmaGatedSupported(args[0], args[1]))
     return Fail(MLDHIP_FAILED_PRECONDITION,
-                "gate and up are not a pair of int4 fp16 FullyConnected ops over one tensor with one shape, "
-                "symmetric weights and scale groups the int4 kernels serve");
+                "gate and up are not a pair of fp16 FullyConnected ops over one tensor with one shape and weight "
+                "type, symmetric weights and scale groups the gated kernels serve (int8 weights: above 4 tokens)");
   const size_t need = (size_t)DivUp(args[0].n, 4) * 4 * args[0].m * sizeof(uint16_t);
   if (dst_bytes < need) return Fail(MLDHIP_INVALID_ARGUMENT, "dst is too small for the gated output");
   const char* name = nullptr;

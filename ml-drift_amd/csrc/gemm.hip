@@ -913,9 +913,13 @@ void LaunchDirectW(bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) 
 // DUAL_OK: the two-tile mode is compiled for this shape.
 template <int FM, int U, int WAVES, bool PAIR, bool DUAL_OK>
 void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const GemmParams& p) {
-  if (p.gate_activation != 0) {  // gated pair: uint4, symmetric
-    hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<4, FM, U, WAVES, false, PAIR, false, kModeGated>), grid,
-                       dim3(WAVES * 64), 0, stream, p);
+  if (p.gate_activation != 0) {  // gated pair: symmetric weights
+    if (weight_bits == 8)
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<8, FM, U, WAVES, false, PAIR, false, kModeGated>), grid,
+                         dim3(WAVES * 64), 0, stream, p);
+    else
+      hipLaunchKernelGGL((fc_w4_mfma_direct_kernel<4, FM, U, WAVES, false, PAIR, false, kModeGated>), grid,
+                         dim3(WAVES * 64), 0, stream, p);
     return;
   }
   if constexpr (DUAL_OK) {
@@ -1107,7 +1111,8 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
   if (gated) n_total = a.n;  // one set of channel tiles, each with twice the work
   for (int i = count; i < kMaxW4Segments; ++i) p.seg[i] = p.seg[0];
   if (kernel_name)
-    *kernel_name = gated ? "fc_w4_gated_mfma_gemm_kernel" : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
+    *kernel_name = gated ? (a.weight_bits == 8 ? "fc_w8_gated_mfma_gemm_kernel" : "fc_w4_gated_mfma_gemm_kernel")
+                         : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
   if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 && a.m % 2 == 0 ? 4 : 2);
@@ -1165,7 +1170,10 @@ hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kern
 
 bool FcW4MfmaGatedSupported(const FcArgs& gate, const FcArgs& up) {
   if (!DirectGemmShapeOk(gate) || !DirectGemmShapeOk(up)) return false;
-  if (gate.weight_bits != 4 || up.weight_bits != 4) return false;
+  if (gate.weight_bits != up.weight_bits) return false;
+  // uint8 pairs of a few tokens are better served by their two streaming GEMVs and the host's
+  // elementwise node than by a 32-token tile
+  if (gate.weight_bits == 8 && gate.m <= kGemvMaxTokens) return false;
   if (gate.has_zero_point || up.has_zero_point) return false;
   return gate.act == up.act && gate.m == up.m && gate.k == up.k && gate.n == up.n && gate.scale_kind == up.scale_kind &&
          gate.groups == up.groups;

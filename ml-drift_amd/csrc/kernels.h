@@ -107,7 +107,8 @@ hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream
 // fp32 workspace the MFMA path wants for token counts up to max_tokens (K split across
 // work-groups); 0 when it never splits.
 size_t FcW4MfmaWorkspaceFloats(int max_tokens, int k, int n);
-// dst = activation(gate(x)) * up(x) on the matrix-core kernel (any token count; uint4, symmetric).
+// dst = activation(gate(x)) * up(x) on the matrix-core kernel (symmetric weights; uint4 at any token
+// count, uint8 above the GEMV token counts).
 bool FcW4MfmaGatedSupported(const FcArgs& gate, const FcArgs& up);
 hipError_t LaunchFcW4MfmaGated(const FcArgs& gate, const FcArgs& up, int activation, void* dst, hipStream_t stream,
                                const char** kernel_name);

@@ -284,16 +284,16 @@ def test_gated_pair(oracle, m, k, n, groups, bias, kind):
     run_gated_pair(oracle, m, k, n, groups, bias, kind, "fc_w4_gated_stream_kernel")
 
 
-def run_gated_pair(oracle, m, k, n, groups, bias, kind, expect_kernel, ulp_check=True):
+def run_gated_pair(oracle, m, k, n, groups, bias, kind, expect_kernel, ulp_check=True, bits=4):
     """dst = activation(gate(x)) * up(x) in one launch against the three separate steps: the two
     FullyConnected launches on the GPU, then the oracle's restatement of the sample's elementwise
     kernel on their fp16 outputs.  Bar: the FullyConnected bar, 2e-2 of the output RMS (the fused
     kernel adds K in another order, so a gate value can differ by an fp16 ulp); besides, 99 % of
     the elements must agree to 2 fp16 ulp."""
     torch = torch_cuda()
-    gate_case = W.make_fc_case(seed=11 + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+    gate_case = W.make_fc_case(seed=11 + n, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
                                with_bias=bias)
-    up_case = W.make_fc_case(seed=12 + n, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+    up_case = W.make_fc_case(seed=12 + n, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
                              with_bias=bias)
     up_case["act"] = gate_case["act"]
     # gate values of a few units so that the activation is in its curved range
@@ -339,6 +339,14 @@ def test_gated_pair_prefill(oracle, m, k, n, groups, bias, kind):
     run_gated_pair(oracle, m, k, n, groups, bias, kind, "fc_w4_gated_mfma_gemm_kernel", ulp_check=m > 4)
 
 
+@pytest.mark.parametrize("m,k,n,groups,bias", [(5, 512, 72, 16, False), (64, 1024, 1032, 32, True),
+                                               (130, 96, 260, 1, True), (1024, 256, 4096, 1, False)])
+@pytest.mark.parametrize("kind", ["gelu_tanh", "silu"])
+def test_gated_pair_prefill_uint8(oracle, m, k, n, groups, bias, kind):
+    """uint8 weights on the same gated matrix-core kernel (above the GEMV token counts)."""
+    run_gated_pair(oracle, m, k, n, groups, bias, kind, "fc_w8_gated_mfma_gemm_kernel", bits=8)
+
+
 def test_gated_pair_refused(oracle):
     torch = torch_cuda()
     a = W.FcDevice(W.make_fc_case(seed=1, m=3, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1))
@@ -347,12 +355,20 @@ def test_gated_pair_refused(oracle):
     with pytest.raises(M.MldhipError) as e:   # two different source tensors
         M.fc_launch_gated(a.op, b.op, M.GATE_SILU, dst, torch.cuda.current_stream().cuda_stream)
     assert e.value.code == M.FAILED_PRECONDITION
-    # uint8 weights: not served by the gated kernels
-    c8 = W.make_fc_case(seed=3, m=8, k=256, n=64, weight_bits=8, tensor_dtype=np.float16, groups=1)
+    # uint8 weights at GEMV token counts: left to the two streaming GEMVs and the host's elementwise node
+    c8 = W.make_fc_case(seed=3, m=3, k=256, n=64, weight_bits=8, tensor_dtype=np.float16, groups=1)
     g8, u8 = W.FcDevice(c8), W.FcDevice(c8)
     u8.op.set_src(0, g8.act)
     with pytest.raises(M.MldhipError) as e:
         M.fc_launch_gated(g8.op, u8.op, M.GATE_SILU, torch.zeros_like(g8.out), torch.cuda.current_stream().cuda_stream)
+    assert e.value.code == M.FAILED_PRECONDITION
+    # a uint4 gate with a uint8 up
+    c48 = W.make_fc_case(seed=3, m=8, k=256, n=64, weight_bits=8, tensor_dtype=np.float16, groups=1)
+    c44 = W.make_fc_case(seed=3, m=8, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1)
+    gm, um = W.FcDevice(c44), W.FcDevice(c48)
+    um.op.set_src(0, gm.act)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_launch_gated(gm.op, um.op, M.GATE_SILU, torch.zeros_like(gm.out), torch.cuda.current_stream().cuda_stream)
     assert e.value.code == M.FAILED_PRECONDITION
     # a destination that is too small
     c4 = W.make_fc_case(seed=4, m=8, k=256, n=64, weight_bits=4, tensor_dtype=np.float16, groups=1)
