@@ -265,7 +265,8 @@ int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);
  * is clamped into the range.
  * src objects: 0 "src_tensor", 1 "batch_ids" (int32 [h]), 2 "weights", then "weights_scale",
  * "weights_zero_point", "biases" as for mldhip_fc_create (fully_connected.cc:1203-1213).
- * Floating-point tensors only; desc->max_tokens bounds h*w. */
+ * With src_type INT8 / dst_type INT32 the integer-math variant runs over the batched weights (no
+ * scale objects).  desc->max_tokens bounds h*w; the tensors have batch 1. */
 int mldhip_fc_batch_ids_create(const mldhip_fc_desc* desc, int weights_batch, int shared_src, mldhip_op** op);
 
 /* CreateQuantization (common/kernels/quantize_and_dequantize.h:57-73, .cc:693-842).

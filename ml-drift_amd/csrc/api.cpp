@@ -310,8 +310,6 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   if (!d || !out) return Fail(MLDHIP_INVALID_ARGUMENT, "null argument");
   *out = nullptr;
   if (batch_ids && weights_batch < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "weights_batch must be positive");
-  if (batch_ids && d->src_type == MLDHIP_INT8)
-    return Fail(MLDHIP_UNIMPLEMENTED, "batched weights are served for floating-point tensors");
   if (d->o <= 0 || d->i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
   if (d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "max_tokens must be positive");
   const mldhip_weights_desc& wd = d->weights;
@@ -601,15 +599,22 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     const mldhip_fc_desc& d = op->fc;
     if (d.src_type == MLDHIP_INT8) {
       const int bits = WeightBits(d.weights.type);
-      if (!EnvFlag("MLDHIP_FORCE_GENERIC") && FcInt8MathStreamSupported(op->Tokens(), d.i, d.o, bits)) {
-        e = LaunchFcInt8MathStream(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
-                                   static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o, bits, stream,
-                                   &op->last_kernel);
-      } else {
-        e = LaunchFcInt8Math(static_cast<const int8_t*>(op->src_ptr[0]), static_cast<const uint8_t*>(op->src_ptr[1]),
-                             static_cast<int32_t*>(op->dst_ptr[0]), op->Tokens(), d.i, d.o, bits, stream,
-                             &op->last_kernel);
+      FcBatchRows batch;
+      int tokens = op->Tokens();
+      if (op->idx_ids >= 0) {  // batched weights: h rows of w tokens
+        batch.ids = static_cast<const int32_t*>(op->src_ptr[op->idx_ids]);
+        batch.rows = op->h;
+        batch.src_rows = op->shared_src ? 1 : op->h;
+        batch.weights_batch = op->weights_batch;
+        tokens = op->w;
       }
+      const int8_t* act = static_cast<const int8_t*>(op->src_ptr[0]);
+      const uint8_t* weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
+      int32_t* dst = static_cast<int32_t*>(op->dst_ptr[0]);
+      if (!EnvFlag("MLDHIP_FORCE_GENERIC") && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
+        e = LaunchFcInt8MathStream(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
+      else
+        e = LaunchFcInt8Math(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;

@@ -177,11 +177,18 @@ template <int WBITS, int TB>
 __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restrict__ act,
                                                            const uint8_t* __restrict__ weights,
                                                            int32_t* __restrict__ dst, int m, int ks_n,
-                                                           int ns) {
+                                                           int ns, FcBatchRows batch) {
   __shared__ int red[kKl][kSl][TB * 4];
   const int tx = threadIdx.x, ty = threadIdx.y;
   const int ds = blockIdx.x * kSl + tx;
   const int tok0 = blockIdx.y * TB;
+  // batched weights: blockIdx.z = dst row (one row, matrix 0, for a plain launch)
+  const int row = blockIdx.z;
+  int wb = batch.ids ? batch.ids[row] : 0;
+  wb = min(max(wb, 0), batch.weights_batch - 1);
+  weights += (size_t)wb * ks_n * ns * (WBITS == 8 ? 16 : 8);
+  const size_t act_stride = (size_t)batch.src_rows * m, dst_stride = (size_t)batch.rows * m;
+  const size_t act_tok0 = (size_t)min(row, batch.src_rows - 1) * m, dst_tok0 = (size_t)row * m;
   int acc[TB][4];
 #pragma unroll
   for (int t = 0; t < TB; ++t)
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
       for (int t = 0; t < TB; ++t) {
         const int tok = tok0 + t;
         if (tok >= m) continue;
-        const int v = *reinterpret_cast<const int*>(act + ((size_t)ks * m + tok) * 4);
+        const int v = *reinterpret_cast<const int*>(act + ((size_t)ks * act_stride + act_tok0 + tok) * 4);
         acc[t][0] = __builtin_amdgcn_sdot4(v, (int)w0, acc[t][0], false);
         acc[t][1] = __builtin_amdgcn_sdot4(v, (int)w1, acc[t][1], false);
         acc[t][2] = __builtin_amdgcn_sdot4(v, (int)w2, acc[t][2], false);
@@ -261,7 +268,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
         int r = 0;
 #pragma unroll
         for (int q = 0; q < kKl; ++q) r += red[q][tx][t * 4 + c];
-        dst[((size_t)ds * m + tok) * 4 + c] = r;
+        dst[((size_t)ds * dst_stride + dst_tok0 + tok) * 4 + c] = r;
       }
     }
   }
@@ -302,16 +309,17 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
 }
 
 hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k,
-                            int n, int weight_bits, hipStream_t stream, const char** kernel_name) {
+                            int n, int weight_bits, hipStream_t stream, const char** kernel_name,
+                            const FcBatchRows& batch) {
   constexpr int TB = 4;
   const int ks = DivUp(k, 4), ns = DivUp(n, 4);
-  dim3 grid(DivUp(ns, kSl), DivUp(m, TB));
+  dim3 grid(DivUp(ns, kSl), DivUp(m, TB), batch.ids ? batch.rows : 1);
   dim3 block(kSl, kKl);
   if (kernel_name) *kernel_name = "fc_int8_math_kernel";
   if (weight_bits == 8)
-    hipLaunchKernelGGL((fc_int8_math_kernel<8, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns);
+    hipLaunchKernelGGL((fc_int8_math_kernel<8, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, batch);
   else
-    hipLaunchKernelGGL((fc_int8_math_kernel<4, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns);
+    hipLaunchKernelGGL((fc_int8_math_kernel<4, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, batch);
   return hipGetLastError();
 }
 

@@ -35,6 +35,7 @@ struct I8MathParams {
   int m, ks, ns;
   int row_u4;  // 16-byte items per K-slice row
   int chunks;  // ceil(ks / 8)
+  FcBatchRows batch;  // batched weights selected by runtime ids: blockIdx.z = dst row
 };
 
 __device__ __forceinline__ uint32_t Perm(uint32_t hi, uint32_t lo, uint32_t sel) {
@@ -42,7 +43,7 @@ __device__ __forceinline__ uint32_t Perm(uint32_t hi, uint32_t lo, uint32_t sel)
 }
 
 // WBITS 8: a lane's 16 bytes are one slice (4 outputs); WBITS 4: two slices (8 outputs).
-template <int WBITS, int LPR, int WAVES, int M>
+template <int WBITS, int LPR, int WAVES, int M, bool BATCHED>
 __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathParams p) {
   constexpr int THREADS = WAVES * 64;
   constexpr int ROWS = THREADS / LPR;
@@ -61,6 +62,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
   const int row = wave * RPW + lane / LPR;
   const int item_raw = blockIdx.x * LPR + col;
   const int item = item_raw < p.row_u4 ? item_raw : p.row_u4 - 1;  // clamp: loads stay in range, result unused
+  // BATCHED: this row's matrix (an id outside the batch is clamped into it), its source row (one
+  // shared row is broadcast) and the token strides of the two tensors
+  const int brow = BATCHED ? (int)blockIdx.z : 0;
+  int wb = BATCHED ? p.batch.ids[brow] : 0;
+  if (BATCHED) wb = min(max(wb, 0), p.batch.weights_batch - 1);
+  const u32x4* weights = p.weights + (BATCHED ? (size_t)wb * p.ks * p.row_u4 : 0);
+  const int act_stride = BATCHED ? p.batch.src_rows * M : M, act_tok0 = BATCHED ? min(brow, p.batch.src_rows - 1) * M : 0;
+  const int dst_stride = BATCHED ? p.batch.rows * M : M, dst_tok0 = BATCHED ? brow * M : 0;
 
   int acc[M][OUTS], asum[M];
 #pragma unroll
@@ -77,10 +86,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
     for (int j = 0; j < 8; ++j) {
       const int ks = c * 8 + j;
       const int ksc = min(ks, p.ks - 1);
-      w[j] = __builtin_nontemporal_load(p.weights + (size_t)ksc * p.row_u4 + item);
+      w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * p.row_u4 + item);
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        const int v = p.act[(size_t)ksc * M + m];
+        const int v = p.act[(size_t)ksc * act_stride + act_tok0 + m];
         a[j][m] = ks < p.ks ? v : 0;
       }
     }
@@ -152,26 +161,30 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
     int v = 0;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
-    p.dst[((size_t)(n >> 2) * M + m) * 4 + (n & 3)] = v;
+    p.dst[((size_t)(n >> 2) * dst_stride + dst_tok0 + m) * 4 + (n & 3)] = v;
   }
 }
 
-template <int WBITS, int LPR, int WAVES>
-hipError_t LaunchM(const I8MathParams& p, dim3 grid, hipStream_t stream) {
+template <int WBITS, int LPR, int WAVES, bool BATCHED>
+hipError_t LaunchMB(const I8MathParams& p, dim3 grid, hipStream_t stream) {
   const dim3 block(WAVES * 64);
   switch (p.m) {
-    case 1: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 1>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 2>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 3>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 4>), grid, block, 0, stream, p); break;
+    case 1: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 1, BATCHED>), grid, block, 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 2, BATCHED>), grid, block, 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 3, BATCHED>), grid, block, 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((fc_i8math_stream_kernel<WBITS, LPR, WAVES, 4, BATCHED>), grid, block, 0, stream, p); break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
+template <int WBITS, int LPR, int WAVES>
+hipError_t LaunchM(const I8MathParams& p, dim3 grid, hipStream_t stream) {
+  return p.batch.ids ? LaunchMB<WBITS, LPR, WAVES, true>(p, grid, stream) : LaunchMB<WBITS, LPR, WAVES, false>(p, grid, stream);
+}
 
 template <int WBITS>
 hipError_t LaunchW(const I8MathParams& p, int lpr, int waves, hipStream_t stream) {
-  const dim3 grid(DivUp(p.row_u4, lpr));
+  const dim3 grid(DivUp(p.row_u4, lpr), 1, p.batch.ids ? p.batch.rows : 1);
   if (lpr == 4) return waves == 4 ? LaunchM<WBITS, 4, 4>(p, grid, stream) : LaunchM<WBITS, 4, 16>(p, grid, stream);
   return waves == 4 ? LaunchM<WBITS, 8, 4>(p, grid, stream) : LaunchM<WBITS, 8, 16>(p, grid, stream);
 }
@@ -186,8 +199,10 @@ bool FcInt8MathStreamSupported(int m, int k, int n, int weight_bits) {
 }
 
 hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k, int n,
-                                  int weight_bits, hipStream_t stream, const char** kernel_name) {
+                                  int weight_bits, hipStream_t stream, const char** kernel_name,
+                                  const FcBatchRows& batch) {
   I8MathParams p;
+  p.batch = batch;
   p.weights = reinterpret_cast<const u32x4*>(weights);
   p.act = reinterpret_cast<const int*>(act);
   p.dst = dst;
@@ -198,7 +213,7 @@ hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int
   p.chunks = DivUp(p.ks, 8);
   // 128-byte row segments when that still gives a work-group to half the CUs, else 64-byte ones;
   // small work-groups for several tokens (LDS) and when K is covered by few rows of chunks
-  const int lpr = DivUp(p.row_u4, 8) >= 128 ? 8 : 4;
+  const int lpr = (long)DivUp(p.row_u4, 8) * (batch.ids ? batch.rows : 1) >= 128 ? 8 : 4;
   const int waves = (m > 1 || p.chunks <= 4 * 64 / lpr) ? 4 : 16;
   if (kernel_name) *kernel_name = "fc_i8math_stream_kernel";
   return weight_bits == 4 ? LaunchW<4>(p, lpr, waves, stream) : LaunchW<8>(p, lpr, waves, stream);

@@ -65,13 +65,22 @@ hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char*
 bool FcW8StreamSupported(const FcArgs& a);
 hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 
+// Batched weights selected by runtime ids, for the integer-math launches (the same fields as in
+// FcArgs): dst row y of `rows` (m tokens each) = source row min(y, src_rows - 1) x matrix ids[y].
+struct FcBatchRows {
+  const int32_t* ids = nullptr;
+  int rows = 1, src_rows = 1, weights_batch = 1;
+};
+
 // int8 activations x uint8/uint4 weights -> int32 (no scales).
 hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k,
-                            int n, int weight_bits, hipStream_t stream, const char** kernel_name);
+                            int n, int weight_bits, hipStream_t stream, const char** kernel_name,
+                            const FcBatchRows& batch = FcBatchRows());
 // The same for 1..4 tokens as an HBM-streaming kernel.
 bool FcInt8MathStreamSupported(int m, int k, int n, int weight_bits);
 hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k, int n,
-                                  int weight_bits, hipStream_t stream, const char** kernel_name);
+                                  int weight_bits, hipStream_t stream, const char** kernel_name,
+                                  const FcBatchRows& batch = FcBatchRows());
 
 struct QuantArgs {
   const void* src = nullptr;

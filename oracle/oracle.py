@@ -256,6 +256,22 @@ def fc_batch_ids_kernel(act_slices, ids, weights, rows, row_tokens, src_rows, we
     return out
 
 
+def fc_batch_ids_int8_kernel(act_slices_i8, ids, weights, rows, row_tokens, src_rows, weights_batch, k, n, weight_bits):
+    """The integer-math variant with batched weights (the same generator with int8 sources:
+    common/kernels/fully_connected.cc:543-621 with the w_batch_id offsets of :549-557, rows as in
+    :804-822): `fc_int8_kernel` per dst row on views of the buffers.  act [Ks][src_rows *
+    row_tokens][4] int8 -> [Ns][rows * row_tokens][4] int32."""
+    ks, ns = div_up(k, 4), div_up(n, 4)
+    act = _c(act_slices_i8, np.int8).reshape(ks, src_rows * row_tokens, 4)
+    w = _c(weights, np.uint8).reshape(weights_batch, -1)
+    out = np.empty((ns, rows * row_tokens, 4), np.int32)
+    for y in range(rows):
+        sy = min(y, src_rows - 1)
+        a = np.ascontiguousarray(act[:, sy * row_tokens:(sy + 1) * row_tokens, :])
+        out[:, y * row_tokens:(y + 1) * row_tokens, :] = fc_int8_kernel(a, w[int(ids[y])], row_tokens, k, n, weight_bits)
+    return out
+
+
 def fc_batch_ids_reference_f32(src, weights_obi, ids):
     """FullyConnectedWeightsBatchIdsReference (common/task/testing_ref_ops.cc:1042-1067): src
     (src_rows, tokens, K) float, weights (O, batch, K) float -> (rows, tokens, O); a source with one

@@ -164,9 +164,8 @@ def test_fc_batch_ids_object_order_and_validation():
     with pytest.raises(M.MldhipError) as e:
         M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 32, 64, wd, scale_shape=(32, 1), weights_batch=0)
     assert e.value.code == M.INVALID_ARGUMENT
-    with pytest.raises(M.MldhipError) as e:   # the integer-math variant has no batched form here
-        M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 32, 64, wd, weights_batch=4)
-    assert e.value.code == M.UNIMPLEMENTED
+    op8 = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 32, 64, wd, max_tokens=8, weights_batch=4)
+    assert op8.src_names == ["src_tensor", "batch_ids", "weights"]
 
 
 def test_scale_to_tensor_batched_matches_oracle(oracle):

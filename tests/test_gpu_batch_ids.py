@@ -9,7 +9,8 @@ pytestmark = pytest.mark.gpu
 
 import mldhip as M
 import workloads as W
-from test_oracle_fc import batch_ids_float_weights, make_batch_ids_case, run_batch_ids_oracle
+from test_oracle_fc import (batch_ids_float_weights, batch_ids_int8_exact, make_batch_ids_case,
+                            make_batch_ids_int8_case, run_batch_ids_int8_oracle, run_batch_ids_oracle)
 
 FP16_TOL = 2e-2
 
@@ -173,3 +174,35 @@ def test_random_sweep(oracle):
         check(c, td, got, oracle)
     print("kernels exercised:", seen)
     assert len(seen) >= 3
+
+
+@pytest.mark.parametrize("bits,rows,row_tokens,src_rows,k,n,batch", [
+    (8, 8, 1, 8, 32, 32, 16), (8, 4, 1, 1, 32, 32, 16),      # the reference's batch-ids shapes, int8 sources
+    (4, 8, 1, 1, 2048, 768, 16), (4, 8, 1, 8, 768, 2048, 16),  # mixture decode shapes (streaming kernel)
+    (8, 3, 4, 3, 1000, 1032, 5), (4, 5, 3, 5, 171, 20, 3),     # ragged K, odd uint4 slice count (tiled kernel)
+    (8, 2, 9, 1, 256, 64, 4),                                   # more than 4 tokens per row (tiled kernel)
+])
+def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, batch):
+    """The integer-math FullyConnected over batched weights: int32 results bit for bit against the
+    closed form and the oracle's kernel restatement."""
+    import torch
+    c = make_batch_ids_int8_case(rows + n + bits, rows, row_tokens, src_rows, k, n, batch, bits)
+    print("batch ids int8", bits, rows, row_tokens, src_rows, k, n, batch, flush=True)
+    ns = W.div_up(n, 4)
+    desc = (M.fc_int8_weights_desc if bits == 8 else M.fc_int4_weights_desc)(n, k)
+    packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
+    act = torch.from_numpy(W.to_slices(c["src"].reshape(-1, k))).cuda()
+    ids = torch.from_numpy(c["ids"]).cuda()
+    weights = torch.from_numpy(packed).cuda()
+    out = torch.zeros((ns, rows * row_tokens, 4), dtype=torch.int32, device="cuda")
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=rows * row_tokens, weights_batch=batch,
+                     shared_src=src_rows == 1 and rows > 1)
+    op.bind([act, ids, weights], [out])
+    op.set_shape(1, rows, row_tokens)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    got = W.from_slices(out.cpu().numpy(), n).reshape(rows, row_tokens, n)
+    assert np.array_equal(got, batch_ids_int8_exact(c))
+    assert np.array_equal(got, run_batch_ids_int8_oracle(oracle, c))
+    stream_ok = row_tokens <= 4 and (bits == 8 or ns % 2 == 0)
+    assert op.kernel_name == ("fc_i8math_stream_kernel" if stream_ok else "fc_int8_math_kernel"), op.kernel_name

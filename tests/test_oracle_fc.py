@@ -294,3 +294,38 @@ def test_batch_ids_int4_groups_zero_points(oracle):
     got = run_batch_ids_oracle(oracle, c, 0)
     ref = oracle.fc_batch_ids_reference_f32(c["src"], batch_ids_float_weights(oracle, c), c["ids"])
     assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+
+
+def make_batch_ids_int8_case(seed, rows, row_tokens, src_rows, k, n, batch, bits):
+    rng = np.random.default_rng(seed)
+    lim = 127 if bits == 8 else 7
+    w = rng.integers(-lim - 1, lim + 1, size=(n, batch, 1, k), dtype=np.int8)
+    src = rng.integers(-128, 128, size=(src_rows, row_tokens, k), dtype=np.int8)
+    ids = rng.integers(0, batch, size=rows).astype(np.int32)
+    return dict(w=w, src=src, ids=ids, rows=rows, row_tokens=row_tokens, src_rows=src_rows, k=k, n=n, batch=batch, bits=bits)
+
+
+def batch_ids_int8_exact(c):
+    """The closed form: int32 products of the selected matrix with the row's tokens."""
+    out = np.empty((c["rows"], c["row_tokens"], c["n"]), np.int64)
+    for y in range(c["rows"]):
+        sy = 0 if c["src_rows"] == 1 else y
+        out[y] = c["src"][sy].astype(np.int64) @ c["w"][:, int(c["ids"][y]), 0, :].astype(np.int64).T
+    return out
+
+
+def run_batch_ids_int8_oracle(o, c):
+    ns = (c["n"] + 3) // 4
+    packed = (o.int8_as_uint8 if c["bits"] == 8 else o.int8_as_uint4)(c["w"], I4O4, ns)
+    act = o.to_slices(c["src"].reshape(-1, c["k"]))
+    out = o.fc_batch_ids_int8_kernel(act, c["ids"], packed, c["rows"], c["row_tokens"], c["src_rows"], c["batch"],
+                                     c["k"], c["n"], c["bits"])
+    return o.from_slices(out, c["n"]).reshape(c["rows"], c["row_tokens"], c["n"])
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("rows,row_tokens,src_rows,k,n,batch", [(8, 1, 8, 32, 32, 16), (4, 1, 1, 32, 32, 16),
+                                                                 (5, 3, 5, 171, 20, 3)])
+def test_batch_ids_int8_math_exact(oracle, bits, rows, row_tokens, src_rows, k, n, batch):
+    c = make_batch_ids_int8_case(rows + k + bits, rows, row_tokens, src_rows, k, n, batch, bits)
+    assert np.array_equal(run_batch_ids_int8_oracle(oracle, c), batch_ids_int8_exact(c))
