@@ -317,9 +317,19 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.m * sg.n_pad) return;
   const int m = idx / sg.n_pad, n = idx % sg.n_pad;
+  // The parts are fetched eight at a time before any is added (a part past the last re-reads the
+  // last one and is dropped by a select), so that their latencies overlap; added in split order.
+  const float scale = GROUPED ? 1.0f : __half2float(sg.scale[n]);
   float v = 0.0f;
-  for (int s = 0; s < p.ksplit; ++s) v += p.partial[((size_t)s * p.m + m) * sg.n_pad + n];
-  if (!GROUPED) v *= __half2float(sg.scale[n]);
+  for (int s0 = 0; s0 < p.ksplit; s0 += 8) {
+    float part[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      part[j] = p.partial[((size_t)min(s0 + j, p.ksplit - 1) * p.m + m) * sg.n_pad + n];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v += s0 + j < p.ksplit ? part[j] : 0.0f;
+  }
+  v *= scale;
   StoreHalf(sg.dst, ((size_t)(n >> 2) * p.m + m) * 4 + (n & 3), v, sg.bias, (size_t)n);
 }
 
