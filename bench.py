@@ -8,10 +8,11 @@ Infinity Cache if one buffer were reused, so the steps rotate over a ring of wei
 larger than that cache, the way the reference's own perf harness does behind
 kUseMultipleWeights (cl/testing/perf_util.cc:2247-2253).
 
-Prints ONE JSON line.  `value` is algorithmic bytes * steps / wall time of the timed region
-(a HIP-graph replay of the steps, inputs resident in HBM); `roofline.achieved` divides the
-same algorithmic bytes by the average launch duration measured with HIP events on the
-launch stream over that region.
+Prints ONE JSON line.  The timed region is R back-to-back replays of a HIP graph that holds the
+steps (inputs resident in HBM; R such that the region lasts at least 5 ms, so that the replay's
+own host cost does not weigh on a 20-step run).  `value` is algorithmic bytes / (wall time of
+the region / launches in it); `roofline.achieved` divides the same bytes by the average launch
+duration measured with HIP events on the launch stream over the same region.
 """
 import argparse
 import ctypes
@@ -41,6 +42,9 @@ def parse():
                    help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
                         "kernels away from the launch-bound regime)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
+    p.add_argument("--layout", default="library", choices=["library", "reference"],
+                   help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
+                        "slices) or in the reference's own FullyConnected layout (one output group)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -55,31 +59,58 @@ def parse():
     return a
 
 
-def time_graph(torch, stream, launch_step, steps, warmup):
-    """`warmup` eager steps, then a graph of `steps` steps: one untimed replay, one timed between two
-    events on `stream`.  Returns (wall seconds, event milliseconds)."""
+MIN_REGION_MS = 5.0  # the timed region is at least this long, whatever --steps says
+
+
+def time_graph(torch, stream, launch_step, steps, warmup, use_graph=True, ring=1):
+    """`warmup` eager steps, then a graph of `steps` steps (rounded up to a whole number of turns of the
+    weight ring, so that replay after replay every weight copy comes back only after all the others).  A single replay of a short graph is
+    dominated by the replay's own host and synchronisation cost (tens of microseconds), so the
+    timed region is R back-to-back replays, R chosen from one untimed replay such that the region
+    lasts at least MIN_REGION_MS.  Returns (wall seconds per step, event microseconds per step, {R, steps per replay}):
+    both are region / (R * steps), the wall clock bracketed by synchronisations, the HIP events
+    recorded on `stream` around the same replays."""
     s = stream.cuda_stream
+    steps = -(-steps // ring) * ring
     with torch.cuda.stream(stream):
         for i in range(warmup):
             launch_step(s, i)
         stream.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            cs = torch.cuda.current_stream().cuda_stream
-            for i in range(steps):
-                launch_step(cs, i)
-        graph.replay()
+        graph = None
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                cs = torch.cuda.current_stream().cuda_stream
+                for i in range(steps):
+                    launch_step(cs, i)
+
+            def replay():
+                graph.replay()
+        else:
+            def replay():
+                for i in range(steps):
+                    launch_step(s, i)
+        replay()  # untimed: the first replay uploads the graph
         stream.synchronize()
         ev0 = torch.cuda.Event(enable_timing=True)
         ev1 = torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        replay()
+        ev1.record(stream)
+        stream.synchronize()
+        one_ms = max(ev0.elapsed_time(ev1), 1e-3)
+        replays = max(1, min(20000, int(np.ceil(MIN_REGION_MS / one_ms))))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         ev0.record(stream)
-        graph.replay()
+        for _ in range(replays):
+            replay()
         ev1.record(stream)
         stream.synchronize()
+        torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-    return wall, ev0.elapsed_time(ev1)
+    n = replays * steps
+    return wall / n, ev0.elapsed_time(ev1) * 1e3 / n, {"graph_replays": replays, "launches_per_replay": steps}
 
 
 def run_other(args, torch, M, W):
@@ -127,11 +158,11 @@ def run_other(args, torch, M, W):
             nbytes = n * k // 2 + k + n * 4  # W + int8 act + int32 out
             label = "f2: int8-math FullyConnected decode GEMV M=1 K=4096 N=14336, int8 act x uint4 weights -> int32"
             metric, dtype = "int8_math_decode_gemv_hbm_bandwidth", "i8 x u4, i32 accumulate (v_dot4)"
-        wall, ev_ms = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup)
-        us = ev_ms * 1e3 / args.steps
-        out = dict(base, metric=metric, value=round(nbytes * args.steps / wall / 1e9, 1), unit="GB/s",
-                   ms_per_step=round(wall * 1e3 / args.steps, 6), dtype=dtype,
-                   config={"workload": label, "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes},
+        wall, us, reg = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup,
+                                   ring=len(ops))
+        out = dict(base, metric=metric, value=round(nbytes / wall / 1e9, 1), unit="GB/s",
+                   ms_per_step=round(wall * 1e3, 6), dtype=dtype,
+                   config=dict({"workload": label, "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes}, **reg),
                    roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
@@ -141,7 +172,7 @@ def run_other(args, torch, M, W):
         # weights exist twice, so a matrix comes back after 470 MB of other weights.
         m, k, n, experts, top = 1, 4096, 14336, 8, 2
         ns = (n + 3) // 4
-        desc = M.fc_int4_weights_desc(n, k)
+        desc = M.fc_int4_weights_desc(n, k, reference=True)  # batched weights: one output group
         rng = np.random.default_rng(0)
         act = torch.from_numpy(W.to_slices(rng.standard_normal((m, k)).astype(np.float16))).cuda()
         scale = torch.from_numpy(M.scale_to_tensor_batched(
@@ -159,28 +190,27 @@ def run_other(args, torch, M, W):
                 ops.append(op)
                 keep += [ids, wt]
         nbytes = top * (n * k // 2 + n * 2 + n * 2 * m) + k * 2 * m + top * 4  # W + scale + out per row, act, ids
-        wall, ev_ms = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup)
-        us = ev_ms * 1e3 / args.steps
-        out = dict(base, metric="int4_moe_decode_gemv_hbm_bandwidth", value=round(nbytes * args.steps / wall / 1e9, 1),
-                   unit="GB/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+        wall, us, reg = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup,
+                                   ring=len(ops))
+        out = dict(base, metric="int4_moe_decode_gemv_hbm_bandwidth", value=round(nbytes / wall / 1e9, 1),
+                   unit="GB/s", ms_per_step=round(wall * 1e3, 6),
                    dtype="u4 weights x f16 activations, f32 accumulate",
-                   config={"workload": "moe: FullyConnected with batched weights by runtime ids, 1 token, 2 of 8 matrices "
-                                       "K=4096 N=14336 int4 per-channel, fp16 act/out",
-                           "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes},
+                   config=dict({"workload": "moe: FullyConnected with batched weights by runtime ids, 1 token, 2 of 8 "
+                                            "matrices K=4096 N=14336 int4 per-channel, fp16 act/out",
+                                "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes}, **reg),
                    roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
     elif args.workload == "c3":
         case = W.make_fc_case(**W.CONFIGS["c3"])
         dev = W.FcDevice(case)
-        wall, ev_ms = time_graph(torch, stream, lambda s, i: dev.op.launch(s), args.steps, args.warmup)
+        wall, us, reg = time_graph(torch, stream, lambda s, i: dev.op.launch(s), args.steps, args.warmup)
         flops = 2.0 * case["m"] * case["k"] * case["n"]
-        us = ev_ms * 1e3 / args.steps
-        out = dict(base, metric="int4_prefill_gemm_throughput", value=round(flops * args.steps / wall / 1e12, 1),
-                   unit="TFLOP/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+        out = dict(base, metric="int4_prefill_gemm_throughput", value=round(flops / wall / 1e12, 1),
+                   unit="TFLOP/s", ms_per_step=round(wall * 1e3, 6),
                    dtype="u4 weights x f16 activations, f32 accumulate (fp16 MFMA)",
-                   config={"workload": "c3: FullyConnected prefill GEMM M=512 K=4096 N=4096 int4 group-32, fp16 act/out",
-                           "flops_per_step": flops},
+                   config=dict({"workload": "c3: FullyConnected prefill GEMM M=512 K=4096 N=4096 int4 group-32, fp16 act/out",
+                                "flops_per_step": flops}, **reg),
                    roofline={"bound": "mfma", "kernel": dev.op.kernel_name, "achieved": round(flops / us / 1e6, 1),
                              "peak": 2500.0, "unit": "TFLOP/s", "frac": round(flops / us / 1e6 / 2500.0, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
@@ -209,16 +239,15 @@ def run_other(args, torch, M, W):
         def step(s, i):
             q.launch(s)
             conv.launch(s)
-        wall, _ = time_graph(torch, stream, step, args.steps, args.warmup)
-        _, conv_ms = time_graph(torch, stream, lambda s, i: conv.launch(s), args.steps, args.warmup)
-        _, q_ms = time_graph(torch, stream, lambda s, i: q.launch(s), args.steps, args.warmup)
+        wall, _, reg = time_graph(torch, stream, step, args.steps, args.warmup)
+        _, us, _ = time_graph(torch, stream, lambda s, i: conv.launch(s), args.steps, args.warmup)
+        _, q_us, _ = time_graph(torch, stream, lambda s, i: q.launch(s), args.steps, args.warmup)
         ops = 2.0 * m * k * n
-        us = conv_ms * 1e3 / args.steps
-        out = dict(base, metric="int8_dynamic_gemm_throughput", value=round(ops * args.steps / wall / 1e12, 1),
-                   unit="TOP/s", ms_per_step=round(wall * 1e3 / args.steps, 6),
+        out = dict(base, metric="int8_dynamic_gemm_throughput", value=round(ops / wall / 1e12, 1),
+                   unit="TOP/s", ms_per_step=round(wall * 1e3, 6),
                    dtype="i8 x i8, i32 accumulate (int8 MFMA), f32 rescale",
-                   config={"workload": "c4: per-token int8 quantization + int8 x int8 GEMM M=2048 K=2048 N=8192, fp16 out",
-                           "ops_per_step": ops, "quantize_us": round(q_ms * 1e3 / args.steps, 3)},
+                   config=dict({"workload": "c4: per-token int8 quantization + int8 x int8 GEMM M=2048 K=2048 N=8192, fp16 out",
+                                "ops_per_step": ops, "quantize_us": round(q_us, 3)}, **reg),
                    roofline={"bound": "mfma", "kernel": conv.kernel_name, "achieved": round(ops / us / 1e6, 1),
                              "peak": 5000.0, "unit": "TOP/s", "frac": round(ops / us / 1e6 / 5000.0, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
@@ -227,24 +256,23 @@ def run_other(args, torch, M, W):
         tokens = 1 if args.workload == "c5-decode" else max(5, args.tokens)
         st = DecoderStack(max_tokens=max(128, tokens))
         st.set_tokens(tokens)
-        wall, ev_ms = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
-        us = ev_ms * 1e3 / args.steps
+        wall, us, reg = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
         wb, fl = st.weight_bytes(), st.flops(tokens)
         if tokens == 1:
-            out = dict(base, metric="int4_decoder_stack_decode_hbm_bandwidth", value=round(wb * args.steps / wall / 1e9, 1),
+            out = dict(base, metric="int4_decoder_stack_decode_hbm_bandwidth", value=round(wb / wall / 1e9, 1),
                        unit="GB/s", roofline={"bound": "hbm", "kernel": "fc_w4_stream_kernel (126 FCs per step; q/k/v and gate/up share a launch)",
                                               "achieved": round(wb / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                               "frac": round(wb / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
                                               "avg_step_us": round(us, 1)})
         else:
-            out = dict(base, metric="int4_decoder_stack_prefill_throughput", value=round(fl * args.steps / wall / 1e12, 1),
+            out = dict(base, metric="int4_decoder_stack_prefill_throughput", value=round(fl / wall / 1e12, 1),
                        unit="TFLOP/s", roofline={"bound": "mfma", "kernel": "fc_w4_mfma_gemm_kernel (126 FCs per step)",
                                                  "achieved": round(fl / us / 1e6, 1), "peak": 2500.0, "unit": "TFLOP/s",
                                                  "frac": round(fl / us / 1e6 / 2500.0, 4), "traffic": None,
                                                  "avg_step_us": round(us, 1)})
-        out.update(ms_per_step=round(wall * 1e3 / args.steps, 6), dtype="u4 weights x f16 activations, f32 accumulate",
-                   config={"workload": "c5: 18 layers x (q,k,v,o,gate,up,down) int4 group-32, hidden 2048, %d token(s) per step"
-                                       % tokens, "weight_bytes_per_step": wb, "flops_per_step": fl})
+        out.update(ms_per_step=round(wall * 1e3, 6), dtype="u4 weights x f16 activations, f32 accumulate",
+                   config=dict({"workload": "c5: 18 layers x (q,k,v,o,gate,up,down) int4 group-32, hidden 2048, %d token(s) "
+                                            "per step" % tokens, "weight_bytes_per_step": wb, "flops_per_step": fl}, **reg))
     print(json.dumps(out))
 
 
@@ -299,7 +327,7 @@ def main():
 
     # ring of ops: copy 0 holds the seeded case, the others random packed bytes (every byte
     # pattern is a valid pair of int4 codes)
-    devs = [W.FcDevice(case)]
+    devs = [W.FcDevice(case, reference_layout=args.layout == "reference")]
     gen = torch.Generator(device="cuda").manual_seed(1)
     ops = [devs[0].op]
     weights = [devs[0].weights]
@@ -320,7 +348,8 @@ def main():
         ops[0].launch(s)
         stream.synchronize()
         got = devs[0].result()
-        ref = case["act"].astype(np.float64) @ W.dequantized_weights(case).T
+        # per-channel symmetric weights: y = (x . q) * s, in float64
+        ref = (case["act"].astype(np.float64) @ case["w"].astype(np.float64).T) * case["scale"][:, 0].astype(np.float64)
         rel = np.abs(got - ref).max() / np.sqrt(np.mean(ref ** 2))
         if not rel <= 2e-2:
             print("result check failed: max|err|/rms = %g" % rel, file=sys.stderr)
@@ -338,40 +367,11 @@ def main():
             print(json.dumps({"traffic_probe": "done", "copy_bytes": 256 << 20, "kernel": kernel}))
             return
 
-        for i in range(max(args.warmup, args.ring)):  # every op allocates its workspace on first use
-            ops[i % args.ring].launch(s)
-        stream.synchronize()
-
-        use_graph = not args.no_graph
-        graph = None
-        if use_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                cs = torch.cuda.current_stream().cuda_stream
-                for i in range(args.steps):
-                    ops[i % args.ring].launch(cs)
-            graph.replay()  # untimed: first replay uploads the graph
-            stream.synchronize()
-
-        ev0 = torch.cuda.Event(enable_timing=True)
-        ev1 = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ev0.record(stream)
-        if use_graph:
-            graph.replay()
-        else:
-            for i in range(args.steps):
-                ops[i % args.ring].launch(s)
-        ev1.record(stream)
-        stream.synchronize()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        ev_ms = ev0.elapsed_time(ev1)
-
-    ms_per_step = wall * 1e3 / args.steps
-    value = algo_bytes * args.steps / wall / 1e9
-    launch_us = ev_ms * 1e3 / args.steps
+        wall, launch_us, reg = time_graph(torch, stream, lambda st, i: ops[i % args.ring].launch(st), args.steps,
+                                          max(args.warmup, args.ring), use_graph=not args.no_graph, ring=args.ring)
+    use_graph = not args.no_graph
+    ms_per_step = wall * 1e3
+    value = algo_bytes / wall / 1e9
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
 
     # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
@@ -397,7 +397,9 @@ def main():
         "dtype": "u4 weights x f16 activations, f32 accumulate",
         "data": "synthetic",
         "config": {"workload": "c2: FullyConnected decode GEMV M=1 K=4096 N=14336 int4 per-channel, fp16 act/out",
-                   "weight_ring": args.ring, "timed_region": "hipGraph replay" if use_graph else "eager launch loop",
+                   "weights_layout": "kOSpatialIOGroupI4O4, output_group_size %d" % devs[0].desc.output_group_size,
+                   "weight_ring": args.ring, "timed_region": "hipGraph replays" if use_graph else "eager launch loop",
+                   "graph_replays": reg["graph_replays"], "launches_per_replay": reg["launches_per_replay"],
                    "algorithmic_bytes_per_step": algo_bytes, "flops_per_step": flops,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,

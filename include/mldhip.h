@@ -13,7 +13,9 @@
  *  - Device pointers are caller-owned (the reference's tensors belong to its
  *    InferenceContext; external weights "must be valid during life of InferenceContext",
  *    common/gpu_model.h:83-96).  An op owns only its metadata and a small private
- *    device workspace allocated at creation.
+ *    device workspace, allocated by the create call (no launch allocates, so a first launch
+ *    may be recorded under stream capture).  Bound buffers must be 16-byte aligned (the kernels
+ *    use 128-bit loads and stores); mldhip_op_set_src / _set_dst reject others.
  *  - Launches are asynchronous on the caller's hipStream_t (passed as void*).  Handles
  *    are not thread-safe; creation functions are re-entrant.
  *  - Weight shapes are OHWI with H = W = 1 for ops; the host packers accept any H, W.
@@ -92,15 +94,34 @@ typedef struct {
 const char* mldhip_last_error(void);
 const char* mldhip_version(void);
 
+/* Overrides a launch heuristic of this library for the whole process (tests and tuning runs;
+ * the reference keeps its counterpart, the work-group size argument of
+ * CreateFullyConnectedExternalWeights, common/kernels/fully_connected.h:155-161, per call).
+ * value -1 restores the heuristic.  Knobs: force_generic, gemv_mfma, gemv_fast, gemv_lpr,
+ * gemv_waves, gemv_ksplit, gemv_narrow_max_mb, gemm_fm, gemm_ksplit, gemm_no_pair, gemm_dual,
+ * gemm_xcd_m, gemm_i8_fm.  MLDHIP_NOT_FOUND for an unknown name.  Not thread-safe against
+ * concurrent launches. */
+int mldhip_set_tuning(const char* name, int value);
+
 /* ------------------------------------------------------------------------------------ */
 /* Weight descriptions and host packers ("weights rearrangement")                         */
 /* ------------------------------------------------------------------------------------ */
 
 /* GetFullyConnectedInt8WeightsDesc / GetFullyConnectedInt4WeightsDesc
- * (common/kernels/fully_connected.h:185-192, .cc:1218-1246): uint8 / uint4,
- * kOSpatialIOGroupI4O4 (buffer storage), output_group_size = ceil(o/4). */
+ * (common/kernels/fully_connected.h:185-192, .cc:1218-1246): the layout this device's
+ * FullyConnected wants the builder to pack the weights in (the reference picks per GPU too:
+ * buffers or textures).  uint8: kOSpatialIOGroupI4O4 (buffer storage), output_group_size =
+ * ceil(o/4), exactly the reference's choice.  uint4: the same layout enum with
+ * output_group_size = 16 slices when o is a multiple of 64 (else ceil(o/4)): the reference's
+ * packers produce it from this description as they do any group size
+ * (common/task/weights_conversion.cc:139-185, 631-708), and the K rows of every 64-channel
+ * strip then lie one after the other in memory, which is what lets the decode GEMV stream at
+ * the rate of a plain copy on this device.  mldhip_fc_create takes either group size. */
 int mldhip_fc_int8_weights_desc(int o, int i, mldhip_weights_desc* desc);
 int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc);
+/* The reference's own GetFullyConnectedInt4WeightsDesc choice (one output group,
+ * output_group_size = ceil(o/4)), for weights that were packed for the reference's kernel. */
+int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* desc);
 
 /* The weights layout the int8 x int8 MFMA convolution asks for, the counterpart of the
  * conv_weights_desc that SelectConvolutionInt8 returns to the builder
@@ -236,7 +257,10 @@ int mldhip_fc_is_recommended(int precision, int tokens);
  * src_type INT8 selects the integer-math variant (fully_connected.cc:543-621, 874-903):
  * no scales, dst_type must be INT32. */
 typedef struct {
-  int32_t precision;  /* MLDHIP_PRECISION_*; F32 <=> fp32 tensors, otherwise fp16 tensors */
+  int32_t precision;  /* MLDHIP_PRECISION_*; F32 <=> fp32 tensors, otherwise fp16 tensors.  F16 is
+                         computed like F32_F16 (fp32 accumulation of fp16 products): at least as
+                         accurate as the reference's all-fp16 arithmetic
+                         (common/kernels/fully_connected_util.cc:167-203), not bit-identical to it */
   int32_t src_type;   /* MLDHIP_FLOAT32 / MLDHIP_FLOAT16 / MLDHIP_INT8 */
   int32_t dst_type;   /* MLDHIP_FLOAT32 / MLDHIP_FLOAT16 / MLDHIP_INT32 */
   int32_t o, i;       /* ExternalWeights::shape = OHWI(o,1,1,i) */

@@ -25,6 +25,10 @@ int Fail(int code, const std::string& msg) {
   g_error = msg;
   return code;
 }
+Tuning& GetTuning() {
+  static Tuning tuning;
+  return tuning;
+}
 }  // namespace mldhip
 
 namespace {
@@ -123,18 +127,45 @@ const char* mldhip_version(void) { return "mldhip 0.1 (gfx950)"; }
 // weight descriptions and packers
 // ---------------------------------------------------------------------------------------
 
-static int FcDesc(int o, int i, int type, mldhip_weights_desc* desc) {
+static int FcDesc(int o, int i, int type, bool native_groups, mldhip_weights_desc* desc) {
   if (!desc) return Fail(MLDHIP_INVALID_ARGUMENT, "null desc");
   if (o <= 0 || i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
   std::memset(desc, 0, sizeof(*desc));
   desc->type = type;
   desc->layout = MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4;
-  desc->output_group_size = DivUp(o, 4);
+  const int ns = DivUp(o, 4);
+  // uint4 weights of whole 64-channel strips: output groups of 16 slices, so that the K rows of a
+  // strip lie one after the other in memory
+  desc->output_group_size = (native_groups && o % 4 == 0 && ns % kNativeGroup == 0) ? kNativeGroup : ns;
   return MLDHIP_OK;
 }
 
-int mldhip_fc_int8_weights_desc(int o, int i, mldhip_weights_desc* desc) { return FcDesc(o, i, MLDHIP_UINT8, desc); }
-int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc) { return FcDesc(o, i, MLDHIP_UINT4, desc); }
+int mldhip_fc_int8_weights_desc(int o, int i, mldhip_weights_desc* desc) {
+  return FcDesc(o, i, MLDHIP_UINT8, false, desc);
+}
+int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc) {
+  return FcDesc(o, i, MLDHIP_UINT4, true, desc);
+}
+int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* desc) {
+  return FcDesc(o, i, MLDHIP_UINT4, false, desc);
+}
+
+int mldhip_set_tuning(const char* name, int value) {
+  if (!name) return Fail(MLDHIP_INVALID_ARGUMENT, "null name");
+  Tuning& t = GetTuning();
+  const struct { const char* name; int* field; } knobs[] = {
+      {"force_generic", &t.force_generic}, {"gemv_mfma", &t.gemv_mfma}, {"gemv_fast", &t.gemv_fast},
+      {"gemv_lpr", &t.gemv_lpr}, {"gemv_waves", &t.gemv_waves}, {"gemv_ksplit", &t.gemv_ksplit},
+      {"gemv_narrow_max_mb", &t.gemv_narrow_max_mb}, {"gemm_fm", &t.gemm_fm}, {"gemm_ksplit", &t.gemm_ksplit},
+      {"gemm_no_pair", &t.gemm_no_pair}, {"gemm_dual", &t.gemm_dual}, {"gemm_xcd_m", &t.gemm_xcd_m},
+      {"gemm_i8_fm", &t.gemm_i8_fm}};
+  for (const auto& k : knobs)
+    if (std::strcmp(name, k.name) == 0) {
+      *k.field = value;
+      return MLDHIP_OK;
+    }
+  return Fail(MLDHIP_NOT_FOUND, std::string("unknown tuning knob: ") + name);
+}
 
 int mldhip_conv_int8_weights_desc(int o, int i, mldhip_weights_desc* desc) {
   if (!desc) return Fail(MLDHIP_INVALID_ARGUMENT, "null desc");
@@ -298,6 +329,13 @@ int mldhip_fc_is_recommended(int precision, int tokens) {
 
 static int AllocWorkspace(mldhip_op* op, int n) {
   if (op->partial) return MLDHIP_OK;
+  // A host without a GPU can still create and inspect ops (object lists, validation); they cannot
+  // be launched there, so they need no workspace.
+  int devices = 0;
+  if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
+    (void)hipGetLastError();
+    return MLDHIP_OK;
+  }
   const int n_pad = DivUp(n, 4) * 4;
   op->partial_floats = std::max((size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad,
                                 FcW4MfmaWorkspaceFloats(op->fc.max_tokens, op->fc.i, op->fc.o));
@@ -323,8 +361,13 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
       return Fail(MLDHIP_UNIMPLEMENTED, "texture weight layouts are not supported; use the buffer layout");
     return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout");
   }
-  if (wd.output_group_size != DivUp(d->o, 4))
-    return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
+  {
+    const int ns = DivUp(d->o, 4);
+    const bool native = wd.type == MLDHIP_UINT4 && wd.output_group_size == kNativeGroup && d->o % 4 == 0 &&
+                        ns % kNativeGroup == 0 && !batch_ids;
+    if (wd.output_group_size != ns && !native)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
+  }
   if (d->precision < MLDHIP_PRECISION_F32 || d->precision > MLDHIP_PRECISION_F16)
     return Fail(MLDHIP_INVALID_ARGUMENT, "bad precision");
   const bool int8_math = d->src_type == MLDHIP_INT8;
@@ -373,6 +416,14 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     op->AddSrc("biases");
   }
   op->AddDst("dst_tensor");
+  // split-K workspace of the fp16 streaming and matrix-core kernels: allocated here, so that no
+  // launch allocates (a first launch may be under stream capture)
+  if (!int8_math && d->src_type == MLDHIP_FLOAT16) {
+    if (int rc = AllocWorkspace(op, d->o)) {
+      delete op;
+      return rc;
+    }
+  }
   *out = op;
   return MLDHIP_OK;
 }
@@ -463,6 +514,8 @@ int mldhip_op_set_src(mldhip_op* op, int index, const void* device_ptr, size_t b
   if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
   if (index < 0 || index >= (int)op->src_ptr.size()) return Fail(MLDHIP_OUT_OF_RANGE, "src index out of range");
   if (!device_ptr) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  if (reinterpret_cast<uintptr_t>(device_ptr) % 16 != 0)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "src object '" + op->src_names[index] + "' is not 16-byte aligned");
   op->src_ptr[index] = device_ptr;
   op->src_bytes[index] = bytes;
   return MLDHIP_OK;
@@ -472,6 +525,8 @@ int mldhip_op_set_dst(mldhip_op* op, int index, void* device_ptr, size_t bytes) 
   if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
   if (index < 0 || index >= (int)op->dst_ptr.size()) return Fail(MLDHIP_OUT_OF_RANGE, "dst index out of range");
   if (!device_ptr) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  if (reinterpret_cast<uintptr_t>(device_ptr) % 16 != 0)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "dst object '" + op->dst_names[index] + "' is not 16-byte aligned");
   op->dst_ptr[index] = device_ptr;
   op->dst_bytes[index] = bytes;
   return MLDHIP_OK;
@@ -547,13 +602,7 @@ static int CheckBindings(const mldhip_op* op) {
   return MLDHIP_OK;
 }
 
-static int EnvFlag(const char* name) {
-  const char* v = std::getenv(name);
-  return v && v[0] && v[0] != '0';
-}
-
-// The launch arguments of a floating-point FC op at its current bindings and shape; allocates
-// the op's split-K workspace on first use.
+// The launch arguments of a floating-point FC op at its current bindings and shape.
 static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
   const mldhip_fc_desc& d = op->fc;
   FcArgs a;
@@ -576,14 +625,12 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
   a.act_f16 = d.src_type == MLDHIP_FLOAT16;
   a.dst_f16 = d.dst_type == MLDHIP_FLOAT16;
   a.weight_bits = WeightBits(d.weights.type);
+  a.group = d.weights.output_group_size;
   a.scale_kind = d.scale_o * d.scale_i == 1 ? kScaleScalar : (d.scale_i == 1 ? kScaleLinear : kScaleBlock);
   a.groups = d.scale_i;
   a.scalar_scale = d.scalar_scale;
   a.has_zero_point = d.has_zero_point_tensor || d.has_scalar_zero_point;
   a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
-  // split-K workspace of the fp16 streaming and matrix-core kernels: allocated once, on the first launch
-  if ((a.weight_bits == 4 || a.weight_bits == 8) && a.act_f16)
-    if (int rc = AllocWorkspace(op, d.o)) return rc;
   a.partial = op->partial;
   a.partial_floats = op->partial_floats;
   *out = a;
@@ -608,17 +655,18 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         batch.weights_batch = op->weights_batch;
         tokens = op->w;
       }
+      batch.group = d.weights.output_group_size;
       const int8_t* act = static_cast<const int8_t*>(op->src_ptr[0]);
       const uint8_t* weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
       int32_t* dst = static_cast<int32_t*>(op->dst_ptr[0]);
-      if (!EnvFlag("MLDHIP_FORCE_GENERIC") && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
+      if (GetTuning().force_generic <= 0 && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
         e = LaunchFcInt8MathStream(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
       else
         e = LaunchFcInt8Math(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
-      const bool force_generic = EnvFlag("MLDHIP_FORCE_GENERIC");
+      const bool force_generic = GetTuning().force_generic > 0;
       // batched weights by runtime ids: the streaming GEMVs, else the unspecialised kernel
       if (a.batch_ids != nullptr) {
         if (!force_generic && FcW4StreamSupported(a))
@@ -629,8 +677,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
           e = LaunchFcGeneric(a, stream, &op->last_kernel);
       } else
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
-      // on the vector-ALU kernel; MLDHIP_GEMV_MFMA=1 forces the matrix-core one there too)
-      if (!force_generic && (a.m >= 2 || EnvFlag("MLDHIP_GEMV_MFMA")) && FcW4MfmaStreamSupported(a)) {
+      // on the vector-ALU kernel; the tuning knob gemv_mfma = 1 forces the matrix-core one there too)
+      if (!force_generic && (a.m >= 2 || GetTuning().gemv_mfma > 0) && FcW4MfmaStreamSupported(a)) {
         e = LaunchFcW4MfmaStream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4StreamSupported(a)) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);

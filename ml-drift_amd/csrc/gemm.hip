@@ -51,6 +51,7 @@ struct W4Segment {
   __half* dst;
   float* partial;  // [ksplit][Ns][m][4] fp32 sums when ksplit > 1
   int n, ns;
+  int group;  // slices per output group of the packed weights (ns: one group, the rows span all of N)
   int tile_end;
   uint32_t a_bytes, s_bytes;
 };
@@ -626,10 +627,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int shares = KW * p.ksplit;  // blockIdx.y selects the work-group's part of K
   const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
   const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * KW + wave % KW) * per_wave);
-  const uint32_t row_w = (uint32_t)sg.ns * kBlk;  // bytes per K-slice row of the weights
+  // Weights with output groups: the K-slice rows of a group lie one after the other (row = the
+  // group's slices), the groups one after the other.  With one group the buffer ends, for this
+  // wave, where its share of K ends; with several, a prefetch past the share reads other rows of
+  // the buffer, which meet the zeros that the activations' descriptor returns there.
+  const bool one_group = sg.group >= sg.ns;
+  const uint32_t row_w = (uint32_t)sg.group * kBlk;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
-  const uint32_t w_end = min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w);
+  const uint32_t w_end = one_group ? (uint32_t)min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w) : sg.a_bytes;
   const uint32_t x_end = min((uint64_t)p.b_bytes, (uint64_t)k_slices_end * row_x);
 
   constexpr uint32_t kOob = 0x7FFFFFF0u;
@@ -657,7 +663,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
   // address lives there.
   const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
-  uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + (uint32_t)nsi * kBlk : kOob;
+  const uint32_t col_w = one_group ? (uint32_t)nsi * kBlk
+                                   : ((uint32_t)(nsi / sg.group) * (uint32_t)p.ks * (uint32_t)sg.group + (uint32_t)(nsi % sg.group)) * kBlk;
+  uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + col_w : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
   // token of this lane in MFMA token block fm
   auto token = [&](int fm) { return PAIR ? m0 + (fm / 2) * 64 + 2 * i32 + (fm & 1) : m0 + fm * 32 + i32; };
@@ -1096,6 +1104,8 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     sg.partial = args[i].partial;
     sg.n = args[i].n;
     sg.ns = DivUp(args[i].n, 4);
+    sg.group = EffectiveGroup(args[i].group, sg.ns);
+    if (sg.ns % sg.group != 0) return hipErrorInvalidValue;  // whole groups only
     if (args[i].weight_bits != a.weight_bits) return hipErrorInvalidValue;
     sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * (a.weight_bits == 8 ? 16 : 8));
     sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8);
@@ -1115,15 +1125,16 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
                          : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
-  if (const char* e = std::getenv("MLDHIP_GEMM_FM")) fm = std::atoi(e) == 1 ? 1 : (std::atoi(e) == 4 && a.m % 2 == 0 ? 4 : 2);
+  const Tuning& tune = GetTuning();
+  if (tune.gemm_fm > 0) fm = tune.gemm_fm == 1 ? 1 : (tune.gemm_fm == 4 && a.m % 2 == 0 ? 4 : 2);
   p.ksplit = 1;
   if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
-  if (const char* e = std::getenv("MLDHIP_GEMM_KSPLIT")) p.ksplit = std::max(1, std::atoi(e));
+  if (tune.gemm_ksplit > 0) p.ksplit = tune.gemm_ksplit;
   if (gated) p.ksplit = 1;  // the epilogue needs whole sums
   for (int i = 0; i < count; ++i)
     while (p.ksplit > 1 && (size_t)p.ksplit * p.seg[i].ns * 4 * a.m > args[i].partial_floats) p.ksplit /= 2;
   const int tiles_m = DivUp(a.m, fm * 32);
-  const bool pair = a.m % 2 == 0 && !std::getenv("MLDHIP_GEMM_NO_PAIR");
+  const bool pair = a.m % 2 == 0 && tune.gemm_no_pair <= 0;
   // Two channel tiles per work-group when the rounds of 256 work-groups come out cheaper: a
   // two-tile work-group takes 1.87 x the time of a one-tile one, and a last round filled to the
   // fraction f costs 0.45 + 0.55 f of a full one (fitted to same-box timings of 14 shapes).
@@ -1133,10 +1144,10 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     return whole + (f > 0.0 ? 0.45 + 0.55 * f : 0.0);
   };
   p.dual = dual_ok && 1.87 * rounds((long)DivUp(tiles_n, 2) * tiles_m) < 0.97 * rounds((long)tiles_n * tiles_m);
-  if (const char* e = std::getenv("MLDHIP_GEMM_DUAL")) p.dual = dual_ok && std::atoi(e) != 0;
+  if (tune.gemm_dual >= 0) p.dual = dual_ok && tune.gemm_dual != 0;
   if (p.dual) tiles_n = DivUp(tiles_n, 2);
   p.xcd_m = W4XcdGrid(tiles_m, tiles_n, fm * 32, a.k, p.groups);
-  if (const char* e = std::getenv("MLDHIP_GEMM_XCD_M")) p.xcd_m = std::atoi(e);
+  if (tune.gemm_xcd_m > 0) p.xcd_m = tune.gemm_xcd_m;
   if (p.xcd_m != 1 && p.xcd_m != 2 && p.xcd_m != 4 && p.xcd_m != 8) p.xcd_m = 8;
   const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
   const bool zp = p.seg[0].zp != nullptr;
@@ -1217,8 +1228,8 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
   if (kernel_name) *kernel_name = "conv_int8_mfma_kernel";
   // token tile: the largest of 256 / 128 / 64 that still gives most CUs a work-group
   auto tiles = [&](int bm) { return (long)DivUp(p.n, 256) * DivUp(p.m, bm); };
-  if (const char* e = std::getenv("MLDHIP_GEMM_I8_FM")) {  // tuning override: token tile in blocks of 64
-    const int fm = std::atoi(e);
+  if (GetTuning().gemm_i8_fm > 0) {  // tuning override: token tile in blocks of 64
+    const int fm = GetTuning().gemm_i8_fm;
     if (fm == 4) return LaunchConvInt8Tile<4>(p, stream);
     if (fm == 2) return LaunchConvInt8Tile<2>(p, stream);
     if (fm == 1) return LaunchConvInt8Tile<1>(p, stream);

@@ -46,6 +46,7 @@ struct GenericParams {
   const void* bias;
   void* dst;
   int m, ks, ns;
+  int wgroup;  // output group size of the packed weights (slices)
   int scale_kind, groups, group_slices;
   float scalar_scale, scalar_zero_point;
   int has_zero_point;
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
           if (zp) z[c] = LoadF(zp, sidx + c);
         }
       }
-      const size_t blk = (size_t)ks * p.ns + ds;
+      const size_t blk = BlockIndex(ks, ds, p.ks, p.ns, p.wgroup);
       float wf[4][4];
       if (WBITS == 8) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(weights + blk * 16);
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
   if (ds < ns) {
 #pragma unroll 4
     for (int ks = ty; ks < ks_n; ks += kKl) {
-      const size_t blk = (size_t)ks * ns + ds;
+      const size_t blk = BlockIndex(ks, ds, ks_n, ns, batch.group);
       uint32_t w0, w1, w2, w3;  // per output channel: the 4 input-channel values, one per byte
       if (WBITS == 4) {
         const u32x2 w = *reinterpret_cast<const u32x2*>(weights + blk * 8);
@@ -287,6 +288,7 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
   p.m = a.m;
   p.ks = DivUp(a.k, 4);
   p.ns = DivUp(a.n, 4);
+  p.wgroup = a.group;
   p.scale_kind = a.scale_kind;
   p.groups = a.groups;
   p.group_slices = a.scale_kind == kScaleBlock ? (p.ks / a.groups > 0 ? p.ks / a.groups : 1) : p.ks;

@@ -34,6 +34,7 @@ struct I8MathParams {
   int* dst;        // [Ns][m][4]
   int m, ks, ns;
   int row_u4;  // 16-byte items per K-slice row
+  int gu4;     // 16-byte items per row of one output group of the packed weights (row_u4: one group)
   int chunks;  // ceil(ks / 8)
   FcBatchRows batch;  // batched weights selected by runtime ids: blockIdx.z = dst row
 };
@@ -67,7 +68,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
   const int brow = BATCHED ? (int)blockIdx.z : 0;
   int wb = BATCHED ? p.batch.ids[brow] : 0;
   if (BATCHED) wb = min(max(wb, 0), p.batch.weights_batch - 1);
-  const u32x4* weights = p.weights + (BATCHED ? (size_t)wb * p.ks * p.row_u4 : 0);
+  // column of this lane: with output groups, the rows of a group lie one after the other
+  const u32x4* weights = p.weights + (BATCHED ? (size_t)wb * p.ks * p.row_u4 : 0) +
+                         ((size_t)(item / p.gu4) * p.ks * p.gu4 + item % p.gu4);
   const int act_stride = BATCHED ? p.batch.src_rows * M : M, act_tok0 = BATCHED ? min(brow, p.batch.src_rows - 1) * M : 0;
   const int dst_stride = BATCHED ? p.batch.rows * M : M, dst_tok0 = BATCHED ? brow * M : 0;
 
@@ -86,7 +89,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
     for (int j = 0; j < 8; ++j) {
       const int ks = c * 8 + j;
       const int ksc = min(ks, p.ks - 1);
-      w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * p.row_u4 + item);
+      w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * p.gu4);
 #pragma unroll
       for (int m = 0; m < M; ++m) {
         const int v = p.act[(size_t)ksc * act_stride + act_tok0 + m];
@@ -210,6 +213,9 @@ hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int
   p.ks = DivUp(k, 4);
   p.ns = DivUp(n, 4);
   p.row_u4 = weight_bits == 4 ? p.ns / 2 : p.ns;
+  const int group = EffectiveGroup(batch.group, p.ns);
+  if (p.ns % group != 0 || (weight_bits == 4 && group % 2 != 0)) return hipErrorInvalidValue;
+  p.gu4 = weight_bits == 4 ? group / 2 : group;
   p.chunks = DivUp(p.ks, 8);
   // 128-byte row segments when that still gives a work-group to half the CUs, else 64-byte ones;
   // small work-groups for several tokens (LDS) and when K is covered by few rows of chunks

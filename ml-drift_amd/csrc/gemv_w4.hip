@@ -25,7 +25,7 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
+#include <algorithm>
 
 #include "../../include/mldhip.h"
 #include "gated.h"
@@ -61,14 +61,17 @@ struct StreamSegment {
   __half* dst;
   int ns, n_pad;  // n_pad = ns * 4
   int row_u4;     // uint4 per packed row = ns / 2
+  int gu4;        // uint4 per row of one output group of the packed weights (row_u4: one group)
   int strip_end;
+  int n_off;      // channels of the launch's matrices before this one (split-K sums of fused launches)
 };
 
 struct StreamParams {
   StreamSegment seg[kMaxSegments];
   int segments;
   const __half* act;
-  float* partial;  // split-K sums (single-matrix launches only)
+  float* partial;  // split-K sums: [split][token][n_total]
+  int n_total;     // padded channels of all matrices of the launch
   int m, ks;
   int chunks;            // ceil(ks / 8)
   int chunks_per_split;
@@ -96,15 +99,16 @@ __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const 
 // be counted down one by one while the arithmetic of the earlier slices runs.
 // act_stride / act_tok0: tokens per K-slice row of the activation tensor and the first token of
 // this launch row in it (M and 0 unless the launch has batched weights).
+// wcol: the lane's column of the packed weights (K-slice row 0), rstride: uint4 per K-slice row.
 template <int M>
-__device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* weights, int row_u4, int c, int pcol,
+__device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* wcol, int rstride, int c,
                                           u32x4 w[8], u32x2 a[8][M], int act_stride = M, int act_tok0 = 0) {
   const int ks0 = c * 8;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const int ks = ks0 + j;
     const int ksc = min(ks, p.ks - 1);
-    w[j] = __builtin_nontemporal_load(weights + (size_t)ksc * row_u4 + pcol);
+    w[j] = __builtin_nontemporal_load(wcol + (size_t)ksc * rstride);
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       const u32x2 v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksc * act_stride + act_tok0 + m) * 4);
@@ -115,8 +119,8 @@ __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* we
 
 // t[m][o] += sum over the chunk of a * (c_o + u), c_o = 1024 for even o, 64 for odd o;
 // asum[m] += sum over the chunk of a.
-template <int M>
-__device__ __forceinline__ void ComputeChunk(const StreamParams& p, const u32x4 w[8], const u32x2 a[8][M],
+template <int M, typename Params>
+__device__ __forceinline__ void ComputeChunk(const Params& p, const u32x4 w[8], const u32x2 a[8][M],
                                              float t[M][8], float asum[M]) {
   const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
@@ -194,6 +198,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   const int pcol_raw = strip * LPR + col;  // uint4 column = output channels 8*pcol .. +7
   const bool col_ok = pcol_raw < row_u4;
   const int pcol = col_ok ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
+  // with output groups, the rows of a group lie one after the other
+  const u32x4* wcol = weights + ((size_t)(pcol / sg.gu4) * p.ks * sg.gu4 + pcol % sg.gu4);
+  const int rstride = sg.gu4;
   const int ky = blockIdx.y;
   const int c_begin = ky * p.chunks_per_split;
   const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
@@ -220,13 +227,13 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   if (c < c_end) {
     u32x4 w[8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, weights, row_u4, c, pcol, w, a, act_stride, act_tok0);
+    LoadChunk<M>(p, wcol, rstride, c, w, a, act_stride, act_tok0);
     while (true) {
       const int cn = c + ROWS;
       const bool more = cn < c_end;
       u32x4 wn[8];
       u32x2 an[8][M];
-      if (more) LoadChunk<M>(p, weights, row_u4, cn, pcol, wn, an, act_stride, act_tok0);
+      if (more) LoadChunk<M>(p, wcol, rstride, cn, wn, an, act_stride, act_tok0);
       u32x4 sv;
       if (GROUPED) {
         int g = c / p.group_chunks;
@@ -310,13 +317,17 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   }
 }
 
-// Adds the split-K partial sums in split order and writes the output.
+// Adds the split-K partial sums in split order and writes the output.  The sums of a launch are
+// [split][token][channels of all its matrices]; n_total = those channels.
 template <bool GROUPED>
-__global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
-  const StreamSegment& sg = p.seg[0];
+__global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p, int n_total) {
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= p.m * sg.n_pad) return;
-  const int m = idx / sg.n_pad, n = idx % sg.n_pad;
+  if (idx >= p.m * n_total) return;
+  const int m = idx / n_total, nt = idx % n_total;
+  int si = 0;
+  if (p.segments > 1 && nt >= p.seg[1].n_off) si = (p.segments > 2 && nt >= p.seg[2].n_off) ? 2 : 1;
+  const StreamSegment& sg = p.seg[si];
+  const int n = nt - sg.n_off;
   // The parts are fetched eight at a time before any is added (a part past the last re-reads the
   // last one and is dropped by a select), so that their latencies overlap; added in split order.
   const float scale = GROUPED ? 1.0f : __half2float(sg.scale[n]);
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p) {
     float part[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j)
-      part[j] = p.partial[((size_t)min(s0 + j, p.ksplit - 1) * p.m + m) * sg.n_pad + n];
+      part[j] = p.partial[((size_t)min(s0 + j, p.ksplit - 1) * p.m + m) * n_total + nt];
 #pragma unroll
     for (int j = 0; j < 8; ++j) v += s0 + j < p.ksplit ? part[j] : 0.0f;
   }
@@ -362,6 +373,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_gated_stream_kernel(StreamPa
   const int row_u4 = p.seg[0].row_u4;
   const int pcol_raw = strip * LPR + col;
   const int pcol = pcol_raw < row_u4 ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
+  const int rstride = p.seg[0].gu4;
+  const size_t wcol_off = (size_t)(pcol / rstride) * p.ks * rstride + pcol % rstride;
 
   // scales / biases of the output this thread finishes, fetched ahead (raw halfs, clamped index)
   const int n_out = min(strip * STRIP + tid % STRIP, p.seg[0].n_pad - 1);
@@ -384,12 +397,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_gated_stream_kernel(StreamPa
   for (int c = row; c < p.chunks; c += ROWS) {
     u32x4 w[2][8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, p.seg[0].weights, row_u4, c, pcol, w[0], a);
+    LoadChunk<M>(p, p.seg[0].weights + wcol_off, rstride, c, w[0], a);
     {
       const int ks0 = c * 8;
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        w[1][j] = __builtin_nontemporal_load(p.seg[1].weights + (size_t)min(ks0 + j, p.ks - 1) * row_u4 + pcol);
+        w[1][j] = __builtin_nontemporal_load(p.seg[1].weights + wcol_off + (size_t)min(ks0 + j, p.ks - 1) * rstride);
     }
     u32x4 sv[2];
     if (GROUPED) {
@@ -548,9 +561,261 @@ hipError_t LaunchBatchedM(const StreamParams& p, bool grouped, dim3 grid, hipStr
   }
 }
 
-int EnvInt(const char* name, int fallback) {
-  const char* v = std::getenv(name);
-  return v ? std::atoi(v) : fallback;
+// ------------------------------------------------------------------------------------------
+// One token over weights packed in output groups of 16 slices (64 channels): the share of a
+// work-group, 64 channels x its range of K, is one contiguous run of 128-byte rows, which HBM
+// delivers at the rate of a plain copy.  Lane = (column of 16 bytes, row): a thread owns 8
+// consecutive K-slices (one 32-channel scale group), its 8 loads are one base address plus
+// immediate offsets, the 8 slices of its activations are 64 contiguous bytes.  Nothing in front of
+// the loads but the address: the kernel's time is the stream's, and every instruction ahead of
+// the first load delays all of it.
+// K reduction: inside a wave by register exchanges that halve the live values per step (the two
+// row halves with v_permlane32_swap, the 16-lane rows with v_permlane16_swap, the 8-lane halves
+// of a row with a DPP rotate), after which lane l holds channel (l % 8) * 8 + l / 8 of the
+// strip; across waves through 4 KB of LDS, fixed order.
+// ------------------------------------------------------------------------------------------
+typedef uint32_t u32x2s __attribute__((ext_vector_type(2)));
+
+// Sum over the 8 rows of a wave of the 8 channel sums of every lane; the result of channel
+// (lane % 8) * 8 + lane / 8 is returned in this lane.  All 64 lanes must be active.
+__device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
+  float s4[4], s2[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const u32x2s r = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[i]), __float_as_uint(acc[i + 4]), false, false);
+    s4[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const u32x2s r = __builtin_amdgcn_permlane16_swap(__float_as_uint(s4[i]), __float_as_uint(s4[i + 2]), false, false);
+    s2[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    s2[i] += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s2[i]), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+  return (lane & 8) ? s2[1] : s2[0];
+}
+
+// Launch parameters of the strip kernel: what a single-matrix launch reads sits in the first
+// 128 bytes, so that two scalar loads issued at the top of the kernel bring all of it.
+struct StripSegment {
+  const u32x4* weights;
+  const __half* scale;
+  const __half* zero_point;  // same shape as scale, or null
+  const __half* bias;
+  __half* dst;
+  int n_pad;      // channels of the matrix (a multiple of 64)
+  int strip_end;  // work-groups [strip_end of the previous, strip_end) belong to this matrix
+  int n_off;      // channels of the launch's matrices before this one (split-K sums)
+  int reserved;
+};
+struct StripParams {
+  const __half* act;
+  float* partial;  // split-K sums: [split][n_total]
+  int ks, chunks, chunks_per_split, ksplit;
+  int group_chunks, n_total, segments, reserved;
+  uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+  StripSegment seg[kMaxSegments];
+};
+
+template <int WAVES, bool GROUPED, bool ZP, bool MULTI>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) {
+  constexpr int ROWS = WAVES * 8;  // chunks of 8 K-slices the work-group covers per pass
+  constexpr int STRIP = 64;
+  __shared__ float red[WAVES][STRIP];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane & 7;
+  const int row = tid >> 3;
+  int si = 0, strip = blockIdx.x;
+  if (MULTI && p.segments > 1 && strip >= p.seg[0].strip_end) {
+    si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
+    strip -= p.seg[si - 1].strip_end;
+  }
+  const StripSegment& sg = p.seg[MULTI ? si : 0];
+  // Everything the loop reads from the arguments, fetched here in one go: a scalar load first
+  // issued inside the loop would be a second round trip in front of the weight loads.
+  struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
+  const u32x4* weights = sg.weights;
+  const u32x4* astrip = reinterpret_cast<const u32x4*>(p.act);  // chunk c: 4 uint4 (8 slices x 4 halfs)
+  const __half* scale = sg.scale;
+  const __half* zero_point = sg.zero_point;
+  int ks = p.ks, group_chunks = p.group_chunks, n_pad = sg.n_pad;
+  asm volatile("" : "+s"(up.mask_lo), "+s"(up.mask_hi), "+s"(ks), "+s"(group_chunks), "+s"(n_pad));
+  // (the pointers are left to the compiler: through an asm operand they would lose their address
+  // space and turn every load into a flat one)
+  const int ky = blockIdx.y;
+  const int c_begin = ky * p.chunks_per_split;
+  const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
+  // the output this thread finishes: channel `ch` of the strip (the channel the wave sum leaves in
+  // this lane when the work-group is one wave, else thread order)
+  const int ch = WAVES == 1 ? (lane & 7) * 8 + (lane >> 3) : (tid & 63);
+  const int n_out = strip * STRIP + ch;
+  const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(sg.bias ? sg.bias : sg.scale);
+  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(scale)[n_out];
+  const unsigned short out_bias_raw = bias_src[n_out];
+
+  float acc[8];
+#pragma unroll
+  for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
+  u32x4 zv = {0u, 0u, 0u, 0u};
+  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * STRIP + col * 8);
+  // row r of the strip: 8 uint4; chunk c: 64 uint4
+  const u32x4* wstrip = weights + (size_t)strip * ks * 8 + col;
+  for (int c = c_begin + row; c < c_end; c += ROWS) {
+    const u32x4* wp = wstrip + (size_t)c * 64;
+    u32x4 w[8], a4[4];
+    // The small loads first (activations and scales come from cache), then the eight weight loads
+    // back to back; the fence keeps the arithmetic behind all of them, so that the waits count the
+    // weight loads down one by one instead of some of them being issued after the first wait.
+#pragma unroll
+    for (int j = 0; j < 4; ++j) a4[j] = astrip[c * 4 + j];
+    u32x4 sv;
+    if (GROUPED) {
+      const int g = c / group_chunks;
+      const size_t so = (size_t)g * n_pad + (size_t)strip * STRIP + col * 8;
+      sv = *reinterpret_cast<const u32x4*>(scale + so);
+      if (ZP) zv = *reinterpret_cast<const u32x4*>(zero_point + so);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + j * 8);
+    __builtin_amdgcn_sched_barrier(0);
+    u32x2 a[8][1];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) a[j][0] = u32x2{a4[j >> 1][2 * (j & 1)], a4[j >> 1][2 * (j & 1) + 1]};
+    float t[1][8], asum[1] = {0.0f};
+#pragma unroll
+    for (int o = 0; o < 8; ++o) t[0][o] = 0.0f;
+    ComputeChunk<1>(up, w, a, t, asum);
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+      float centre = (o & 1) ? -72.0f : -1032.0f;
+      if (ZP) centre -= (float)AsHalf2(zv[o >> 1])[o & 1];
+      const float centered = fmaf(centre, asum[0], t[0][o]);
+      if (GROUPED) {
+        const half2_t sp = AsHalf2(sv[o >> 1]);
+        acc[o] = fmaf((float)sp[o & 1], centered, acc[o]);
+      } else {
+        acc[o] += centered;
+      }
+    }
+  }
+  float v = WaveStripSum(acc, lane);
+  if (WAVES > 1) {
+    red[wave][(lane & 7) * 8 + (lane >> 3)] = v;
+    __syncthreads();
+    if (tid >= STRIP) return;
+    v = 0.0f;
+#pragma unroll
+    for (int q = 0; q < WAVES; ++q) v += red[q][tid];
+  }
+  if (p.ksplit == 1) {
+    if (!GROUPED) v *= __half2float(__ushort_as_half(out_scale_raw));
+    __half h = __float2half_rn(v);
+    if (sg.bias) h = __hadd(h, __ushort_as_half(out_bias_raw));
+    sg.dst[n_out] = h;
+  } else {
+    p.partial[(size_t)ky * p.n_total + sg.n_off + n_out] = v;
+  }
+}
+
+template <int WAVES>
+hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
+  const dim3 block(WAVES * 64);
+#define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<WAVES, G, Z, MU>), grid, block, 0, stream, p)
+  if (grouped) {
+    if (zp) { if (multi) MLD_STRIP(true, true, true); else MLD_STRIP(true, true, false); }
+    else    { if (multi) MLD_STRIP(true, false, true); else MLD_STRIP(true, false, false); }
+  } else {
+    if (zp) { if (multi) MLD_STRIP(false, true, true); else MLD_STRIP(false, true, false); }
+    else    { if (multi) MLD_STRIP(false, false, true); else MLD_STRIP(false, false, false); }
+  }
+#undef MLD_STRIP
+  return hipGetLastError();
+}
+
+// The contiguous-strip kernel serves: one token, every matrix of the launch packed in output
+// groups of 16 slices, K a multiple of 32 channels (whole chunks).
+bool StripKernelServes(const FcArgs* args, int count) {
+  if (GetTuning().gemv_fast == 0) return false;
+  if (args[0].m != 1 || args[0].batch_ids != nullptr) return false;
+  if (DivUp(args[0].k, 4) % 8 != 0 || args[0].k % 4 != 0) return false;
+  for (int i = 0; i < count; ++i) {
+    const int ns = DivUp(args[i].n, 4);
+    if (args[i].n % 4 != 0 || ns % kNativeGroup != 0 || EffectiveGroup(args[i].group, ns) != kNativeGroup) return false;
+  }
+  return true;
+}
+
+hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grouped, hipStream_t stream) {
+  const Tuning& tune = GetTuning();
+  int strips = 0;
+  for (int i = 0; i < count; ++i) {
+    strips += p.seg[i].ns / kNativeGroup;
+    p.seg[i].strip_end = strips;
+  }
+  // K stays inside the work-group when the strips alone fill the chip; else it is split into
+  // power-of-two runs of at least 8 chunks (one wave) so that about 256 work-groups exist.
+  int cps = p.chunks;
+  if (strips < 128 && p.chunks > 8) {
+    const int want = DivUp(256, strips);
+    cps = 8;
+    while (cps * 2 * want <= p.chunks) cps *= 2;
+  }
+  if (tune.gemv_ksplit > 0) cps = std::max(1, DivUp(p.chunks, tune.gemv_ksplit));
+  int ksplit = DivUp(p.chunks, cps);
+  if (ksplit > kGemvMaxKSplit) {
+    ksplit = kGemvMaxKSplit;
+    cps = DivUp(p.chunks, ksplit);
+    ksplit = DivUp(p.chunks, cps);
+  }
+  while (ksplit > 1 && (size_t)ksplit * p.n_total > args[0].partial_floats) {
+    --ksplit;
+    cps = DivUp(p.chunks, ksplit);
+    ksplit = DivUp(p.chunks, cps);
+  }
+  p.chunks_per_split = cps;
+  p.ksplit = ksplit;
+  int waves = 1;
+  while (waves < 16 && waves * 8 < cps) waves *= 2;
+  if (tune.gemv_waves > 0) waves = tune.gemv_waves;
+  const dim3 grid(strips, ksplit);
+  StripParams sp;
+  sp.act = p.act;
+  sp.partial = p.partial;
+  sp.ks = p.ks;
+  sp.chunks = p.chunks;
+  sp.chunks_per_split = p.chunks_per_split;
+  sp.ksplit = p.ksplit;
+  sp.group_chunks = p.group_chunks;
+  sp.n_total = p.n_total;
+  sp.segments = p.segments;
+  sp.reserved = 0;
+  sp.mask_lo = p.mask_lo;
+  sp.mask_hi = p.mask_hi;
+  sp.magic_lo = p.magic_lo;
+  sp.magic_hi = p.magic_hi;
+  for (int i = 0; i < kMaxSegments; ++i) {
+    const StreamSegment& g = p.seg[i];
+    sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, g.strip_end, g.n_off, 0};
+  }
+  hipError_t e;
+  switch (waves) {
+    case 1: e = LaunchStripW<1>(sp, grouped, grid, stream); break;
+    case 2: e = LaunchStripW<2>(sp, grouped, grid, stream); break;
+    case 4: e = LaunchStripW<4>(sp, grouped, grid, stream); break;
+    case 8: e = LaunchStripW<8>(sp, grouped, grid, stream); break;
+    default: e = LaunchStripW<16>(sp, grouped, grid, stream); break;
+  }
+  if (e != hipSuccess || ksplit == 1) return e;
+  const int total = p.m * p.n_total;
+  if (grouped)
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.n_total);
+  else
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.n_total);
+  return hipGetLastError();
 }
 
 }  // namespace
@@ -586,7 +851,7 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   p.mask_hi = 0x00F000F0u;
   p.magic_lo = 0x64006400u;
   p.magic_hi = 0x54005400u;
-  int total_row_u4 = 0;
+  int total_row_u4 = 0, n_total = 0;
   size_t weight_bytes = 0;
   for (int i = 0; i < count; ++i) {
     StreamSegment& sg = p.seg[i];
@@ -598,10 +863,16 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     sg.ns = DivUp(args[i].n, 4);
     sg.n_pad = sg.ns * 4;
     sg.row_u4 = sg.ns / 2;
+    const int group = EffectiveGroup(args[i].group, sg.ns);
+    if (sg.ns % group != 0 || group % 2 != 0) return hipErrorInvalidValue;  // whole groups of whole 16-byte items
+    sg.gu4 = group / 2;
+    sg.n_off = n_total;
+    n_total += sg.n_pad;
     total_row_u4 += sg.row_u4;
     weight_bytes += (size_t)p.ks * sg.ns * 8;
   }
   for (int i = count; i < kMaxSegments; ++i) p.seg[i] = p.seg[0];
+  p.n_total = n_total;
   p.batch_ids = a.batch_ids;
   p.rows = a.rows;
   p.src_rows = a.src_rows;
@@ -620,6 +891,11 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     return wide ? LaunchBatchedM<8, 8>(p, grouped, grid_b, stream) : LaunchBatchedM<4, 4>(p, grouped, grid_b, stream);
   }
 
+  if (StripKernelServes(args, count)) {
+    if (kernel_name) *kernel_name = "fc_w4_strip_kernel";
+    return LaunchStrip(p, args, count, grouped, stream);
+  }
+
   // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the
   // grid has at least ~one work-group per CU.  Narrow row segments (LPR = 8: 128 contiguous
   // bytes) keep K inside one work-group for wide layers; when the layer is too narrow for
@@ -627,19 +903,20 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   // Narrow layers of a few MB take narrower strips first (LPR = 4 or 2: 64- or 32-byte
   // segments): there a second kernel costs more than the poorer coalescing.
   // Very wide launches (the fused gate / up pair) fill the chip with 256-byte segments (LPR = 16).
+  const Tuning& tune = GetTuning();
   int lpr = 8, waves = 16;
   if (DivUp(total_row_u4, 16) >= 256)
     lpr = 16;
-  else if (DivUp(total_row_u4, 8) < 128 && weight_bytes <= (size_t)EnvInt("MLDHIP_GEMV_NARROW_MAX_MB", 4) << 20)
+  else if (DivUp(total_row_u4, 8) < 128 && weight_bytes <= (size_t)(tune.gemv_narrow_max_mb >= 0 ? tune.gemv_narrow_max_mb : 4) << 20)
     lpr = DivUp(total_row_u4, 4) >= 64 ? 4 : 2;
-  lpr = EnvInt("MLDHIP_GEMV_LPR", lpr);
+  if (tune.gemv_lpr > 0) lpr = tune.gemv_lpr;
   if (lpr != 2 && lpr != 4 && lpr != 8 && lpr != 16) lpr = 8;
   // two and more tokens need the registers of a small work-group (the 1024-thread shapes spill)
   if (p.m >= 2) {
     waves = 4;
     if (lpr == 16) lpr = 8;
   }
-  waves = EnvInt("MLDHIP_GEMV_WAVES", waves);
+  if (tune.gemv_waves > 0) waves = tune.gemv_waves;
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
   int strips = 0;
   for (int i = 0; i < count; ++i) {
@@ -667,7 +944,7 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     const int max_split = DivUp(p.chunks, rows);
     if (ksplit > max_split) ksplit = max_split;
   }
-  if (count == 1) ksplit = EnvInt("MLDHIP_GEMV_KSPLIT", ksplit);
+  if (count == 1 && tune.gemv_ksplit > 0) ksplit = tune.gemv_ksplit;
   if (ksplit > kGemvMaxKSplit) ksplit = kGemvMaxKSplit;
   if (ksplit < 1) ksplit = 1;
   while (ksplit > 1 && (size_t)ksplit * p.m * p.seg[0].n_pad > a.partial_floats) --ksplit;
@@ -681,9 +958,9 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   if (e != hipSuccess || p.ksplit == 1) return e;
   const int total = p.m * p.seg[0].n_pad;
   if (grouped)
-    hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.seg[0].n_pad);
   else
-    hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.seg[0].n_pad);
   return hipGetLastError();
 }
 
@@ -724,6 +1001,10 @@ hipError_t LaunchFcW4Gated(const FcArgs& gate, const FcArgs& up, int activation,
     sg.ns = DivUp(both[i]->n, 4);
     sg.n_pad = sg.ns * 4;
     sg.row_u4 = sg.ns / 2;
+    const int group = EffectiveGroup(both[i]->group, sg.ns);
+    if (sg.ns % group != 0 || group % 2 != 0 || group != EffectiveGroup(gate.group, sg.ns)) return hipErrorInvalidValue;
+    sg.gu4 = group / 2;
+    sg.n_off = 0;
     sg.strip_end = 0;
   }
   p.seg[2] = p.seg[0];

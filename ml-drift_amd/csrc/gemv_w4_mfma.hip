@@ -43,6 +43,7 @@ struct MsParams {
   const __half* bias;
   __half* dst;  // [Ns][m][4]
   int m, ks, ns;
+  int group;  // slices per output group of the packed weights (ns: one group)
   int steps_per_wave;
   uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
 };
@@ -72,7 +73,8 @@ __global__ __launch_bounds__(kMsWaves * 64) void fc_w4_mfma_stream_kernel(MsPara
   const int r = lane & 15, g = lane >> 4;
   const int slice0 = blockIdx.x * 16;
   const int slice = min(slice0 + r, p.ns - 1);  // clamp: loads stay in range, result unused
-  const uint32_t row_w = (uint32_t)p.ns * 8u;  // bytes per K-slice row of the weights
+  const uint32_t row_w = (uint32_t)p.group * 8u;  // bytes per K-slice row of the weights (of one output group)
+  const size_t col_w = ((size_t)(slice / p.group) * p.ks * p.group + slice % p.group) * 8;
   const uint32_t row_x = (uint32_t)p.m * 8u;
 
   int tok[FT];
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kMsWaves * 64) void fc_w4_mfma_stream_kernel(MsPara
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int ksc = min((s0 + u) * 8 + 2 * g + h, p.ks - 1);
-        w[u][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p.weights + (size_t)ksc * row_w + (size_t)slice * 8));
+        w[u][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p.weights + (size_t)ksc * row_w + col_w));
       }
     // keep the loads together and ahead of the arithmetic (the scheduler would otherwise sink
     // them next to their uses to save registers, a few at a time)
@@ -208,6 +210,8 @@ hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char*
   p.m = a.m;
   p.ks = DivUp(a.k, 4);
   p.ns = DivUp(a.n, 4);
+  p.group = EffectiveGroup(a.group, p.ns);
+  if (p.ns % p.group != 0) return hipErrorInvalidValue;
   p.steps_per_wave = DivUp(DivUp(p.ks, 8), kMsWaves);
   p.mask_lo = 0x000F000Fu;
   p.mask_hi = 0x00F000F0u;

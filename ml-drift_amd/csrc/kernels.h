@@ -10,6 +10,18 @@ namespace mldhip {
 
 inline int DivUp(int a, int b) { return (a + b - 1) / b; }
 
+// The I4O4 weights layout with output groups (WeightsDescription::output_group_size, in 4-channel
+// slices): [output group][K-slice][slice inside the group] blocks of 4 x 4 elements.  The
+// reference's FullyConnected uses one group (group = ns); groups of 16 slices make the share of
+// every 64-channel strip one contiguous run of K rows of 128 bytes.
+// Index of block (K-slice ks, output slice s); group = 0 stands for one group.
+__host__ __device__ inline size_t BlockIndex(int ks, int s, int ks_total, int ns, int group) {
+  const int g = group > 0 && group < ns ? group : ns;
+  return ((size_t)(s / g) * ks_total + ks) * g + s % g;
+}
+inline int EffectiveGroup(int group, int ns) { return group > 0 && group < ns ? group : ns; }
+constexpr int kNativeGroup = 16;  // slices per output group of the layout mldhip_fc_int4_weights_desc asks for
+
 enum ScaleKind { kScaleScalar = 0, kScaleLinear = 1, kScaleBlock = 2 };
 
 // One FullyConnected launch.  Tensors are slice-major: act [Ks][m][4], dst [Ns][m][4].
@@ -24,6 +36,7 @@ struct FcArgs {
   bool act_f16 = true;   // activations / scale / zero-point element type
   bool dst_f16 = true;   // output / bias element type
   int weight_bits = 4;
+  int group = 0;  // output group size of the packed weights in slices; 0 = one group (the reference's FC layout)
   int scale_kind = kScaleLinear;
   int groups = 1;
   float scalar_scale = 1.0f;
@@ -70,6 +83,7 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
 struct FcBatchRows {
   const int32_t* ids = nullptr;
   int rows = 1, src_rows = 1, weights_batch = 1;
+  int group = 0;  // output group size of the packed weights (plain launches only; 0 = one group)
 };
 
 // int8 activations x uint8/uint4 weights -> int32 (no scales).
@@ -81,6 +95,18 @@ bool FcInt8MathStreamSupported(int m, int k, int n, int weight_bits);
 hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int32_t* dst, int m, int k, int n,
                                   int weight_bits, hipStream_t stream, const char** kernel_name,
                                   const FcBatchRows& batch = FcBatchRows());
+
+// Process-wide overrides of the launch heuristics, set through mldhip_set_tuning (tests and
+// tuning runs); -1 = leave the choice to the heuristic.  Read at launch, never from the environment.
+struct Tuning {
+  int force_generic = -1;       // 1: every FullyConnected launch takes the unspecialised kernels
+  int gemv_mfma = -1;           // 1: one token also runs on the matrix-core GEMV
+  int gemv_fast = -1;           // 0: never take the contiguous-strip GEMV (grouped layout)
+  int gemv_lpr = -1, gemv_waves = -1, gemv_ksplit = -1, gemv_narrow_max_mb = -1;
+  int gemm_fm = -1, gemm_ksplit = -1, gemm_no_pair = -1, gemm_dual = -1, gemm_xcd_m = -1;
+  int gemm_i8_fm = -1;
+};
+Tuning& GetTuning();
 
 struct QuantArgs {
   const void* src = nullptr;

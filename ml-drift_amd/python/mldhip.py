@@ -32,6 +32,7 @@ SYMBOLS = [
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
+    "mldhip_fc_int4_weights_desc_reference", "mldhip_set_tuning",
 ]
 
 
@@ -102,6 +103,7 @@ def lib():
         _lib.mldhip_op_cost.argtypes = [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
         _lib.mldhip_op_destroy.argtypes = [C.c_void_p]
         _lib.mldhip_op_destroy.restype = None
+        _lib.mldhip_set_tuning.argtypes = [C.c_char_p, C.c_int]
     return _lib
 
 
@@ -125,10 +127,30 @@ def fc_int8_weights_desc(o, i):
     return d
 
 
-def fc_int4_weights_desc(o, i):
+def fc_int4_weights_desc(o, i, reference=False):
+    """The layout this library asks for (output groups of 16 slices where the shape allows), or with
+    `reference` the reference's own choice (one output group)."""
     d = WeightsDesc()
-    check(lib().mldhip_fc_int4_weights_desc(o, i, C.byref(d)))
+    fn = lib().mldhip_fc_int4_weights_desc_reference if reference else lib().mldhip_fc_int4_weights_desc
+    check(fn(o, i, C.byref(d)))
     return d
+
+
+class tuning:
+    """Context manager: overrides launch heuristics (mldhip_set_tuning) inside the block."""
+
+    def __init__(self, **knobs):
+        self.knobs = knobs
+
+    def __enter__(self):
+        for name, value in self.knobs.items():
+            check(lib().mldhip_set_tuning(name.encode(), int(value)))
+        return self
+
+    def __exit__(self, *exc):
+        for name in self.knobs:
+            check(lib().mldhip_set_tuning(name.encode(), -1))
+        return False
 
 
 def conv_int8_weights_desc(o, i):

@@ -57,10 +57,12 @@ def make_fc_case(seed, m, k, n, weight_bits, tensor_dtype, groups=1, with_bias=F
     return case
 
 
-def pack_fc_weights(case):
+def pack_fc_weights(case, reference_layout=False):
+    """Packs the case's weights for the FullyConnected op: in the layout the library asks for, or
+    with `reference_layout` in the reference's own FullyConnected layout (one output group)."""
     n, k = case["n"], case["k"]
     if case["weight_bits"] == 4:
-        desc = M.fc_int4_weights_desc(n, k)
+        desc = M.fc_int4_weights_desc(n, k, reference=reference_layout)
         return desc, M.rearrange_int8_as_uint4(case["w"], desc)
     desc = M.fc_int8_weights_desc(n, k)
     return desc, M.rearrange_int8_as_uint8(case["w"], desc)
@@ -73,14 +75,14 @@ def mld_type(np_dtype):
 class FcDevice:
     """An FC op with its device buffers (torch tensors) for one synthetic case."""
 
-    def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None):
+    def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None, reference_layout=False):
         import torch
         self.torch = torch
         self.case = case
         m, k, n = case["m"], case["k"], case["n"]
         td = case["tensor_dtype"]
         tt = torch.float16 if td == np.float16 else torch.float32
-        self.desc, packed = pack_fc_weights(case)
+        self.desc, packed = pack_fc_weights(case, reference_layout)
         self.packed_host = packed
         self.weights = torch.from_numpy(packed).to(device)
         self.act = torch.from_numpy(to_slices(case["act"]).astype(td)).to(device)
@@ -119,18 +121,6 @@ class FcDevice:
     def result(self):
         self.torch.cuda.synchronize()
         return from_slices(self.out.cpu().numpy().astype(np.float32), self.case["n"])
-
-
-def dequantized_weights(case):
-    """float64 [n][k] weights (q - zp) * s of a case (plain arithmetic, used for inputs of
-    chained layers and by tests as the textbook operand)."""
-    n, k, groups = case["n"], case["k"], case["groups"]
-    gs = k // groups
-    s = np.repeat(case["scale"].astype(np.float64), gs, axis=1)
-    q = case["w"].astype(np.float64)
-    if case["zero_point"] is not None:
-        q = q - np.repeat(case["zero_point"].astype(np.float64), gs, axis=1)
-    return q * s
 
 
 # The benchmark configurations 1-4 as make_fc_case arguments.

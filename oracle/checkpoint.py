@@ -139,8 +139,10 @@ def load_scale_or_zp(path, o, scale_i):
     return (raw.astype(np.float32) / np.float32(1024.0)).reshape(o, scale_i)
 
 
-def load_fc(directory, base, o, i, bits, tensor_dtype, swap_dims=False):
-    """-> dict(group_size, scale_i, weights, scale, zero_point, weights_sum_i): what the FC op binds."""
+def load_fc(directory, base, o, i, bits, tensor_dtype, swap_dims=False, output_group=None):
+    """-> dict(group_size, scale_i, weights, scale, zero_point, weights_sum_i): what the FC op binds.
+    `output_group`: output_group_size of the WeightsDescription the loader is handed (the reference
+    passes the FullyConnected's own description, llm_weights_loader.cc:29-71); default one group."""
     w_path = os.path.join(directory, base + ".weight")
     s_path = os.path.join(directory, base + ".weight_quantized_scale")
     z_path = os.path.join(directory, base + ".weight_quantized_zp")
@@ -149,7 +151,8 @@ def load_fc(directory, base, o, i, bits, tensor_dtype, swap_dims=False):
     ns = O.div_up(o, 4)
     if bits == 4:
         raw = _read_prefix(w_path, np.uint8, o * i // 2)
-        weights, sums = O.uint4_packed(raw, (o, 1, 1, i), O.LAYOUT_I4O4, ns, pad=8, swap_dims=swap_dims)
+        weights, sums = O.uint4_packed(raw, (o, 1, 1, i), O.LAYOUT_I4O4, output_group or ns, pad=8,
+                                       swap_dims=swap_dims)
     else:
         raw = _read_prefix(w_path, np.int8, o * i)
         q = raw.reshape(i, o).T if swap_dims else raw.reshape(o, i)

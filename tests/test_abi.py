@@ -29,8 +29,14 @@ def test_library_exports_every_declared_symbol():
 
 def test_fc_weights_desc_matches_reference_factories():
     # common/kernels/fully_connected.cc:1218-1246
-    d = M.fc_int4_weights_desc(14336, 4096)
+    d = M.fc_int4_weights_desc(14336, 4096, reference=True)
     assert (d.type, d.layout, d.output_group_size) == (M.UINT4, M.LAYOUT_I4O4, 3584)
+    # this device's choice: the same layout enum in output groups of 16 slices (whole 64-channel
+    # strips), one group where the channel count does not divide
+    d = M.fc_int4_weights_desc(14336, 4096)
+    assert (d.type, d.layout, d.output_group_size) == (M.UINT4, M.LAYOUT_I4O4, 16)
+    assert M.fc_int4_weights_desc(533, 171).output_group_size == 134
+    assert M.fc_int4_weights_desc(1032, 64).output_group_size == 258
     d = M.fc_int8_weights_desc(533, 171)
     assert (d.type, d.layout, d.output_group_size) == (M.UINT8, M.LAYOUT_I4O4, 134)
     assert M.packed_bytes(M.fc_int4_weights_desc(14336, 4096), 14336, 1, 1, 4096) == 29360128

@@ -111,13 +111,15 @@ def _make(tmp_path, o, i, bits, block, zp, fmt, swap, seed=0):
     (16, 64, 8, 0, False, "f32", False),
     (12, 72, 8, 0, True, "f32", True),
     (24, 128, 4, 64, False, "i8", False),
+    (128, 64, 4, 32, True, "f32", False),   # two output groups of 16 slices
+    (192, 96, 4, 0, False, "f32", True),
 ])
 @pytest.mark.parametrize("tensor_type", [M.FLOAT16, M.FLOAT32])
 def test_loader_matches_oracle(oracle, tmp_path, o, i, bits, block, zp, fmt, swap, tensor_type):
     d, q, s, z = _make(tmp_path, o, i, bits, block, zp, fmt, swap, seed=o + i)
     info = M.checkpoint_fc_probe(d, "layer.weight", "layer", o, i, bits)
     td = np.float16 if tensor_type == M.FLOAT16 else np.float32
-    ref = CK.load_fc(d, "layer", o, i, bits, td, swap_dims=swap)
+    ref = CK.load_fc(d, "layer", o, i, bits, td, swap_dims=swap, output_group=info.weights.output_group_size)
     assert info.group_size == ref["group_size"] == (block if block else i)
     assert info.scale_i == ref["scale_i"]
     assert bool(info.has_zero_point) == zp

@@ -21,7 +21,8 @@ def run_device(c, td, bias=None, max_tokens=None):
     mt = M.FLOAT16 if td == np.float16 else M.FLOAT32
     n, k, batch = c["n"], c["k"], c["batch"]
     ns = W.div_up(n, 4)
-    desc = (M.fc_int8_weights_desc if c["bits"] == 8 else M.fc_int4_weights_desc)(n, k)
+    # batched weights come in the reference's layout (one output group, the batch outermost)
+    desc = M.fc_int8_weights_desc(n, k) if c["bits"] == 8 else M.fc_int4_weights_desc(n, k, reference=True)
     packed = (M.rearrange_int8_as_uint8 if c["bits"] == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
     src2 = c["src"].reshape(c["src_rows"] * c["row_tokens"], k)
     act = torch.from_numpy(W.to_slices(src2).astype(td)).cuda()
@@ -189,7 +190,7 @@ def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, bat
     c = make_batch_ids_int8_case(rows + n + bits, rows, row_tokens, src_rows, k, n, batch, bits)
     print("batch ids int8", bits, rows, row_tokens, src_rows, k, n, batch, flush=True)
     ns = W.div_up(n, 4)
-    desc = (M.fc_int8_weights_desc if bits == 8 else M.fc_int4_weights_desc)(n, k)
+    desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
     packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
     act = torch.from_numpy(W.to_slices(c["src"].reshape(-1, k))).cuda()
     ids = torch.from_numpy(c["ids"]).cuda()

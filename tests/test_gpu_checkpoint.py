@@ -59,4 +59,4 @@ def test_fc_from_checkpoint_files(oracle, tmp_path, o, i, bits, block, zp, token
     ref = x.astype(np.float64) @ deq.T
     rms = np.sqrt(np.mean(ref ** 2))
     assert np.abs(got - ref).max() <= FP16_TOL * rms
-    assert op.kernel_name in ("fc_w4_stream_kernel", "fc_w4_mfma_gemm_kernel", "fc_w8_stream_kernel"), op.kernel_name
+    assert op.kernel_name in ("fc_w4_stream_kernel", "fc_w4_strip_kernel", "fc_w4_mfma_gemm_kernel", "fc_w8_stream_kernel"), op.kernel_name

@@ -12,8 +12,12 @@ pytestmark = pytest.mark.gpu
 
 import mldhip as M
 import workloads as W
+from refmath import textbook  # noqa: F401  (re-exported: the other GPU tests import it from here)
 
 FP16_TOL = 2e-2
+# The int4 GEMV kernels: the streaming kernel (any layout) and the contiguous-strip kernel, which
+# serves one token over weights packed in output groups of 16 slices.
+W4_GEMV = ("fc_w4_stream_kernel", "fc_w4_strip_kernel")
 
 
 def torch_cuda():
@@ -51,13 +55,6 @@ def oracle_fc(o, case, precision=None, use_kernel=True, wg_y=1):
     return o.from_slices(out, n)
 
 
-def textbook(case):
-    ref = case["act"].astype(np.float64) @ W.dequantized_weights(case).T
-    if case["bias"] is not None:
-        ref = ref + case["bias"]
-    return ref
-
-
 def check_fp(got, ref, case, label=""):
     err = np.abs(got.astype(np.float64) - ref).max()
     rms = np.sqrt(np.mean(ref.astype(np.float64) ** 2))
@@ -69,32 +66,40 @@ def check_fp(got, ref, case, label=""):
     return err / rms
 
 
-def run_case(oracle, case, expect_kernel=None, env=None):
+def native_layout_differs(case):
+    """True when the library asks for another int4 layout than the reference's (output groups)."""
+    if case["weight_bits"] != 4:
+        return False
+    a = M.fc_int4_weights_desc(case["n"], case["k"])
+    b = M.fc_int4_weights_desc(case["n"], case["k"], reference=True)
+    return a.output_group_size != b.output_group_size
+
+
+def run_case(oracle, case, expect_kernel=None, tune=None, layouts=None):
+    """Runs the case through the C-ABI and checks it against the textbook reference and the oracle's
+    restatement of the reference kernel.  int4 cases run in both weight layouts (the one the
+    library asks for and the reference's) where they differ; `tune` = tuning knobs for the run."""
     torch_cuda()
-    old = {}
-    for key, val in (env or {}).items():
-        old[key] = os.environ.get(key)
-        os.environ[key] = val
-    try:
-        print("case", {k: case[k] for k in ("m", "k", "n", "weight_bits", "groups")}, env, flush=True)
-        dev = W.FcDevice(case)
-        dev.run()
-        got = dev.result()
-        if expect_kernel:
-            assert dev.op.kernel_name == expect_kernel, dev.op.kernel_name
-        # a second launch must reproduce the first bit for bit
-        dev.run()
-        assert np.array_equal(got, dev.result())
-    finally:
-        for key, val in old.items():
-            if val is None:
-                os.environ.pop(key, None)
-            else:
-                os.environ[key] = val
-    ref_tb = textbook(case)
-    check_fp(got, ref_tb, case, "textbook")
-    if case["m"] * case["k"] * case["n"] <= 1 << 27:
-        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+    if layouts is None:
+        layouts = [False, True] if native_layout_differs(case) else [True]
+    got = None
+    for reference_layout in layouts:
+        print("case", {k: case[k] for k in ("m", "k", "n", "weight_bits", "groups")}, tune,
+              "reference layout" if reference_layout else "library layout", flush=True)
+        with M.tuning(**(tune or {})):
+            dev = W.FcDevice(case, reference_layout=reference_layout)
+            dev.run()
+            got = dev.result()
+            if expect_kernel:
+                names = (expect_kernel,) if isinstance(expect_kernel, str) else tuple(expect_kernel)
+                assert dev.op.kernel_name in names, dev.op.kernel_name
+            # a second launch must reproduce the first bit for bit
+            dev.run()
+            assert np.array_equal(got, dev.result())
+        ref_tb = textbook(case)
+        check_fp(got, ref_tb, case, "textbook")
+        if case["m"] * case["k"] * case["n"] <= 1 << 27:
+            check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
     return got
 
 
@@ -105,16 +110,15 @@ def test_config1_int8_fp32(oracle):
 
 def test_config2_int4_decode(oracle):
     case = W.make_fc_case(**W.CONFIGS["c2"])
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
-@pytest.mark.parametrize("lpr", ["8", "16"])
-@pytest.mark.parametrize("waves", ["4", "8", "16"])
-@pytest.mark.parametrize("ksplit", ["1", "3", "16"])
+@pytest.mark.parametrize("lpr", [8, 16])
+@pytest.mark.parametrize("waves", [4, 8, 16])
+@pytest.mark.parametrize("ksplit", [1, 3, 16])
 def test_stream_kernel_shapes(oracle, lpr, waves, ksplit):
     case = W.make_fc_case(seed=3, m=1, k=4096, n=1536, weight_bits=4, tensor_dtype=np.float16)
-    run_case(oracle, case, "fc_w4_stream_kernel",
-             {"MLDHIP_GEMV_LPR": lpr, "MLDHIP_GEMV_WAVES": waves, "MLDHIP_GEMV_KSPLIT": ksplit})
+    run_case(oracle, case, "fc_w4_stream_kernel", dict(gemv_lpr=lpr, gemv_waves=waves, gemv_ksplit=ksplit, gemv_fast=0))
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
@@ -123,7 +127,7 @@ def test_stream_kernel_variants_ragged(oracle, m, groups):
     # N = 8*129: the last 4-column block of the strip is partly outside the matrix
     case = W.make_fc_case(seed=17 + m, m=m, k=1024, n=1032, weight_bits=4, tensor_dtype=np.float16,
                           groups=groups, with_bias=True)
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
@@ -131,7 +135,7 @@ def test_stream_kernel_variants_ragged(oracle, m, groups):
 def test_stream_kernel_tokens_and_groups(oracle, m, groups):
     case = W.make_fc_case(seed=5 + m, m=m, k=2048, n=2048, weight_bits=4, tensor_dtype=np.float16,
                           groups=groups, with_bias=True)
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
 @pytest.mark.parametrize("m", [1, 3, 4])
@@ -140,7 +144,7 @@ def test_stream_kernel_zero_points(oracle, m, groups):
     """Asymmetric int4 weights (a zero-point tensor shaped like the scales) on the streaming kernel."""
     case = W.make_fc_case(seed=23 + m, m=m, k=2048, n=1032, weight_bits=4, tensor_dtype=np.float16,
                           groups=groups, with_bias=True, with_zero_point=True)
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
@@ -157,13 +161,13 @@ def test_w8_stream_kernel(oracle, dtype, m, k, n, groups, zp):
 @pytest.mark.parametrize("name,k,n", W.C5_LAYER)
 def test_config5_decode_layer_shapes(oracle, name, k, n):
     case = W.make_fc_case(seed=7, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=k // 32)
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
 def test_stream_kernel_ragged(oracle):
     # K not a multiple of 32 (partial chunk), N = 8*odd (partial strip)
     case = W.make_fc_case(seed=11, m=2, k=1000, n=1032, weight_bits=4, tensor_dtype=np.float16)
-    run_case(oracle, case, "fc_w4_stream_kernel")
+    run_case(oracle, case, W4_GEMV)
 
 
 @pytest.mark.parametrize("bits", [4, 8])
@@ -181,7 +185,7 @@ def test_generic_kernel_reference_test_shapes(oracle, bits, dtype, kind):
         fast = bits == 4 and dtype == np.float16 and kind == "linear"
         expect = "fc_generic_kernel"
         if fast:  # symmetric fp16 int4: streaming GEMV up to 4 tokens, MFMA GEMM beyond
-            expect = "fc_w4_stream_kernel" if m <= 4 else "fc_w4_mfma_gemm_kernel"
+            expect = W4_GEMV if m <= 4 else "fc_w4_mfma_gemm_kernel"
         if bits == 8 and kind == "linear" and m <= 4:  # per-channel int8, either tensor type
             expect = "fc_w8_stream_kernel"
         if bits == 8 and kind == "linear" and m > 4 and dtype == np.float16:
@@ -271,8 +275,10 @@ def test_int8_math_bit_exact(oracle, bits, m, k, n):
     # 1..4 tokens stream (uint4 rows with an odd number of slices keep the tiled kernel)
     streams = m <= 4 and (bits == 8 or ((n + 3) // 4) % 2 == 0)
     assert op.kernel_name == ("fc_i8math_stream_kernel" if streams else "fc_int8_math_kernel"), op.kernel_name
-    if m * k * n <= 1 << 24:
-        mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed, m, k, n, bits), n)
+    if m * k * n <= 1 << 24:  # the restatement reads the reference's layout
+        ns = (n + 3) // 4
+        packed_ref = (oracle.int8_as_uint4 if bits == 4 else oracle.int8_as_uint8)(w, oracle.LAYOUT_I4O4, ns)
+        mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed_ref, m, k, n, bits), n)
         assert np.array_equal(got, mimic)
 
 

@@ -17,15 +17,25 @@ from test_gpu_fc import check_fp, oracle_fc, textbook
 FP16_TOL = 2e-2
 
 
-def run_w4(case):
-    print("w%d gemm" % case["weight_bits"], {k: case[k] for k in ("m", "k", "n", "groups")}, flush=True)
-    dev = W.FcDevice(case)
-    dev.run()
-    got = dev.result()
-    assert dev.op.kernel_name == "fc_w%d_mfma_gemm_kernel" % case["weight_bits"], dev.op.kernel_name
-    dev.run()
-    assert np.array_equal(got, dev.result())
-    return got
+def run_w4(case, reference_layout=None):
+    """Runs the case on the matrix-core GEMM.  int4 cases whose library layout (output groups of 16
+    slices) differs from the reference's run in both, and the two results must agree bit for bit:
+    the layout moves the blocks in memory, not the order of the arithmetic."""
+    print("w%d gemm" % case["weight_bits"], {k: case[k] for k in ("m", "k", "n", "groups")}, reference_layout, flush=True)
+    from test_gpu_fc import native_layout_differs
+    layouts = [reference_layout] if reference_layout is not None else ([False, True] if native_layout_differs(case) else [True])
+    results = []
+    for ref_layout in layouts:
+        dev = W.FcDevice(case, reference_layout=ref_layout)
+        dev.run()
+        got = dev.result()
+        assert dev.op.kernel_name == "fc_w%d_mfma_gemm_kernel" % case["weight_bits"], dev.op.kernel_name
+        dev.run()
+        assert np.array_equal(got, dev.result())
+        results.append(got)
+    if len(results) == 2:
+        assert np.array_equal(results[0], results[1]), "the two weight layouts give different sums"
+    return results[0]
 
 
 @pytest.mark.parametrize("m,k,n,groups", [(16, 256, 128, 8), (5, 64, 8, 1), (128, 2048, 2048, 64),
@@ -106,15 +116,15 @@ def test_gemm_fractional_zero_points(oracle, bits, m, k, n, groups):
                                                   (8, 128, 1024, 640, 8, True),
                                                   (4, 4096, 64, 2048, 2, True),    # 128-token tile
                                                   (8, 2050, 96, 1100, 1, False)])
-def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp, monkeypatch):
+def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp):
     """The two-tile mode (half of a work-group's waves per channel tile), forced on shapes of test
     size: odd tile counts, ragged edges, zero points, both weight types, both token tiles; and
     the same bytes as the one-tile mode where the K shares coincide is not required - the bar is
     the FullyConnected one."""
-    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "1")
     case = W.make_fc_case(seed=m + n + bits, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
                           with_bias=True, with_zero_point=zp)
-    got = run_w4(case)
+    with M.tuning(gemm_dual=1):
+        got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
     small = min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
@@ -122,7 +132,7 @@ def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp, monkey
         check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
 
 
-def test_gemm_modes_random_sweep(monkeypatch):
+def test_gemm_modes_random_sweep():
     """Seeded sweep over shapes with the two-tile mode forced on and off and every token tile
     forced in turn: all against the textbook reference at the fp16 bar."""
     rng = np.random.default_rng(31)
@@ -136,15 +146,14 @@ def test_gemm_modes_random_sweep(monkeypatch):
         if k % gs == 0 and rng.random() < 0.6:
             groups = k // gs
         zp = bool(rng.random() < 0.4)
-        monkeypatch.setenv("MLDHIP_GEMM_DUAL", str(it % 2))
-        monkeypatch.setenv("MLDHIP_GEMM_FM", str([1, 2, 4][it % 3]))
         case = W.make_fc_case(seed=900 + it, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
                               with_bias=bool(it % 2), with_zero_point=zp)
-        got = run_w4(case)
+        with M.tuning(gemm_dual=it % 2, gemm_fm=[1, 2, 4][it % 3]):
+            got = run_w4(case, reference_layout=bool((it // 6) % 2))
         check_fp(got, textbook(case), case, "sweep %d" % it)
 
 
-def test_gemm_two_tiles_fused_launch(monkeypatch):
+def test_gemm_two_tiles_fused_launch():
     """Three matrices in one two-tile launch: pairs of tiles that straddle two matrices (3 + 1 + 2
     channel tiles) against the single one-tile launches."""
     import torch
@@ -156,14 +165,14 @@ def test_gemm_two_tiles_fused_launch(monkeypatch):
     devs = [W.FcDevice(c) for c in cases]
     for d in devs[1:]:
         d.op.set_src(0, devs[0].act)
-    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "0")
     single = []
-    for d in devs:
-        d.run()
-        single.append(d.result())
-        d.out.zero_()
-    monkeypatch.setenv("MLDHIP_GEMM_DUAL", "1")
-    M.fc_launch_fused([d.op for d in devs], torch.cuda.current_stream().cuda_stream)
+    with M.tuning(gemm_dual=0):
+        for d in devs:
+            d.run()
+            single.append(d.result())
+            d.out.zero_()
+    with M.tuning(gemm_dual=1):
+        M.fc_launch_fused([d.op for d in devs], torch.cuda.current_stream().cuda_stream)
     for d, c, ref in zip(devs, cases, single):
         got = d.result()
         check_fp(got, textbook(c), c, "two-tile fused")

@@ -32,7 +32,7 @@ def test_stack_parity(stack, tokens):
             check_fp(got, refs[idx], stack.case(idx), "layer %d %s" % (layer, case["name"]))
             first[(layer, idx)] = got
     names = set(stack.kernel_names())
-    assert names <= {"fc_w4_stream_kernel", "fc_w4_mfma_gemm_kernel"}, names
+    assert names <= {"fc_w4_stream_kernel", "fc_w4_strip_kernel", "fc_w4_mfma_gemm_kernel"}, names
     stack.launch()
     for (layer, idx), got in first.items():
         assert np.array_equal(got, stack.result(layer, idx))
