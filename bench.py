@@ -45,6 +45,7 @@ def parse():
     p.add_argument("--layout", default="library", choices=["library", "reference"],
                    help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
                         "slices) or in the reference's own FullyConnected layout (one output group)")
+    p.add_argument("--tune", default="", help="tuning knobs for the run, e.g. gemv_ksplit=1,gemm_dual=0 (mldhip_set_tuning)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
     p.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -318,6 +319,9 @@ def main():
         print("no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    for item in filter(None, args.tune.split(",")):
+        name, value = item.split("=")
+        M.check(M.lib().mldhip_set_tuning(name.encode(), int(value)))
     if args.workload != "c2":
         run_other(args, torch, M, W)
         return

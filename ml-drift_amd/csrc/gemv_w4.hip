@@ -756,10 +756,14 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
     strips += p.seg[i].ns / kNativeGroup;
     p.seg[i].strip_end = strips;
   }
-  // K stays inside the work-group when the strips alone fill the chip; else it is split into
-  // power-of-two runs of at least 8 chunks (one wave) so that about 256 work-groups exist.
+  // K stays inside the work-group when the strips alone fill the chip, and for matrices of a few
+  // MB, where a second kernel for the sums costs more (2.8 us) than running on the 30-40 CUs that
+  // the strips give; else it is split into power-of-two runs of at least 8 chunks (one wave) so
+  // that about 256 work-groups exist.
+  size_t weight_bytes = 0;
+  for (int i = 0; i < count; ++i) weight_bytes += (size_t)p.ks * p.seg[i].ns * 8;
   int cps = p.chunks;
-  if (strips < 128 && p.chunks > 8) {
+  if (strips < 128 && p.chunks > 8 && weight_bytes > ((size_t)6 << 20)) {
     const int want = DivUp(256, strips);
     cps = 8;
     while (cps * 2 * want <= p.chunks) cps *= 2;
