@@ -388,6 +388,24 @@ enum { MLDHIP_GATE_GELU_TANH = 1, MLDHIP_GATE_SILU = 2 };
 int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void* dst,
                            size_t dst_bytes, void* stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it): the int4 decode
+ * FullyConnected of mldhip_op_launch (fp16 tensors, 1..4 tokens, symmetric uint4 weights,
+ * per-channel scales or scale groups of whole multiples of 32 input channels, optional bias)
+ * without an op object: the buffers are passed directly and the split-K sums, which an op keeps in
+ * the workspace that its create call allocates, go to an array of 2 MiB that the library holds
+ * statically on every GPU it runs on (until the process ends).  Calls no hipMalloc / hipFree.
+ * Same kernels and same results as mldhip_op_launch on an op of the same description.
+ * Limits: o <= 65536 (MLDHIP_OUT_OF_RANGE beyond), an even number of 4-channel slices,
+ * output_group_size = ceil(o/4) or 16 as mldhip_fc_create takes it.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (different streams) race; calls on
+ * one stream are ordered.  The array needs no clearing between calls.
+ *   src [ceil(i/4)][tokens][4] halfs, weights packed uint4, weights_scale [scale_groups][ceil(o/4)][4]
+ *   halfs, biases ceil(o/4)*4 halfs or null, dst [ceil(o/4)][tokens][4] halfs. */
+int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const void* weights_scale,
+                                  const void* biases, void* dst, int o, int i, int scale_groups,
+                                  int output_group_size, int tokens, void* stream);
+
 /* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
  * at the current shape (GPUOperation::flops_/read_size_/write_size_,
  * common/task/gpu_operation.h:190-195). */

@@ -786,6 +786,45 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
   return MLDHIP_OK;
 }
 
+int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const void* weights_scale, const void* biases,
+                                  void* dst, int o, int i, int scale_groups, int output_group_size, int tokens,
+                                  void* stream_ptr) {
+  if (!src || !weights || !weights_scale || !dst) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  if (o <= 0 || i <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "weights shape must be positive");
+  if (o > kNoAllocMaxChannels)
+    return Fail(MLDHIP_OUT_OF_RANGE, "more output channels than the static scratch array serves (65536)");
+  if (tokens < 1 || tokens > kGemvMaxTokens)
+    return Fail(MLDHIP_OUT_OF_RANGE, "the allocation-free entry point serves 1..4 tokens");
+  const int ns = DivUp(o, 4), ks = DivUp(i, 4);
+  if (ns % 2 != 0) return Fail(MLDHIP_UNIMPLEMENTED, "an odd number of 4-channel output slices is not served here");
+  if (scale_groups < 1 || ks % scale_groups != 0 || (scale_groups > 1 && (ks / scale_groups) % 8 != 0))
+    return Fail(MLDHIP_INVALID_ARGUMENT, "scale groups must be whole multiples of 32 input channels");
+  const bool native = output_group_size == kNativeGroup && o % 4 == 0 && ns % kNativeGroup == 0;
+  if (output_group_size != ns && !native)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
+  const void* ptrs[5] = {src, weights, weights_scale, biases, dst};
+  for (const void* ptr : ptrs)
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return Fail(MLDHIP_INVALID_ARGUMENT, "a buffer is not 16-byte aligned");
+  FcArgs a;
+  a.act = src;
+  a.weights = static_cast<const uint8_t*>(weights);
+  a.scale = weights_scale;
+  a.bias = biases;
+  a.dst = dst;
+  a.m = tokens;
+  a.k = i;
+  a.n = o;
+  a.act_f16 = a.dst_f16 = true;
+  a.weight_bits = 4;
+  a.group = output_group_size;
+  a.scale_kind = scale_groups == 1 ? kScaleLinear : kScaleBlock;
+  a.groups = scale_groups;
+  const char* name = nullptr;
+  hipError_t e = LaunchFcW4StreamNoAlloc(a, static_cast<hipStream_t>(stream_ptr), &name);
+  if (e != hipSuccess) return HipFail(e, "allocation-free launch");
+  return MLDHIP_OK;
+}
+
 const char* mldhip_op_kernel_name(const mldhip_op* op) { return op ? op->last_kernel : ""; }
 
 int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {

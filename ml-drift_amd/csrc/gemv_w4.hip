@@ -1023,4 +1023,35 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
   return LaunchFcW4StreamFused(&a, 1, stream, kernel_name);
 }
 
+// ------------------------------------------------------------------------------------------
+// The streaming GEMV for callers that cannot allocate: its split-K sums go to a statically
+// allocated array instead of an op's workspace.  Every GPU the library runs on holds its own
+// copy of the array (at its own address) until the process ends.  The array's name is only a
+// host-side handle: the device address comes from hipGetSymbolAddress, once per device, and that
+// pointer is what the kernels get, as they get the workspace pointer of an op.
+// ------------------------------------------------------------------------------------------
+namespace {
+static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+hipError_t LaunchFcW4StreamNoAlloc(FcArgs a, hipStream_t stream, const char** kernel_name) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return e;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  if (g_scratch_ptr[device] == nullptr) {  // first call on this device, which is current
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    g_scratch_ptr[device] = ptr;
+  }
+  // Nothing has to start at zero: a split launch writes every sum that its second kernel reads.
+  a.partial = g_scratch_ptr[device];
+  a.partial_floats = kNoAllocScratchFloats;
+  if (!FcW4StreamSupported(a)) return hipErrorInvalidValue;
+  return LaunchFcW4StreamFused(&a, 1, stream, kernel_name);
+}
+
 }  // namespace mldhip

@@ -64,6 +64,12 @@ hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** ke
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);
 
+// The same launch with the split-K sums in the library's statically allocated scratch array
+// (kNoAllocScratchFloats floats per device) instead of a.partial: allocates nothing.
+constexpr size_t kNoAllocScratchFloats = (size_t)512 * 1024;  // 2 MiB
+constexpr int kNoAllocMaxChannels = 65536;                    // leaves room for an 8-way K split
+hipError_t LaunchFcW4StreamNoAlloc(FcArgs a, hipStream_t stream, const char** kernel_name);
+
 // dst = activation(gate(x)) * up(x) for a pair of int4 layers of one shape on the streaming GEMV
 // (1..2 tokens).
 bool FcW4GatedSupported(const FcArgs& gate, const FcArgs& up);

@@ -32,7 +32,7 @@ SYMBOLS = [
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
-    "mldhip_fc_int4_weights_desc_reference", "mldhip_set_tuning",
+    "mldhip_fc_int4_weights_desc_reference", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
 ]
 
 
@@ -104,6 +104,7 @@ def lib():
         _lib.mldhip_op_destroy.argtypes = [C.c_void_p]
         _lib.mldhip_op_destroy.restype = None
         _lib.mldhip_set_tuning.argtypes = [C.c_char_p, C.c_int]
+        _lib.mldhip_fc_int4_decode_noalloc.argtypes = [C.c_void_p] * 5 + [C.c_int] * 5 + [C.c_void_p]
     return _lib
 
 
@@ -404,3 +405,10 @@ def conv_int8_create(dst_type, o, i, weights_desc, has_zero_point=False, has_bia
     h = C.c_void_p()
     check(lib().mldhip_conv_int8_create(C.byref(d), C.byref(h)))
     return Op(h)
+
+
+def fc_int4_decode_noalloc(src, weights, scale, bias, dst, o, i, scale_groups, output_group_size, tokens, stream=0):
+    """mldhip_fc_int4_decode_noalloc over torch tensors (or None for `bias`)."""
+    ptr = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    check(lib().mldhip_fc_int4_decode_noalloc(ptr(src), ptr(weights), ptr(scale), ptr(bias), ptr(dst), o, i,
+                                              scale_groups, output_group_size, tokens, C.c_void_p(stream)))
