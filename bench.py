@@ -8,9 +8,9 @@ Infinity Cache if one buffer were reused, so the steps rotate over a ring of wei
 larger than that cache, the way the reference's own perf harness does behind
 kUseMultipleWeights (cl/testing/perf_util.cc:2247-2253).
 
-Prints ONE JSON line.  The timed region is R back-to-back replays of a HIP graph that holds the
-steps (inputs resident in HBM; R such that the region lasts at least 5 ms, so that the replay's
-own host cost does not weigh on a 20-step run).  `value` is algorithmic bytes / (wall time of
+Prints ONE JSON line.  The timed region is one replay of a HIP graph that holds R x steps launches
+(inputs resident in HBM; R such that the region lasts at least 25 ms, so that the replay's own host
+cost does not weigh on a 20-step run); it is timed 5 times and the median region is reported.  `value` is algorithmic bytes / (wall time of
 the region / launches in it); `roofline.achieved` divides the same bytes by the average launch
 duration measured with HIP events on the launch stream over the same region.
 """
@@ -60,58 +60,71 @@ def parse():
     return a
 
 
-MIN_REGION_MS = 5.0  # the timed region is at least this long, whatever --steps says
+# The timed region is at least this long, whatever --steps says.  (Long enough for the host side
+# too: on this stack a stream synchronisation that waits between about 5 and 8 ms returns after
+# 8 ms, which would inflate a 5 ms region by half; at 25 ms wall clock and HIP events agree to 0.3 %.)
+MIN_REGION_MS = 25.0
+REGIONS = 5          # the region is timed this many times; the median one is reported
 
 
 def time_graph(torch, stream, launch_step, steps, warmup, use_graph=True, ring=1):
-    """`warmup` eager steps, then a graph of `steps` steps (rounded up to a whole number of turns of the
-    weight ring, so that replay after replay every weight copy comes back only after all the others).  A single replay of a short graph is
-    dominated by the replay's own host and synchronisation cost (tens of microseconds), so the
-    timed region is R back-to-back replays, R chosen from one untimed replay such that the region
-    lasts at least MIN_REGION_MS.  Returns (wall seconds per step, event microseconds per step, {R, steps per replay}):
-    both are region / (R * steps), the wall clock bracketed by synchronisations, the HIP events
-    recorded on `stream` around the same replays."""
+    """`warmup` eager steps, then the timed region: ONE replay of a HIP graph that holds the steps.
+    A replay of a short graph is dominated by its own host and synchronisation cost (tens of
+    microseconds, and back-to-back replays of one graph do not overlap: each waits for the one
+    before and leaves the GPU idle while it is submitted), so the graph holds R * steps launches,
+    R chosen from an untimed replay of a `steps`-launch graph such that the region lasts at least
+    MIN_REGION_MS (rounded up to whole turns of the weight ring, so that every weight copy comes
+    back only after all the others).  The region is timed REGIONS times and the median one is
+    reported.  Returns (wall seconds per step, event microseconds per step, {R, launches}): both
+    are region / launches in it, the wall clock bracketed by synchronisations, the HIP events
+    recorded on `stream` around the same replay."""
     s = stream.cuda_stream
-    steps = -(-steps // ring) * ring
+
+    def build(launches):
+        if not use_graph:
+            def run():
+                for i in range(launches):
+                    launch_step(s, i)
+            return run
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            cs = torch.cuda.current_stream().cuda_stream
+            for i in range(launches):
+                launch_step(cs, i)
+        return graph.replay
+
+    def timed(run):
+        ev0 = torch.cuda.Event(enable_timing=True)
+        ev1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(stream)
+        run()
+        ev1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, ev0.elapsed_time(ev1)
+
     with torch.cuda.stream(stream):
         for i in range(warmup):
             launch_step(s, i)
         stream.synchronize()
-        graph = None
-        if use_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                cs = torch.cuda.current_stream().cuda_stream
-                for i in range(steps):
-                    launch_step(cs, i)
-
-            def replay():
-                graph.replay()
-        else:
-            def replay():
-                for i in range(steps):
-                    launch_step(s, i)
-        replay()  # untimed: the first replay uploads the graph
+        launches = -(-steps // ring) * ring
+        run = build(launches)
+        run()  # untimed: the first replay uploads the graph
         stream.synchronize()
-        ev0 = torch.cuda.Event(enable_timing=True)
-        ev1 = torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        replay()
-        ev1.record(stream)
-        stream.synchronize()
-        one_ms = max(ev0.elapsed_time(ev1), 1e-3)
-        replays = max(1, min(20000, int(np.ceil(MIN_REGION_MS / one_ms))))
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        ev0.record(stream)
-        for _ in range(replays):
-            replay()
-        ev1.record(stream)
-        stream.synchronize()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-    n = replays * steps
-    return wall / n, ev0.elapsed_time(ev1) * 1e3 / n, {"graph_replays": replays, "launches_per_replay": steps}
+        _, one_ms = timed(run)
+        reps = max(1, min(5000, int(np.ceil(MIN_REGION_MS / max(one_ms, 1e-3)))))
+        if reps > 1:
+            launches = reps * launches
+            run = build(launches)
+            run()
+            stream.synchronize()
+        regions = [timed(run) for _ in range(REGIONS)]
+    # the median region: a host hiccup of a millisecond (seen on shared boxes) drops out
+    wall, event_ms = sorted(regions)[REGIONS // 2]
+    return wall / launches, event_ms * 1e3 / launches, {"steps_multiple": reps, "launches_in_region": launches,
+                                                         "timed_regions": REGIONS, "reported_region": "median by wall time"}
 
 
 def run_other(args, torch, M, W):
@@ -403,7 +416,8 @@ def main():
         "config": {"workload": "c2: FullyConnected decode GEMV M=1 K=4096 N=14336 int4 per-channel, fp16 act/out",
                    "weights_layout": "kOSpatialIOGroupI4O4, output_group_size %d" % devs[0].desc.output_group_size,
                    "weight_ring": args.ring, "timed_region": "hipGraph replays" if use_graph else "eager launch loop",
-                   "graph_replays": reg["graph_replays"], "launches_per_replay": reg["launches_per_replay"],
+                   "steps_multiple": reg["steps_multiple"], "launches_in_region": reg["launches_in_region"],
+                   "timed_regions": reg["timed_regions"], "reported_region": reg["reported_region"],
                    "algorithmic_bytes_per_step": algo_bytes, "flops_per_step": flops,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,

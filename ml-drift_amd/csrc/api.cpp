@@ -134,9 +134,14 @@ static int FcDesc(int o, int i, int type, bool native_groups, mldhip_weights_des
   desc->type = type;
   desc->layout = MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4;
   const int ns = DivUp(o, 4);
-  // uint4 weights of whole 64-channel strips: output groups of 16 slices, so that the K rows of a
-  // strip lie one after the other in memory
-  desc->output_group_size = (native_groups && o % 4 == 0 && ns % kNativeGroup == 0) ? kNativeGroup : ns;
+  // uint4 weights: output groups of 16, 8 or 4 slices, so that the K rows of a strip of channels
+  // lie one after the other in memory
+  desc->output_group_size = ns;
+  if (native_groups) {
+    desc->output_group_size = NativeGroupFor(o);
+    const int forced = GetTuning().fc_group;
+    if (forced > 0 && o % 4 == 0 && ns % forced == 0 && (IsNativeGroup(forced) || forced == ns)) desc->output_group_size = forced;
+  }
   return MLDHIP_OK;
 }
 
@@ -155,6 +160,7 @@ int mldhip_set_tuning(const char* name, int value) {
   Tuning& t = GetTuning();
   const struct { const char* name; int* field; } knobs[] = {
       {"force_generic", &t.force_generic}, {"gemv_mfma", &t.gemv_mfma}, {"gemv_fast", &t.gemv_fast},
+      {"fc_group", &t.fc_group},
       {"gemv_lpr", &t.gemv_lpr}, {"gemv_waves", &t.gemv_waves}, {"gemv_ksplit", &t.gemv_ksplit},
       {"gemv_narrow_max_mb", &t.gemv_narrow_max_mb}, {"gemm_fm", &t.gemm_fm}, {"gemm_ksplit", &t.gemm_ksplit},
       {"gemm_no_pair", &t.gemm_no_pair}, {"gemm_dual", &t.gemm_dual}, {"gemm_xcd_m", &t.gemm_xcd_m},
@@ -363,8 +369,8 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   }
   {
     const int ns = DivUp(d->o, 4);
-    const bool native = wd.type == MLDHIP_UINT4 && wd.output_group_size == kNativeGroup && d->o % 4 == 0 &&
-                        ns % kNativeGroup == 0 && !batch_ids;
+    const bool native = wd.type == MLDHIP_UINT4 && IsNativeGroup(wd.output_group_size) && d->o % 4 == 0 &&
+                        ns % wd.output_group_size == 0 && !batch_ids;
     if (wd.output_group_size != ns && !native)
       return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
   }
@@ -799,7 +805,7 @@ int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const vo
   if (ns % 2 != 0) return Fail(MLDHIP_UNIMPLEMENTED, "an odd number of 4-channel output slices is not served here");
   if (scale_groups < 1 || ks % scale_groups != 0 || (scale_groups > 1 && (ks / scale_groups) % 8 != 0))
     return Fail(MLDHIP_INVALID_ARGUMENT, "scale groups must be whole multiples of 32 input channels");
-  const bool native = output_group_size == kNativeGroup && o % 4 == 0 && ns % kNativeGroup == 0;
+  const bool native = IsNativeGroup(output_group_size) && o % 4 == 0 && ns % output_group_size == 0;
   if (output_group_size != ns && !native)
     return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
   const void* ptrs[5] = {src, weights, weights_scale, biases, dst};

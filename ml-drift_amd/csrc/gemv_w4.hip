@@ -576,8 +576,11 @@ hipError_t LaunchBatchedM(const StreamParams& p, bool grouped, dim3 grid, hipStr
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x2s __attribute__((ext_vector_type(2)));
 
-// Sum over the 8 rows of a wave of the 8 channel sums of every lane; the result of channel
-// (lane % 8) * 8 + lane / 8 is returned in this lane.  All 64 lanes must be active.
+// LPR lanes (16 bytes each) cover a row; a wave holds 64 / LPR rows.  Sum over the rows of a wave
+// of the 8 channel sums of every lane; the result of channel (lane % LPR) * 8 + (lane / 8) % 8 is
+// returned in this lane (lanes that differ only in the bits between LPR and 8 hold the same
+// sums).  All 64 lanes must be active.
+template <int LPR>
 __device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
   float s4[4], s2[2];
 #pragma unroll
@@ -593,7 +596,11 @@ __device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
 #pragma unroll
   for (int i = 0; i < 2; ++i)
     s2[i] += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s2[i]), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
-  return (lane & 8) ? s2[1] : s2[0];
+  float v = (lane & 8) ? s2[1] : s2[0];
+  // narrower rows: the lanes 4 (and 2) apart hold further rows of the same channels
+  if (LPR <= 4) v += __shfl_xor(v, 4, 64);
+  if (LPR <= 2) v += __shfl_xor(v, 2, 64);
+  return v;
 }
 
 // Launch parameters of the strip kernel: what a single-matrix launch reads sits in the first
@@ -618,16 +625,16 @@ struct StripParams {
   StripSegment seg[kMaxSegments];
 };
 
-template <int WAVES, bool GROUPED, bool ZP, bool MULTI>
+template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) {
-  constexpr int ROWS = WAVES * 8;  // chunks of 8 K-slices the work-group covers per pass
-  constexpr int STRIP = 64;
+  constexpr int ROWS = WAVES * 64 / LPR;  // chunks of 8 K-slices the work-group covers per pass
+  constexpr int STRIP = LPR * 8;          // channels of a strip (one output group of the layout)
   __shared__ float red[WAVES][STRIP];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int col = lane & 7;
-  const int row = tid >> 3;
+  const int col = lane % LPR;
+  const int row = tid / LPR;
   int si = 0, strip = blockIdx.x;
   if (MULTI && p.segments > 1 && strip >= p.seg[0].strip_end) {
     si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
@@ -650,28 +657,25 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
   // the output this thread finishes: channel `ch` of the strip (the channel the wave sum leaves in
   // this lane when the work-group is one wave, else thread order)
-  const int ch = WAVES == 1 ? (lane & 7) * 8 + (lane >> 3) : (tid & 63);
+  const int ch_wave = col * 8 + ((lane >> 3) & 7);  // the channel whose wave sum this lane holds
+  const int ch = WAVES == 1 ? ch_wave : (tid % STRIP);
   const int n_out = strip * STRIP + ch;
   const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(sg.bias ? sg.bias : sg.scale);
-  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(scale)[n_out];
-  const unsigned short out_bias_raw = bias_src[n_out];
 
   float acc[8];
 #pragma unroll
   for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
   u32x4 zv = {0u, 0u, 0u, 0u};
-  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * STRIP + col * 8);
-  // row r of the strip: 8 uint4; chunk c: 64 uint4
-  const u32x4* wstrip = weights + (size_t)strip * ks * 8 + col;
-  for (int c = c_begin + row; c < c_end; c += ROWS) {
-    const u32x4* wp = wstrip + (size_t)c * 64;
-    u32x4 w[8], a4[4];
-    // The small loads first (activations and scales come from cache), then the eight weight loads
-    // back to back; the fence keeps the arithmetic behind all of them, so that the waits count the
-    // weight loads down one by one instead of some of them being issued after the first wait.
+  // row r of the strip: LPR uint4; chunk c: 8 rows
+  const u32x4* wstrip = weights + (size_t)strip * ks * LPR + col;
+  // Loads of one chunk, in the order the memory pipeline returns them (loads return in order): the
+  // small ones that come from cache first (activations, group scales), then the eight weight loads
+  // back to back.
+  u32x4 w[8], a4[4], sv;
+  auto issue = [&](int c) {
+    const u32x4* wp = wstrip + (size_t)c * (8 * LPR);
 #pragma unroll
     for (int j = 0; j < 4; ++j) a4[j] = astrip[c * 4 + j];
-    u32x4 sv;
     if (GROUPED) {
       const int g = c / group_chunks;
       const size_t so = (size_t)g * n_pad + (size_t)strip * STRIP + col * 8;
@@ -679,8 +683,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
       if (ZP) zv = *reinterpret_cast<const u32x4*>(zero_point + so);
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + j * 8);
-    __builtin_amdgcn_sched_barrier(0);
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + j * LPR);
+  };
+  auto consume = [&]() {
     u32x2 a[8][1];
 #pragma unroll
     for (int j = 0; j < 8; ++j) a[j][0] = u32x2{a4[j >> 1][2 * (j & 1)], a4[j >> 1][2 * (j & 1) + 1]};
@@ -700,10 +705,30 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
         acc[o] += centered;
       }
     }
+  };
+  // First chunk (the only one in the launch shapes that give every thread one chunk).  The scale
+  // and bias of the output this thread finishes are fetched behind its weight loads: in front of
+  // them, their trip to memory would hold back the use of every weight that arrives before they do.
+  int c = c_begin + row;
+  const bool first = c < c_end;
+  if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * STRIP + col * 8);
+  if (first) issue(c);
+  const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(scale)[n_out];
+  const unsigned short out_bias_raw = bias_src[n_out];
+  // the fence keeps the arithmetic behind all the loads, so that the waits count the weight loads
+  // down one by one instead of some of them being issued after the first wait
+  __builtin_amdgcn_sched_barrier(0);
+  if (first) {
+    consume();
+    for (c += ROWS; c < c_end; c += ROWS) {
+      issue(c);
+      __builtin_amdgcn_sched_barrier(0);
+      consume();
+    }
   }
-  float v = WaveStripSum(acc, lane);
+  float v = WaveStripSum<LPR>(acc, lane);
   if (WAVES > 1) {
-    red[wave][(lane & 7) * 8 + (lane >> 3)] = v;
+    red[wave][ch_wave] = v;  // (lanes that hold the same channel write the same value)
     __syncthreads();
     if (tid >= STRIP) return;
     v = 0.0f;
@@ -720,11 +745,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   }
 }
 
-template <int WAVES>
+template <int LPR, int WAVES>
 hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
   const dim3 block(WAVES * 64);
-#define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<WAVES, G, Z, MU>), grid, block, 0, stream, p)
+#define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
     if (zp) { if (multi) MLD_STRIP(true, true, true); else MLD_STRIP(true, true, false); }
     else    { if (multi) MLD_STRIP(true, false, true); else MLD_STRIP(true, false, false); }
@@ -736,24 +761,39 @@ hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream
   return hipGetLastError();
 }
 
+template <int LPR>
+hipError_t LaunchStripL(const StripParams& p, int waves, bool grouped, dim3 grid, hipStream_t stream) {
+  switch (waves) {
+    case 1: return LaunchStripW<LPR, 1>(p, grouped, grid, stream);
+    case 2: return LaunchStripW<LPR, 2>(p, grouped, grid, stream);
+    case 4: return LaunchStripW<LPR, 4>(p, grouped, grid, stream);
+    case 8: return LaunchStripW<LPR, 8>(p, grouped, grid, stream);
+    default: return LaunchStripW<LPR, 16>(p, grouped, grid, stream);
+  }
+}
+
 // The contiguous-strip kernel serves: one token, every matrix of the launch packed in output
-// groups of 16 slices, K a multiple of 32 channels (whole chunks).
+// groups of the same size (16, 8 or 4 slices), K a multiple of 32 channels (whole chunks).
 bool StripKernelServes(const FcArgs* args, int count) {
   if (GetTuning().gemv_fast == 0) return false;
   if (args[0].m != 1 || args[0].batch_ids != nullptr) return false;
   if (DivUp(args[0].k, 4) % 8 != 0 || args[0].k % 4 != 0) return false;
+  const int group = EffectiveGroup(args[0].group, DivUp(args[0].n, 4));
+  if (!IsNativeGroup(group)) return false;
   for (int i = 0; i < count; ++i) {
     const int ns = DivUp(args[i].n, 4);
-    if (args[i].n % 4 != 0 || ns % kNativeGroup != 0 || EffectiveGroup(args[i].group, ns) != kNativeGroup) return false;
+    if (args[i].n % 4 != 0 || ns % group != 0 || EffectiveGroup(args[i].group, ns) != group) return false;
   }
   return true;
 }
 
 hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grouped, hipStream_t stream) {
   const Tuning& tune = GetTuning();
+  const int group = EffectiveGroup(args[0].group, p.seg[0].ns);  // 16, 8 or 4 slices: 8, 4 or 2 lanes per row
+  const int lpr = group / 2;
   int strips = 0;
   for (int i = 0; i < count; ++i) {
-    strips += p.seg[i].ns / kNativeGroup;
+    strips += p.seg[i].ns / group;
     p.seg[i].strip_end = strips;
   }
   // K stays inside the work-group when the strips alone fill the chip, and for matrices of a few
@@ -763,9 +803,9 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   size_t weight_bytes = 0;
   for (int i = 0; i < count; ++i) weight_bytes += (size_t)p.ks * p.seg[i].ns * 8;
   int cps = p.chunks;
-  if (strips < 128 && p.chunks > 8 && weight_bytes > ((size_t)6 << 20)) {
+  if (strips < 128 && p.chunks > 64 / lpr && weight_bytes > ((size_t)6 << 20)) {
     const int want = DivUp(256, strips);
-    cps = 8;
+    cps = 64 / lpr;
     while (cps * 2 * want <= p.chunks) cps *= 2;
   }
   if (tune.gemv_ksplit > 0) cps = std::max(1, DivUp(p.chunks, tune.gemv_ksplit));
@@ -783,7 +823,7 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   p.chunks_per_split = cps;
   p.ksplit = ksplit;
   int waves = 1;
-  while (waves < 16 && waves * 8 < cps) waves *= 2;
+  while (waves < 16 && waves * 64 / lpr < cps) waves *= 2;
   if (tune.gemv_waves > 0) waves = tune.gemv_waves;
   const dim3 grid(strips, ksplit);
   StripParams sp;
@@ -806,12 +846,10 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
     sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, g.strip_end, g.n_off, 0};
   }
   hipError_t e;
-  switch (waves) {
-    case 1: e = LaunchStripW<1>(sp, grouped, grid, stream); break;
-    case 2: e = LaunchStripW<2>(sp, grouped, grid, stream); break;
-    case 4: e = LaunchStripW<4>(sp, grouped, grid, stream); break;
-    case 8: e = LaunchStripW<8>(sp, grouped, grid, stream); break;
-    default: e = LaunchStripW<16>(sp, grouped, grid, stream); break;
+  switch (lpr) {
+    case 2: e = LaunchStripL<2>(sp, waves, grouped, grid, stream); break;
+    case 4: e = LaunchStripL<4>(sp, waves, grouped, grid, stream); break;
+    default: e = LaunchStripL<8>(sp, waves, grouped, grid, stream); break;
   }
   if (e != hipSuccess || ksplit == 1) return e;
   const int total = p.m * p.n_total;

@@ -20,7 +20,15 @@ __host__ __device__ inline size_t BlockIndex(int ks, int s, int ks_total, int ns
   return ((size_t)(s / g) * ks_total + ks) * g + s % g;
 }
 inline int EffectiveGroup(int group, int ns) { return group > 0 && group < ns ? group : ns; }
-constexpr int kNativeGroup = 16;  // slices per output group of the layout mldhip_fc_int4_weights_desc asks for
+// Output group size (slices) of the layout mldhip_fc_int4_weights_desc asks for: 16 (64-channel
+// strips, 128-byte rows).  The kernels also read groups of 8 and 4 slices (narrower strips, more of
+// them), which measured slower on every layer width tried (the rows fall below a cache line).
+constexpr int kNativeGroup = 16;
+inline bool IsNativeGroup(int group) { return group == 4 || group == 8 || group == 16; }
+inline int NativeGroupFor(int o) {
+  const int ns = DivUp(o, 4);
+  return (o % 4 == 0 && ns % kNativeGroup == 0) ? kNativeGroup : ns;
+}
 
 enum ScaleKind { kScaleScalar = 0, kScaleLinear = 1, kScaleBlock = 2 };
 
@@ -108,6 +116,7 @@ struct Tuning {
   int force_generic = -1;       // 1: every FullyConnected launch takes the unspecialised kernels
   int gemv_mfma = -1;           // 1: one token also runs on the matrix-core GEMV
   int gemv_fast = -1;           // 0: never take the contiguous-strip GEMV (grouped layout)
+  int fc_group = -1;            // output group size that mldhip_fc_int4_weights_desc returns where it divides the slices
   int gemv_lpr = -1, gemv_waves = -1, gemv_ksplit = -1, gemv_narrow_max_mb = -1;
   int gemm_fm = -1, gemm_ksplit = -1, gemm_no_pair = -1, gemm_dual = -1, gemm_xcd_m = -1;
   int gemm_i8_fm = -1;

@@ -85,6 +85,14 @@ def lib():
             raise ImportError(
                 "libmldhip.so is not built (expected at %s); run `make -C ml-drift_amd/csrc` or "
                 "__graft_entry__.build()" % LIB_PATH)
+        # torch, where it is installed, is the device allocator of the tests and the bench, and it
+        # ships a HIP runtime of its own: it has to be in the process first, so that this library
+        # binds to the same runtime (loaded the other way round, launches from here fail with
+        # "no ROCm-capable device is detected").
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _lib = C.CDLL(LIB_PATH)
         _lib.mldhip_last_error.restype = C.c_char_p
         _lib.mldhip_version.restype = C.c_char_p

@@ -31,12 +31,19 @@ def test_fc_weights_desc_matches_reference_factories():
     # common/kernels/fully_connected.cc:1218-1246
     d = M.fc_int4_weights_desc(14336, 4096, reference=True)
     assert (d.type, d.layout, d.output_group_size) == (M.UINT4, M.LAYOUT_I4O4, 3584)
-    # this device's choice: the same layout enum in output groups of 16 slices (whole 64-channel
-    # strips), one group where the channel count does not divide
+    # this device's choice: the same layout enum in output groups of 16 slices (64-channel strips),
+    # one group where the channel count does not divide; groups of 8 and 4 slices are read as well
     d = M.fc_int4_weights_desc(14336, 4096)
     assert (d.type, d.layout, d.output_group_size) == (M.UINT4, M.LAYOUT_I4O4, 16)
+    assert M.fc_int4_weights_desc(256, 2048).output_group_size == 16
     assert M.fc_int4_weights_desc(533, 171).output_group_size == 134
     assert M.fc_int4_weights_desc(1032, 64).output_group_size == 258
+    with M.tuning(fc_group=4):
+        assert M.fc_int4_weights_desc(2048, 16384).output_group_size == 4
+        assert M.fc_int4_weights_desc(1032, 64).output_group_size == 258  # 258 slices do not divide
+    for g in (4, 8, 16):
+        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 128, 64, M.make_desc(M.UINT4, M.LAYOUT_I4O4, g),
+                    scale_shape=(128, 1))
     d = M.fc_int8_weights_desc(533, 171)
     assert (d.type, d.layout, d.output_group_size) == (M.UINT8, M.LAYOUT_I4O4, 134)
     assert M.packed_bytes(M.fc_int4_weights_desc(14336, 4096), 14336, 1, 1, 4096) == 29360128

@@ -416,3 +416,18 @@ def test_random_shapes_sweep(oracle):
         check_fp(got, textbook(case), case, "sweep %d (%s)" % (it, dev.op.kernel_name))
     print("kernels exercised:", seen)
     assert len(seen) >= 4
+
+
+@pytest.mark.parametrize("group", [4, 8, 16])
+@pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 64, False, True), (16384, 2048, 512, False, False),
+                                               (4096, 1536, 1, True, True), (512, 256, 1, False, False),
+                                               (2048, 16384, 64, True, False), (96, 64, 3, False, True)])
+def test_strip_kernel_group_sizes(oracle, group, k, n, groups, zp, bias):
+    """One token on the contiguous-strip kernel over weights packed in output groups of 4, 8 and 16
+    slices: K inside the work-group and split across work-groups, per-channel and group-wise scales,
+    zero points, a single chunk per wave row and several."""
+    case = W.make_fc_case(seed=k + n + group, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    with M.tuning(fc_group=group):
+        assert M.fc_int4_weights_desc(n, k).output_group_size == group
+        run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
