@@ -745,6 +745,35 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   }
 }
 
+// Second pass of a K-split strip launch: one 64-thread work-group per 64 channels, numbered like
+// the strips of the first pass.  Work-groups go round-robin to the 8 XCDs, so with a strip count
+// that is a multiple of 8 the sums of a strip are added on the XCD whose L2 they were written
+// through.  Added in split order (fixed), up to 8 sums in flight at a time.
+template <bool GROUPED>
+__global__ __launch_bounds__(64) void fc_w4_strip_reduce_kernel(StripParams p) {
+  const int nt = blockIdx.x * 64 + threadIdx.x;
+  if (nt >= p.n_total) return;
+  int si = 0;
+  if (p.segments > 1 && nt >= p.seg[1].n_off) si = (p.segments > 2 && nt >= p.seg[2].n_off) ? 2 : 1;
+  const StripSegment& sg = p.seg[si];
+  const int n = nt - sg.n_off;
+  const unsigned short* bias_src = reinterpret_cast<const unsigned short*>(sg.bias ? sg.bias : sg.scale);
+  const unsigned short scale_raw = reinterpret_cast<const unsigned short*>(sg.scale)[n];
+  const unsigned short bias_raw = bias_src[n];
+  float v = 0.0f;
+  for (int s0 = 0; s0 < p.ksplit; s0 += 8) {
+    float part[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) part[j] = p.partial[(size_t)min(s0 + j, p.ksplit - 1) * p.n_total + nt];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v += s0 + j < p.ksplit ? part[j] : 0.0f;
+  }
+  if (!GROUPED) v *= __half2float(__ushort_as_half(scale_raw));
+  __half h = __float2half_rn(v);
+  if (sg.bias) h = __hadd(h, __ushort_as_half(bias_raw));
+  sg.dst[n] = h;
+}
+
 template <int LPR, int WAVES>
 hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
@@ -852,11 +881,10 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
     default: e = LaunchStripL<8>(sp, waves, grouped, grid, stream); break;
   }
   if (e != hipSuccess || ksplit == 1) return e;
-  const int total = p.m * p.n_total;
   if (grouped)
-    hipLaunchKernelGGL(fc_w4_reduce_kernel<true>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.n_total);
+    hipLaunchKernelGGL(fc_w4_strip_reduce_kernel<true>, dim3(DivUp(p.n_total, 64)), dim3(64), 0, stream, sp);
   else
-    hipLaunchKernelGGL(fc_w4_reduce_kernel<false>, dim3(DivUp(total, 256)), dim3(256), 0, stream, p, p.n_total);
+    hipLaunchKernelGGL(fc_w4_strip_reduce_kernel<false>, dim3(DivUp(p.n_total, 64)), dim3(64), 0, stream, sp);
   return hipGetLastError();
 }
 

@@ -431,3 +431,29 @@ def test_strip_kernel_group_sizes(oracle, group, k, n, groups, zp, bias):
     with M.tuning(fc_group=group):
         assert M.fc_int4_weights_desc(n, k).output_group_size == group
         run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
+
+
+@pytest.mark.parametrize("bits,k,n,groups", [(4, 4096, 2048, 1), (4, 1024, 1032, 32), (8, 2048, 2048, 1), (4, 171, 533, 1)])
+@pytest.mark.parametrize("b,w", [(2, 4), (2, 1), (10, 3)])
+def test_fc_tensor_batch(oracle, bits, k, n, groups, b, w):
+    """Activation tensors with batch > 1 (the reference's big tests use B in {2, 10, 20},
+    fully_connected_test_util.cc:935-1001): the token index of the buffer layout is
+    (y*W + x)*B + b, so BHWC(b, 1, w, k) is b*w tokens; the result must be that of the same
+    tokens given as BHWC(1, 1, b*w, k), bit for bit, and meet the FullyConnected bar."""
+    import torch
+    m = b * w
+    case = W.make_fc_case(seed=b + w + n, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True)
+    print("fc batch", bits, k, n, groups, b, w, flush=True)
+    dev = W.FcDevice(case)
+    dev.op.set_shape(1, 1, m)
+    dev.run()
+    flat = dev.result()
+    dev.out.zero_()
+    dev.op.set_shape(b, 1, w)
+    dev.run()
+    batched = dev.result()
+    assert np.array_equal(flat, batched)
+    check_fp(batched, textbook(case), case, "textbook")
+    if m * k * n <= 1 << 27:
+        check_fp(batched, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")

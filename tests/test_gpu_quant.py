@@ -95,3 +95,14 @@ def test_batched_seed_element(oracle):
     rcodes, rparams = oracle.quantize(src, tokens, channels, oracle.PACKED_INT8C4, False, False, batch=batch)
     assert np.array_equal(params.view(np.uint32), rparams.view(np.uint32))
     assert np.array_equal(codes, rcodes)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_symmetric_literal_tie_vector_on_gpu(dtype):
+    """The hand-worked half-up case of tests/test_oracle_quant.py, on the GPU: absmax 127 gives
+    scale 1, and 0.5 -> 1, -0.5 -> 0, 1.5 -> 2, -1.5 -> -1."""
+    from test_oracle_quant import LITERAL_TIE_CODES, LITERAL_TIE_ROW
+    src = W.to_slices(LITERAL_TIE_ROW[None]).astype(dtype)
+    codes, params = run_quant(src, 1, 8, M.PACKED_INT8C4, True, True)
+    assert params[0, 0] == 1.0 and params[0, 1] == 0.0 and params[0, 2] == LITERAL_TIE_CODES.sum()
+    assert np.array_equal(W.from_slices(codes, 8).astype(np.int32)[0], LITERAL_TIE_CODES)

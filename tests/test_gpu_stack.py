@@ -114,3 +114,46 @@ def test_graph_replays_match_eager():
             # eager work between replays
             st.launch()
             torch.cuda.synchronize()
+
+
+@pytest.mark.timeout(900)
+def test_stack_chain_18_layers_decode():
+    """The whole 18-layer stack at one token with the values flowing through it: every FC has its
+    own weights (seed layer * 7 + index) and reads the re-normalised output of the FC before it in
+    the layer's graph (q, k, v read the layer input; o reads q's output; gate and up read o's; down
+    reads gate's; the next layer reads down's), N(0,1) after re-normalisation as the synthetic
+    inputs are.  Each FC goes through the C-ABI on the kernel the bench uses and is held to the
+    FullyConnected bar against float64 arithmetic over its dequantised weights."""
+    import torch
+    rng = np.random.default_rng(1234)
+    x = rng.standard_normal(2048).astype(np.float16).astype(np.float32)
+
+    def renorm(v):
+        v = v.astype(np.float64)
+        return ((v - v.mean()) / v.std()).astype(np.float16).astype(np.float32)
+
+    def reference(case):
+        q = case["w"].astype(np.float32)
+        gs = case["k"] // case["groups"]
+        prod = (q * case["act"][0][None, :]).reshape(case["n"], case["groups"], gs).sum(axis=2, dtype=np.float64)
+        return (prod * case["scale"].astype(np.float64)).sum(axis=1)[None, :]
+
+    worst = 0.0
+    for layer in range(W.C5_LAYERS):
+        outs = {}
+        for idx, (name, k, n) in enumerate(W.C5_LAYER):
+            src = {"q": x, "k": x, "v": x, "o": outs.get("q"), "gate": outs.get("o"), "up": outs.get("o"),
+                   "down": outs.get("gate")}[name]
+            case = W.make_fc_case(seed=layer * 7 + idx, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16,
+                                  groups=k // 32)
+            case["act"] = src[None, :].astype(np.float32)
+            dev = W.FcDevice(case)
+            dev.run()
+            got = dev.result()
+            assert dev.op.kernel_name == "fc_w4_strip_kernel", dev.op.kernel_name
+            worst = max(worst, check_fp(got, reference(case), case, "layer %d %s" % (layer, name)))
+            outs[name] = renorm(got[0])
+            del dev
+        x = outs["down"]
+        print("layer", layer, "worst so far", worst, flush=True)
+    torch.cuda.synchronize()

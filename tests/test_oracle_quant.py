@@ -174,3 +174,26 @@ def test_dequantize_algebra(oracle, with_zp):
     w_deq = w.astype(np.float64) * ws[:, None] + (0 if wzp is None else wzp[:, None])
     ref = a_deq @ w_deq.T
     assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+
+
+LITERAL_TIE_ROW = np.array([127.0, 0.5, -0.5, 1.5, -1.5, 2.4, -2.6, -127.0], np.float32)
+# absmax 127 -> inv_scale = scale = 1 exactly, so code = floor(x + 128.5) - 128: ties go up
+# (0.5 -> 1, -0.5 -> 0, 1.5 -> 2, -1.5 -> -1), 2.4 -> 2, -2.6 -> -3.  Worked by hand from
+# common/kernels/quantize_and_dequantize.cc:363-377, 423-429; round-to-nearest-even would give
+# 0, 0, 2, -2 for the four ties.
+LITERAL_TIE_CODES = np.array([127, 1, 0, 2, -1, 2, -3, -127], np.int32)
+
+
+@pytest.mark.parametrize("f16", [True, False])
+def test_symmetric_literal_tie_vector(oracle, f16):
+    o = oracle
+    src = o.to_slices(LITERAL_TIE_ROW[None])
+    src = o.f32_to_f16_bits(src) if f16 else src
+    codes, params = o.quantize(src, 1, 8, o.PACKED_INT8C4, symmetric=True, calculate_sum=True)
+    assert params[0, 0] == 1.0 and params[0, 1] == 0.0
+    assert np.array_equal(o.from_slices(codes, 8).astype(np.int32)[0], LITERAL_TIE_CODES)
+    assert params[0, 2] == LITERAL_TIE_CODES.sum()
+    # unsigned codes: the same + 128, offset -128 * inv_scale
+    codes_u, params_u = o.quantize(src, 1, 8, o.PACKED_UINT8C4, symmetric=True)
+    assert np.array_equal(o.from_slices(codes_u, 8).astype(np.int32)[0], LITERAL_TIE_CODES + 128)
+    assert params_u[0, 0] == 1.0 and params_u[0, 1] == -128.0
