@@ -268,7 +268,7 @@ def run_other(args, torch, M, W):
     else:
         from decoder_stack import DecoderStack
         tokens = 1 if args.workload == "c5-decode" else max(5, args.tokens)
-        st = DecoderStack(max_tokens=max(128, tokens))
+        st = DecoderStack(max_tokens=max(128, tokens), keep_host=False)
         st.set_tokens(tokens)
         wall, us, reg = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
         wb, fl = st.weight_bytes(), st.flops(tokens)

@@ -4,9 +4,11 @@ it per layer (samples/llm/gemma3_model_builder.cc:1115-1128): q, k, v, o, gate, 
 
 Only the FCs are reproduced (no attention, norm or activation): every FC reads a synthetic
 N(0,1) activation tensor of its input width and writes its own output tensor, and the FCs run
-in the graph's order on one stream, i.e. with the dependencies of the real layer.  Every
-layer owns its device copy of the packed weights and scales, so a decode step streams the
-whole stack's 1.1 GB through HBM.
+in the graph's order on one stream, i.e. with the dependencies of the real layer.  Every FC of
+every layer has weights and scales of its own (seed layer * 7 + index), so a decode step streams
+the whole stack's 1.1 GB through HBM.  (What a GEMV or GEMM costs does not depend on the values of
+its activations, so the synthetic inputs time like the fed-forward ones; the chain with the values
+flowing through it is a parity test.)
 
 Nothing here computes a result on the host.
 """
@@ -17,47 +19,48 @@ import workloads as W
 
 
 class DecoderStack:
-    def __init__(self, layers=W.C5_LAYERS, max_tokens=128, seed=5, layer_shapes=None, device="cuda"):
+    def __init__(self, layers=W.C5_LAYERS, max_tokens=128, seed=5, layer_shapes=None, device="cuda", keep_host=True):
         import torch
         self.torch = torch
         self.layers = layers
         self.max_tokens = max_tokens
         self.shapes = list(layer_shapes or W.C5_LAYER)
         self.device = device
-        # host-side cases of one layer (all layers hold the same values in distinct memory)
-        self.cases = []
-        for idx, (name, k, n) in enumerate(self.shapes):
-            case = W.make_fc_case(seed=seed * 100 + idx, m=max_tokens, k=k, n=n, weight_bits=4,
-                                  tensor_dtype=np.float16, groups=k // 32)
-            case["name"] = name
-            self.cases.append(case)
-        # one activation tensor per input width, shared by the FCs that read that width
+        # host-side cases: every FC of every layer has weights and scales of its own, seed
+        # layer * 7 + index; the FCs of one input width share one synthetic N(0,1) activation tensor
         self.inputs = {}
-        for case in self.cases:
-            k = case["k"]
+        rng = np.random.default_rng(seed)
+        for _, k, _ in self.shapes:
             if k not in self.inputs:
-                self.inputs[k] = case["act"]
-        for case in self.cases:
-            case["act"] = self.inputs[case["k"]]
+                self.inputs[k] = W.round_to(rng.standard_normal((max_tokens, k)), np.float16)
+        self.keep_host = keep_host
+        self.layer_cases = []
         self.tokens = None
         self.src = {}
-        self.nodes = []  # (layer, case index, op, out tensor)
-        packed = []
-        for case in self.cases:
-            desc, w = W.pack_fc_weights(case)
-            sc = M.scale_to_tensor(case["scale"], M.FLOAT16).view(np.float16)
-            packed.append((desc, torch.from_numpy(w), torch.from_numpy(sc)))
+        self.nodes = []  # (layer, case index, op, out tensor, weights, scales)
         self._weights = []
         for layer in range(layers):
-            for idx, case in enumerate(self.cases):
-                desc, w_host, s_host = packed[idx]
-                w_dev = w_host.to(device)
-                s_dev = s_host.to(device)
-                out = torch.zeros((W.div_up(case["n"], 4), max_tokens, 4), dtype=torch.float16, device=device)
-                op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, case["n"], case["k"], desc,
-                                 scale_shape=(case["n"], case["groups"]), max_tokens=max_tokens)
+            cases = []
+            for idx, (name, k, n) in enumerate(self.shapes):
+                case = W.make_fc_case(seed=layer * 7 + idx, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16,
+                                      groups=k // 32)
+                case["name"] = name
+                case["m"] = max_tokens
+                case["act"] = self.inputs[k]
+                desc, w = W.pack_fc_weights(case)
+                sc = M.scale_to_tensor(case["scale"], M.FLOAT16).view(np.float16)
+                w_dev = torch.from_numpy(w).to(device)
+                s_dev = torch.from_numpy(sc).to(device)
+                out = torch.zeros((W.div_up(n, 4), max_tokens, 4), dtype=torch.float16, device=device)
+                op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, n, k, desc,
+                                 scale_shape=(n, case["groups"]), max_tokens=max_tokens)
                 self._weights.append((w_dev, s_dev))
                 self.nodes.append((layer, idx, op, out, w_dev, s_dev))
+                if not keep_host:  # the bench needs the shapes only
+                    case = dict(case, w=None, scale=None)
+                cases.append(case)
+            self.layer_cases.append(cases)
+        self.cases = self.layer_cases[0]
         self.set_tokens(1)
 
     def weight_bytes(self):
@@ -121,7 +124,7 @@ class DecoderStack:
         (On MI355X the fork/join of the branches costs more than the overlap gains: 1093 us
         against 873 us for a decode step, hence the default.)"""
         torch = self.torch
-        self.launch(fused=False)  # workspaces are allocated on the first launch, outside the capture
+        self.launch(fused=False)  # warm-up
         torch.cuda.synchronize()
         main = torch.cuda.Stream()
         side = [torch.cuda.Stream(), torch.cuda.Stream()]
@@ -159,10 +162,10 @@ class DecoderStack:
         pos = layer * len(self.cases) + idx
         return W.from_slices(self.outs[pos].cpu().numpy().astype(np.float32), self.cases[idx]["n"])
 
-    def case(self, idx, tokens=None):
-        """The host-side case of FC `idx` restricted to the current token count."""
+    def case(self, idx, tokens=None, layer=0):
+        """The host-side case of FC `idx` of `layer` restricted to the current token count."""
         t = self.tokens if tokens is None else tokens
-        c = dict(self.cases[idx])
+        c = dict(self.layer_cases[layer][idx])
         c["m"] = t
         c["act"] = c["act"][:t]
         return c

@@ -24,12 +24,12 @@ def test_stack_parity(stack, tokens):
     print("decoder stack, tokens =", tokens, flush=True)
     stack.set_tokens(tokens)
     stack.launch()
-    refs = [textbook(stack.case(idx)) for idx in range(len(stack.cases))]
     first = {}
     for layer in range(LAYERS):
         for idx, case in enumerate(stack.cases):
             got = stack.result(layer, idx)
-            check_fp(got, refs[idx], stack.case(idx), "layer %d %s" % (layer, case["name"]))
+            ref = textbook(stack.case(idx, layer=layer))
+            check_fp(got, ref, stack.case(idx, layer=layer), "layer %d %s" % (layer, case["name"]))
             first[(layer, idx)] = got
     names = set(stack.kernel_names())
     assert names <= {"fc_w4_stream_kernel", "fc_w4_strip_kernel", "fc_w4_mfma_gemm_kernel"}, names
@@ -72,13 +72,13 @@ def test_fused_launch_matches_single_launches(stack):
         for out in stack.outs:
             out.zero_()
         stack.launch(fused=True)
-        refs = [textbook(stack.case(idx)) for idx in range(len(stack.cases))]
         pos = 0
         for layer in range(LAYERS):
             for idx, case in enumerate(stack.cases):
                 got = stack.result(layer, idx)
-                check_fp(got, refs[idx], stack.case(idx), "fused layer %d %s" % (layer, case["name"]))
-                rms = np.sqrt(np.mean(refs[idx] ** 2))
+                ref = textbook(stack.case(idx, layer=layer))
+                check_fp(got, ref, stack.case(idx, layer=layer), "fused layer %d %s" % (layer, case["name"]))
+                rms = np.sqrt(np.mean(ref ** 2))
                 worst = np.abs(got - single[pos]).max()
                 print("tokens", tokens, case["name"], "fused vs single max|diff|/rms = %.2e" % (worst / rms), flush=True)
                 assert worst <= 2e-3 * rms
