@@ -406,6 +406,13 @@ int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const vo
                                   const void* biases, void* dst, int o, int i, int scale_groups,
                                   int output_group_size, int tokens, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the two floors that a memory-bound launch is
+ * read against on a given box.  kind 0: an empty launch (224 work-groups of 1024 threads);
+ * kind 1: a plain streaming read of `bytes` of `src` (whole multiples of 128 KB; 16-byte loads,
+ * one contiguous 128 KB run per work-group, nothing kept).  `sink`: at least 4 KB of device memory
+ * (never written in practice).  bench.py --workload floors times both the way it times the ops. */
+int mldhip_probe_launch(int kind, const void* src, size_t bytes, void* sink, void* stream);
+
 /* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
  * at the current shape (GPUOperation::flops_/read_size_/write_size_,
  * common/task/gpu_operation.h:190-195). */

@@ -831,6 +831,13 @@ int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const vo
   return MLDHIP_OK;
 }
 
+int mldhip_probe_launch(int kind, const void* src, size_t bytes, void* sink, void* stream_ptr) {
+  if (!sink || (kind == 1 && !src)) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
+  hipError_t e = LaunchProbe(kind, src, bytes, sink, static_cast<hipStream_t>(stream_ptr));
+  if (e != hipSuccess) return HipFail(e, "probe launch");
+  return MLDHIP_OK;
+}
+
 const char* mldhip_op_kernel_name(const mldhip_op* op) { return op ? op->last_kernel : ""; }
 
 int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {

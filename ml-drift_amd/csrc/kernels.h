@@ -123,6 +123,10 @@ struct Tuning {
 };
 Tuning& GetTuning();
 
+// Measurement aids (mldhip_probe_launch): kind 0 = an empty launch of 224 x 1024 threads, kind 1 = a
+// plain streaming read of `bytes` (whole multiples of 128 KB are read).
+hipError_t LaunchProbe(int kind, const void* src, size_t bytes, void* sink, hipStream_t stream);
+
 struct QuantArgs {
   const void* src = nullptr;
   void* codes = nullptr;

@@ -33,6 +33,7 @@ SYMBOLS = [
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
     "mldhip_fc_int4_weights_desc_reference", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
+    "mldhip_probe_launch",
 ]
 
 
@@ -113,6 +114,7 @@ def lib():
         _lib.mldhip_op_destroy.restype = None
         _lib.mldhip_set_tuning.argtypes = [C.c_char_p, C.c_int]
         _lib.mldhip_fc_int4_decode_noalloc.argtypes = [C.c_void_p] * 5 + [C.c_int] * 5 + [C.c_void_p]
+        _lib.mldhip_probe_launch.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     return _lib
 
 
@@ -420,3 +422,10 @@ def fc_int4_decode_noalloc(src, weights, scale, bias, dst, o, i, scale_groups, o
     ptr = lambda t: None if t is None else C.c_void_p(t.data_ptr())
     check(lib().mldhip_fc_int4_decode_noalloc(ptr(src), ptr(weights), ptr(scale), ptr(bias), ptr(dst), o, i,
                                               scale_groups, output_group_size, tokens, C.c_void_p(stream)))
+
+
+def probe_launch(kind, src, sink, stream=0):
+    """mldhip_probe_launch over torch tensors: kind 0 = empty launch, 1 = streaming read of `src`."""
+    nbytes = 0 if src is None else src.numel() * src.element_size()
+    check(lib().mldhip_probe_launch(kind, None if src is None else C.c_void_p(src.data_ptr()), nbytes,
+                                    C.c_void_p(sink.data_ptr()), C.c_void_p(stream)))
