@@ -248,6 +248,7 @@ int mldhip_fc_is_recommended(int precision, int tokens);
  *   2 "weights_scale"         present iff scale_o*scale_i > 1
  *   3 "weights_zero_point"    present iff has_zero_point_tensor
  *   4 "biases"                present iff has_bias, ceil(o/4)*4 values of dst_type
+ *   5 "params"                present iff a runtime channel bound is set (int32, see below)
  * (absent objects do not take an index).  dst 0 "dst_tensor": [ceil(o/4)][tokens][4].
  *
  * Zero points (fully_connected_util.cc:91-99: w = u*s - s*(shift + zp)) are taken by every
@@ -272,6 +273,20 @@ typedef struct {
   float scalar_zero_point;
   int32_t has_bias;
   int32_t max_tokens; /* upper bound for mldhip_op_set_shape's b*h*w */
+  /* ConvRuntimeCheckDesc (common/task/gpu_operation.h:384-412), read when has_runtime_check != 0;
+   * an index < 0 means "not set".  With a channel bound set, the op takes one more src object,
+   * "params" (int32 values in device memory, registered last, as the reference's tests bind it:
+   * common/kernels/tests/fully_connected_test_util.cc:1195-1204), read at launch on the device:
+   *   src_end_ch = min(params[src_end_ch_index], i): the K loop stops after ceil(src_end_ch / 4)
+   *     slices (fully_connected.cc:750-755, 795; not applied with group-wise scales, whose loop runs
+   *     over all groups, :784-794);
+   *   dst slices from min(round_up(params[dst_end_ch_index], 32) / 4, ceil(o/4)) on are not
+   *     written (fully_connected_util.cc:231-243, fully_connected.cc:644-652).
+   * Ringed weights are refused as the reference refuses them for these weights: uint4 by type,
+   * uint8 I4O4 by layout (fully_connected.cc:1087-1097). */
+  int32_t has_runtime_check;
+  int32_t src_end_ch_index, dst_end_ch_index;
+  int32_t ring_o_offset_index, ring_i_offset_index, ring_size;
 } mldhip_fc_desc;
 
 int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);

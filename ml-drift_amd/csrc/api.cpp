@@ -99,6 +99,7 @@ struct mldhip_op {
   int idx_scale = -1, idx_zp = -1, idx_bias = -1;
   // FullyConnected with batched weights selected by a runtime tensor of ids
   int idx_weights = 1, idx_ids = -1;
+  int idx_params = -1;  // runtime channel bounds
   int weights_batch = 1;  // ExternalWeights::shape.h
   int shared_src = 0;     // the source tensor has one row that every dst row reads
   float* partial = nullptr;
@@ -395,10 +396,23 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     if (d->has_zero_point_tensor && d->scale_o * d->scale_i == 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "a zero-point tensor needs a scale tensor of the same shape");
   }
+  bool runtime_bounds = false;
+  if (d->has_runtime_check) {
+    // ringed weights: refused as the reference refuses them for these weights (fully_connected.cc:1087-1097)
+    if (d->ring_o_offset_index >= 0 || d->ring_i_offset_index >= 0) {
+      if (wd.type == MLDHIP_UINT4)
+        return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type for ringed weights.");
+      return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout for ringed weights.");
+    }
+    runtime_bounds = d->src_end_ch_index >= 0 || d->dst_end_ch_index >= 0;
+    if (runtime_bounds && batch_ids)
+      return Fail(MLDHIP_UNIMPLEMENTED, "runtime channel bounds with batched weights are not supported");
+  }
   mldhip_op* op = new (std::nothrow) mldhip_op();
   if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
   op->kind = mldhip_op::kFc;
   op->fc = *d;
+  if (!d->has_runtime_check) op->fc.src_end_ch_index = op->fc.dst_end_ch_index = -1;
   op->max_tokens = d->max_tokens;
   op->AddSrc("src_tensor");
   if (batch_ids) {  // registered before the weights objects (fully_connected.cc:1203-1208)
@@ -420,6 +434,10 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   if (d->has_bias) {
     op->idx_bias = (int)op->src_names.size();
     op->AddSrc("biases");
+  }
+  if (runtime_bounds) {
+    op->idx_params = (int)op->src_names.size();
+    op->AddSrc("params");
   }
   op->AddDst("dst_tensor");
   // split-K workspace of the fp16 streaming and matrix-core kernels: allocated here, so that no
@@ -566,6 +584,8 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
     if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
+    if (op->idx_params >= 0)
+      (*src)[op->idx_params] = (size_t)(std::max(d.src_end_ch_index, d.dst_end_ch_index) + 1) * sizeof(int32_t);
     (*dst)[0] = ns * m * 4 * TypeBytes(d.dst_type);
   } else if (op->kind == mldhip_op::kQuant) {
     const mldhip_quant_desc& d = op->q;
@@ -639,6 +659,11 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
   a.scalar_zero_point = d.has_scalar_zero_point ? d.scalar_zero_point : 0.0f;
   a.partial = op->partial;
   a.partial_floats = op->partial_floats;
+  if (op->idx_params >= 0) {
+    a.params = static_cast<const int32_t*>(op->src_ptr[op->idx_params]);
+    a.src_end_ch_index = d.src_end_ch_index;
+    a.dst_end_ch_index = d.dst_end_ch_index;
+  }
   *out = a;
   return MLDHIP_OK;
 }
@@ -662,17 +687,23 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         tokens = op->w;
       }
       batch.group = d.weights.output_group_size;
+      if (op->idx_params >= 0) {
+        batch.params = static_cast<const int32_t*>(op->src_ptr[op->idx_params]);
+        batch.src_end_ch_index = d.src_end_ch_index;
+        batch.dst_end_ch_index = d.dst_end_ch_index;
+      }
       const int8_t* act = static_cast<const int8_t*>(op->src_ptr[0]);
       const uint8_t* weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
       int32_t* dst = static_cast<int32_t*>(op->dst_ptr[0]);
-      if (GetTuning().force_generic <= 0 && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
+      if (GetTuning().force_generic <= 0 && op->idx_params < 0 && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
         e = LaunchFcInt8MathStream(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
       else
         e = LaunchFcInt8Math(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
-      const bool force_generic = GetTuning().force_generic > 0;
+      // runtime channel bounds are served by the unspecialised kernel
+      const bool force_generic = GetTuning().force_generic > 0 || a.params != nullptr;
       // batched weights by runtime ids: the streaming GEMVs, else the unspecialised kernel
       if (a.batch_ids != nullptr) {
         if (!force_generic && FcW4StreamSupported(a))
@@ -741,8 +772,8 @@ int mldhip_fc_launch_fused(mldhip_op* const* ops, int count, void* stream_ptr) {
   for (int i = 0; i < count; ++i) {
     mldhip_op* op = ops[i];
     if (!op) return Fail(MLDHIP_INVALID_ARGUMENT, "null op");
-    if (op->kind != mldhip_op::kFc || op->fc.src_type == MLDHIP_INT8 || op->idx_ids >= 0)
-      return Fail(MLDHIP_FAILED_PRECONDITION, "fused launch takes floating-point FullyConnected ops without batched weights");
+    if (op->kind != mldhip_op::kFc || op->fc.src_type == MLDHIP_INT8 || op->idx_ids >= 0 || op->idx_params >= 0)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "fused launch takes floating-point FullyConnected ops without batched weights or runtime channel bounds");
     if (int rc = CheckBindings(op)) return rc;
     if (int rc = BuildFcArgs(op, &args[i])) return rc;
     const FcArgs &a = args[i], &f = args[0];
@@ -770,8 +801,8 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
   mldhip_op* ops[2] = {gate, up};
   FcArgs args[2];
   for (int i = 0; i < 2; ++i) {
-    if (ops[i]->kind != mldhip_op::kFc || ops[i]->fc.src_type == MLDHIP_INT8 || ops[i]->idx_ids >= 0)
-      return Fail(MLDHIP_FAILED_PRECONDITION, "gated launch takes floating-point FullyConnected ops without batched weights");
+    if (ops[i]->kind != mldhip_op::kFc || ops[i]->fc.src_type == MLDHIP_INT8 || ops[i]->idx_ids >= 0 || ops[i]->idx_params >= 0)
+      return Fail(MLDHIP_FAILED_PRECONDITION, "gated launch takes floating-point FullyConnected ops without batched weights or runtime channel bounds");
     if (int rc = CheckBindings(ops[i])) return rc;
     if (int rc = BuildFcArgs(ops[i], &args[i])) return rc;
   }

@@ -54,7 +54,25 @@ struct GenericParams {
   // 279-290): blockIdx.z = dst row; m = tokens per row
   const int32_t* batch_ids;
   int rows, src_rows, weights_batch;
+  // runtime channel bounds (common/task/gpu_operation.h:384-412): device values, index < 0 = not set
+  const int32_t* params;
+  int src_end_ch_index, dst_end_ch_index;
+  int k_channels;
 };
+
+// K-slices the loop covers and dst slices that are written, with runtime channel bounds
+// (fully_connected.cc:750-755, 795; fully_connected_util.cc:231-243 with
+// ConvRuntimeCheckDesc::GetRuntimeEndSlice, common/task/gpu_operation.cc:1832-1836).  The source
+// bound does not apply to group-wise scales: that loop runs over all groups (fully_connected.cc:784-794).
+__device__ __forceinline__ int RuntimeSrcEndSlices(const int32_t* params, int index, int k_channels, int ks, bool block) {
+  if (params == nullptr || index < 0 || block) return ks;
+  const int end_ch = min(params[index], k_channels);
+  return min(max((end_ch + 3) / 4, 0), ks);
+}
+__device__ __forceinline__ int RuntimeDstEndSlice(const int32_t* params, int index, int ns) {
+  if (params == nullptr || index < 0) return ns;
+  return min(max(((params[index] + 31) / 32) * 32 / 4, 0), ns);
+}
 
 template <typename ActT, typename DstT, int WBITS, int TB>
 __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
@@ -82,7 +100,9 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[t][c] = 0.0f;
 
-  if (ds < p.ns) {
+  const int ks_end = RuntimeSrcEndSlices(p.params, p.src_end_ch_index, p.k_channels, p.ks, p.scale_kind == kScaleBlock);
+  const int ns_end = RuntimeDstEndSlice(p.params, p.dst_end_ch_index, p.ns);
+  if (ds < ns_end) {
     float s[4], z[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -97,7 +117,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
       }
     }
 #pragma unroll 4
-    for (int ks = ty; ks < p.ks; ks += kKl) {
+    for (int ks = ty; ks < ks_end; ks += kKl) {
       if (p.scale_kind == kScaleBlock) {
         int g = ks / p.group_slices;
         if (g >= p.groups) g = p.groups - 1;
@@ -144,7 +164,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 #pragma unroll
     for (int c = 0; c < 4; ++c) red[ty][tx][t * 4 + c] = acc[t][c];
   __syncthreads();
-  if (ty == 0 && ds < p.ns) {
+  if (ty == 0 && ds < ns_end) {
     DstT* dst = static_cast<DstT*>(p.dst);
     const DstT* bias = static_cast<const DstT*>(p.bias);
 #pragma unroll
@@ -178,7 +198,7 @@ template <int WBITS, int TB>
 __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restrict__ act,
                                                            const uint8_t* __restrict__ weights,
                                                            int32_t* __restrict__ dst, int m, int ks_n,
-                                                           int ns, FcBatchRows batch) {
+                                                           int ns, int k_channels, FcBatchRows batch) {
   __shared__ int red[kKl][kSl][TB * 4];
   const int tx = threadIdx.x, ty = threadIdx.y;
   const int ds = blockIdx.x * kSl + tx;
@@ -195,9 +215,11 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
   for (int t = 0; t < TB; ++t)
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[t][c] = 0;
-  if (ds < ns) {
+  const int ks_end = RuntimeSrcEndSlices(batch.params, batch.src_end_ch_index, k_channels, ks_n, false);
+  const int ns_end = RuntimeDstEndSlice(batch.params, batch.dst_end_ch_index, ns);
+  if (ds < ns_end) {
 #pragma unroll 4
-    for (int ks = ty; ks < ks_n; ks += kKl) {
+    for (int ks = ty; ks < ks_end; ks += kKl) {
       const size_t blk = BlockIndex(ks, ds, ks_n, ns, batch.group);
       uint32_t w0, w1, w2, w3;  // per output channel: the 4 input-channel values, one per byte
       if (WBITS == 4) {
@@ -258,7 +280,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
 #pragma unroll
     for (int c = 0; c < 4; ++c) red[ty][tx][t * 4 + c] = acc[t][c];
   __syncthreads();
-  if (ty == 0 && ds < ns) {
+  if (ty == 0 && ds < ns_end) {
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
       const int tok = tok0 + t;
@@ -299,6 +321,10 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
   p.rows = a.rows;
   p.src_rows = a.src_rows;
   p.weights_batch = a.weights_batch;
+  p.params = a.params;
+  p.src_end_ch_index = a.src_end_ch_index;
+  p.dst_end_ch_index = a.dst_end_ch_index;
+  p.k_channels = a.k;
   if (kernel_name) *kernel_name = "fc_generic_kernel";
   const bool w8 = a.weight_bits == 8;
   if (a.act_f16 && a.dst_f16)
@@ -319,9 +345,9 @@ hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* 
   dim3 block(kSl, kKl);
   if (kernel_name) *kernel_name = "fc_int8_math_kernel";
   if (weight_bits == 8)
-    hipLaunchKernelGGL((fc_int8_math_kernel<8, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, batch);
+    hipLaunchKernelGGL((fc_int8_math_kernel<8, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, k, batch);
   else
-    hipLaunchKernelGGL((fc_int8_math_kernel<4, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, batch);
+    hipLaunchKernelGGL((fc_int8_math_kernel<4, TB>), grid, block, 0, stream, act, weights, dst, m, ks, ns, k, batch);
   return hipGetLastError();
 }
 

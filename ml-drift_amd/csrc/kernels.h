@@ -60,6 +60,10 @@ struct FcArgs {
   // Plain launches: batch_ids = nullptr, rows = src_rows = weights_batch = 1.
   const int32_t* batch_ids = nullptr;
   int rows = 1, src_rows = 1, weights_batch = 1;
+  // Runtime channel bounds (ConvRuntimeCheckDesc): int32 values in device memory, read by the
+  // kernel; an index < 0 = not set.  Served by the unspecialised kernels.
+  const int32_t* params = nullptr;
+  int src_end_ch_index = -1, dst_end_ch_index = -1;
 };
 
 // Split-K workspace sizing for the streaming GEMV.
@@ -98,6 +102,9 @@ struct FcBatchRows {
   const int32_t* ids = nullptr;
   int rows = 1, src_rows = 1, weights_batch = 1;
   int group = 0;  // output group size of the packed weights (plain launches only; 0 = one group)
+  // runtime channel bounds, as in FcArgs (the tiled kernel only)
+  const int32_t* params = nullptr;
+  int src_end_ch_index = -1, dst_end_ch_index = -1;
 };
 
 // int8 activations x uint8/uint4 weights -> int32 (no scales).

@@ -104,6 +104,17 @@ struct ExternalWeights {
   float scalar_zero_point = 0.0f;
 };
 
+// ConvRuntimeCheckDesc (common/task/gpu_operation.h:384-412): indices into the int32 "params"
+// object of the op, -1 = not set.
+struct ConvRuntimeCheckDesc {
+  int src_end_ch_index = -1;
+  int dst_end_ch_index = -1;
+  int ring_o_offset_index = -1;
+  int ring_i_offset_index = -1;
+  int ring_size = 0;
+  bool HasValues() const { return src_end_ch_index >= 0 || dst_end_ch_index >= 0; }
+};
+
 // A node executor: what ClOperation is to a GPUOperation in the reference.
 class HipOperation {
  public:
@@ -143,7 +154,8 @@ class HipOperation {
 
 namespace detail {
 inline mldhip_fc_desc FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
-                               const ExternalWeights& weights, bool has_bias, int max_tokens);
+                               const ExternalWeights& weights, bool has_bias, int max_tokens,
+                               const ConvRuntimeCheckDesc& runtime_check = {});
 }  // namespace detail
 
 // CreateFullyConnectedWeightsBatchIds (common/kernels/fully_connected.h, .cc:1174-1216): the
@@ -162,10 +174,12 @@ inline Status CreateFullyConnectedWeightsBatchIds(CalculationsPrecision precisio
   return {};
 }
 
+// With runtime channel bounds the op takes a last src object "params" (int32 values on the device).
 inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precision, DataType src_type,
                                                   DataType dst_type, const ExternalWeights& weights, bool has_bias,
-                                                  int max_tokens, HipOperation* result) {
-  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens);
+                                                  int max_tokens, HipOperation* result,
+                                                  const ConvRuntimeCheckDesc& runtime_check = {}) {
+  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens, runtime_check);
   mldhip_op* op = nullptr;
   const int rc = mldhip_fc_create(&d, &op);
   if (rc != MLDHIP_OK) return Status::FromCode(rc);
@@ -174,8 +188,15 @@ inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precisio
 }
 
 inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
-                                       const ExternalWeights& weights, bool has_bias, int max_tokens) {
+                                       const ExternalWeights& weights, bool has_bias, int max_tokens,
+                                       const ConvRuntimeCheckDesc& runtime_check) {
   mldhip_fc_desc d{};
+  d.has_runtime_check = 1;
+  d.src_end_ch_index = runtime_check.src_end_ch_index;
+  d.dst_end_ch_index = runtime_check.dst_end_ch_index;
+  d.ring_o_offset_index = runtime_check.ring_o_offset_index;
+  d.ring_i_offset_index = runtime_check.ring_i_offset_index;
+  d.ring_size = runtime_check.ring_size;
   d.precision = (int)precision;
   d.src_type = (int)src_type;
   d.dst_type = (int)dst_type;

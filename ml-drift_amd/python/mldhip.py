@@ -49,7 +49,9 @@ class FcDesc(C.Structure):
                 ("scale_o", C.c_int32), ("scale_i", C.c_int32), ("scalar_scale", C.c_float),
                 ("has_zero_point_tensor", C.c_int32), ("has_scalar_zero_point", C.c_int32),
                 ("scalar_zero_point", C.c_float), ("has_bias", C.c_int32),
-                ("max_tokens", C.c_int32)]
+                ("max_tokens", C.c_int32), ("has_runtime_check", C.c_int32),
+                ("src_end_ch_index", C.c_int32), ("dst_end_ch_index", C.c_int32),
+                ("ring_o_offset_index", C.c_int32), ("ring_i_offset_index", C.c_int32), ("ring_size", C.c_int32)]
 
 
 class QuantDesc(C.Structure):
@@ -378,8 +380,10 @@ def fc_launch_gated(gate, up, activation, dst, stream=0):
 
 def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1, 1),
               scalar_scale=1.0, has_zero_point_tensor=False, scalar_zero_point=None,
-              has_bias=False, max_tokens=1, weights_batch=None, shared_src=False):
-    """weights_batch: number of weight matrices of a batch-ids op (mldhip_fc_batch_ids_create)."""
+              has_bias=False, max_tokens=1, weights_batch=None, shared_src=False, src_end_ch_index=None,
+              dst_end_ch_index=None, ring_o_offset_index=None, ring_i_offset_index=None, ring_size=0):
+    """weights_batch: number of weight matrices of a batch-ids op (mldhip_fc_batch_ids_create).
+    src_end_ch_index / dst_end_ch_index: ConvRuntimeCheckDesc indices into the "params" object."""
     d = FcDesc()
     d.precision, d.src_type, d.dst_type, d.o, d.i = precision, src_type, dst_type, o, i
     d.weights = weights_desc
@@ -390,6 +394,11 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
     d.scalar_zero_point = 0.0 if scalar_zero_point is None else scalar_zero_point
     d.has_bias = int(has_bias)
     d.max_tokens = max_tokens
+    checks = (src_end_ch_index, dst_end_ch_index, ring_o_offset_index, ring_i_offset_index)
+    d.has_runtime_check = int(any(v is not None for v in checks))
+    d.src_end_ch_index, d.dst_end_ch_index, d.ring_o_offset_index, d.ring_i_offset_index = [
+        -1 if v is None else v for v in checks]
+    d.ring_size = ring_size
     h = C.c_void_p()
     if weights_batch is not None:
         check(lib().mldhip_fc_batch_ids_create(C.byref(d), weights_batch, int(shared_src), C.byref(h)))

@@ -227,6 +227,52 @@ def fc_kernel(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=S
     return out
 
 
+def runtime_end_slices(src_end_ch, dst_end_ch, k, n, block_quantized):
+    """(K-slices the loop covers, dst slices written) under runtime channel bounds:
+    src_end_ch = min(params value, src channels), src_end_slices = (src_end_ch + 3) / 4
+    (common/kernels/fully_connected.cc:750-755, 795; the group-wise loop runs over all groups,
+    :784-794); dst_end_slice = min(round_up(params value, 32) / 4, dst slices)
+    (ConvRuntimeCheckDesc::GetRuntimeEndSlice, common/task/gpu_operation.cc:1832-1836, with
+    kChannelsAlignment = 32; fully_connected_util.cc:231-243)."""
+    ks, ns = div_up(k, 4), div_up(n, 4)
+    ks_end = ks
+    if src_end_ch is not None and not block_quantized:
+        ks_end = max(0, min(ks, (min(int(src_end_ch), k) + 3) // 4))
+    ns_end = ns
+    if dst_end_ch is not None:
+        ns_end = max(0, min(ns, ((int(dst_end_ch) + 31) // 32) * 32 // 4))
+    return ks_end, ns_end
+
+
+def fc_kernel_runtime_check(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=SCALE_LINEAR, scale=None,
+                            zero_point=None, bias=None, groups=1, src_end_ch=None, dst_end_ch=None, dst_before=None):
+    """The generated kernel with ConvRuntimeCheckDesc channel bounds (fully_connected.cc:644-652: work
+    items of slices >= dst_end_slice return before they write; :750-755, 795: the K loop stops at
+    src_end_slices).  The K loop over the first src_end_slices slices is the kernel on the leading
+    rows of the packed buffer (the one-group I4O4 layout has the K-slice outermost), so this
+    restatement runs `fc_kernel` on that prefix; dst slices that are not written keep `dst_before`
+    (zeros when not given).  `weights`: packed in the reference's one-group layout."""
+    tdt = np.float32 if precision == PREC_F32 else np.uint16
+    ks, ns = div_up(k, 4), div_up(n, 4)
+    ks_end, ns_end = runtime_end_slices(src_end_ch, dst_end_ch, k, n, scale_kind == SCALE_BLOCK)
+    out = np.zeros((ns, m, 4), tdt) if dst_before is None else _c(dst_before, tdt).reshape(ns, m, 4).copy()
+    if ns_end == 0:
+        return out
+    block_bytes = 16 if weight_bits == 8 else 8
+    act = _c(act_slices, tdt).reshape(ks, m, 4)
+    w = _c(weights, np.uint8).reshape(ks, ns * block_bytes)
+    if ks_end == 0:
+        # no K-slice: the result is the bias alone (0 without one), converted like any result
+        zero_act = np.zeros((1, m, 4), tdt)
+        full = fc_kernel(zero_act, w[:1].copy(), m, 4, n, precision, weight_bits, scale_kind, scale, zero_point, bias,
+                         1 if scale_kind != SCALE_BLOCK else groups)
+    else:
+        full = fc_kernel(np.ascontiguousarray(act[:ks_end]), np.ascontiguousarray(w[:ks_end]), m, ks_end * 4, n, precision,
+                         weight_bits, scale_kind, scale, zero_point, bias, groups)
+    out[:ns_end] = full[:ns_end]
+    return out
+
+
 def fc_batch_ids_kernel(act_slices, ids, weights, rows, row_tokens, src_rows, weights_batch, k, n, precision,
                         weight_bits, scale_kind=SCALE_LINEAR, scale=None, zero_point=None, bias=None, groups=1):
     """The generated kernel with batched weights and runtime batch ids

@@ -59,6 +59,24 @@ int main() {
                                            false, 1, &bad);
   EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !bad.valid());
 
+  // runtime channel bounds: one more src object, "params", registered last; ringed weights are refused
+  w.desc = GetFullyConnectedInt4WeightsDesc(w.shape);
+  ConvRuntimeCheckDesc rc_desc;
+  rc_desc.src_end_ch_index = 1;
+  rc_desc.dst_end_ch_index = 3;
+  HipOperation bounded;
+  EXPECT(CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
+                                             /*has_bias=*/true, 4, &bounded, rc_desc)
+             .ok());
+  names = bounded.GetSrcTensorsNames();
+  EXPECT(names.size() == 5 && names[3] == "biases" && names[4] == "params");
+  rc_desc.ring_o_offset_index = 0;
+  rc_desc.ring_size = 14336;
+  HipOperation ringed;
+  st = CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
+                                           false, 1, &ringed, rc_desc);
+  EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !ringed.valid());
+
   // the mixture-of-experts FullyConnected: fully_connected.cc:1203-1213 registers batch_ids before the weights
   ExternalWeights we;
   we.shape = OHWI{768, 128, 1, 2048};

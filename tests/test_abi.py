@@ -191,3 +191,18 @@ def test_scale_to_tensor_batched_matches_oracle(oracle):
     assert np.array_equal(got16, oracle.f32_to_f16_bits(oracle.scale_to_hoio4_batched(s).reshape(-1)))
     # one matrix: the unbatched conversion
     assert np.array_equal(M.scale_to_tensor_batched(s[:, :1, :], M.FLOAT32), M.scale_to_tensor(s[:, 0, :], M.FLOAT32))
+
+
+def test_runtime_check_objects_and_ringed_weights():
+    """Runtime channel bounds add a last src object "params"; ringed weights are refused with the
+    reference's messages (common/kernels/fully_connected.cc:1087-1097)."""
+    d4 = M.fc_int4_weights_desc(64, 64)
+    op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4, scale_shape=(64, 1), has_bias=True,
+                     src_end_ch_index=1, dst_end_ch_index=3)
+    assert op.src_names == ["src_tensor", "weights", "weights_scale", "biases", "params"]
+    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4,
+                       scale_shape=(64, 1), ring_o_offset_index=0, ring_size=64)
+    assert "type for ringed weights" in msg
+    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64,
+                       M.fc_int8_weights_desc(64, 64), scale_shape=(64, 1), ring_i_offset_index=0, ring_size=64)
+    assert "layout for ringed weights" in msg

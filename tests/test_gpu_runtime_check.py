@@ -1,0 +1,111 @@
+"""GPU parity of the FullyConnected with runtime channel bounds (ConvRuntimeCheckDesc: src_end_ch /
+dst_end_ch read at launch from the int32 "params" object), through the C-ABI, against the oracle's
+restatement of the bounded kernel; the reference's own test shape and runtime channels
+(common/kernels/tests/fully_connected_test_util.cc:1260-1300) and larger layers."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mldhip as M
+import workloads as W
+from test_gpu_fc import check_fp
+
+
+def run_bounded(oracle, case, src_end_ch, dst_end_ch, params_values=None):
+    import torch
+    o = oracle
+    m, k, n, bits, groups = case["m"], case["k"], case["n"], case["weight_bits"], case["groups"]
+    f16 = case["tensor_dtype"] == np.float16
+    td = case["tensor_dtype"]
+    tt = torch.float16 if f16 else torch.float32
+    mt = M.FLOAT16 if f16 else M.FLOAT32
+    ns = (n + 3) // 4
+    desc, packed = W.pack_fc_weights(case, reference_layout=True)
+    # params: 4 int32 values as the reference's tests lay them out (src start, src end, dst start, dst end)
+    params = np.full(4, -1, np.int32)
+    kwargs = {}
+    if src_end_ch is not None:
+        params[1] = src_end_ch
+        kwargs["src_end_ch_index"] = 1
+    if dst_end_ch is not None:
+        params[3] = dst_end_ch
+        kwargs["dst_end_ch_index"] = 3
+    scale_dev = torch.from_numpy(M.scale_to_tensor(case["scale"], mt).view(td) if f16 else M.scale_to_tensor(case["scale"], mt)).cuda()
+    srcs = [torch.from_numpy(W.to_slices(case["act"]).astype(td)).cuda(), torch.from_numpy(packed).cuda(), scale_dev]
+    bias = None
+    if case["bias"] is not None:
+        bias = np.zeros(ns * 4, td)
+        bias[:n] = case["bias"]
+        srcs.append(torch.from_numpy(bias).cuda())
+    srcs.append(torch.from_numpy(params).cuda())
+    out = torch.full((ns, m, 4), 7.0, dtype=tt, device="cuda")
+    op = M.fc_create(M.PRECISION_F32_F16 if f16 else M.PRECISION_F32, mt, mt, n, k, desc, scale_shape=(n, groups),
+                     has_bias=case["bias"] is not None, max_tokens=m, **kwargs)
+    assert op.src_names[-1] == "params"
+    op.bind(srcs, [out])
+    op.set_shape(1, 1, m)
+    print("runtime check", m, k, n, bits, groups, src_end_ch, dst_end_ch, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert op.kernel_name == "fc_generic_kernel", op.kernel_name
+    got = out.cpu().numpy().astype(np.float32)
+    # oracle: the bounded kernel restatement over the reference's layout
+    prec = o.PREC_F32F16 if f16 else o.PREC_F32
+    conv = (lambda a: o.f32_to_f16_bits(np.asarray(a, np.float32))) if f16 else (lambda a: np.asarray(a, np.float32))
+    if groups == 1:
+        sc = np.zeros(ns * 4, np.float32); sc[:n] = case["scale"][:, 0]
+        kind = o.SCALE_LINEAR
+    else:
+        sc = o.scale_to_hoio4(case["scale"]); kind = o.SCALE_BLOCK
+    ref = o.fc_kernel_runtime_check(conv(o.to_slices(case["act"])), packed, m, k, n, prec, bits, kind, conv(sc), None,
+                                    None if bias is None else conv(bias.astype(np.float32)), groups,
+                                    src_end_ch=src_end_ch, dst_end_ch=dst_end_ch,
+                                    dst_before=conv(np.full((ns, m, 4), 7.0, np.float32)))
+    ref = o.f16_bits_to_f32(ref) if f16 else ref
+    ks_end, ns_end = o.runtime_end_slices(src_end_ch, dst_end_ch, k, n, groups > 1)
+    # untouched slices are bit-identical (the fill), written ones meet the FullyConnected bar
+    assert np.array_equal(got[ns_end:], ref[ns_end:]) and np.all(got[ns_end:] == 7.0)
+    if ns_end:
+        sub = dict(case, n=ns_end * 4)
+        check_fp(W.from_slices(got[:ns_end], ns_end * 4), W.from_slices(ref[:ns_end], ns_end * 4).astype(np.float64), sub,
+                 "bounded kernel restatement")
+    return got
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rc", [dict(src_end_ch=4, dst_end_ch=8), dict(src_end_ch=8), dict(src_end_ch=175), dict(dst_end_ch=14)])
+def test_reference_runtime_channel_cases(oracle, dtype, rc):
+    case = W.make_fc_case(seed=9, m=1, k=171, n=533, weight_bits=8, tensor_dtype=dtype, groups=1, with_bias=True,
+                          act_uniform=True)
+    run_bounded(oracle, case, rc.get("src_end_ch"), rc.get("dst_end_ch"))
+
+
+@pytest.mark.parametrize("bits,m,k,n,groups,src_end,dst_end", [
+    (4, 1, 4096, 2048, 1, 1000, 300), (4, 3, 2048, 1024, 64, 77, 1000), (8, 5, 1024, 516, 1, 0, 33),
+    (4, 1, 512, 256, 1, 512, 0), (4, 2, 256, 8192, 1, 129, 4097), (8, 1, 96, 64, 3, 5, 64)])
+def test_runtime_bounds_sweep(oracle, bits, m, k, n, groups, src_end, dst_end):
+    """Bounds inside the tensors, at and beyond their ends, zero, unaligned to 4 and to 32; group-wise
+    scales ignore the source bound (the reference's group loop runs over all groups)."""
+    case = W.make_fc_case(seed=k + n, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups, with_bias=True)
+    run_bounded(oracle, case, src_end, dst_end)
+
+
+def test_bounds_are_read_at_launch(oracle):
+    """The same op, the bound rewritten on the device between two launches."""
+    import torch
+    case = W.make_fc_case(seed=4, m=1, k=1024, n=1024, weight_bits=4, tensor_dtype=np.float16, groups=1)
+    a = run_bounded(oracle, case, 1024, 64)
+    b = run_bounded(oracle, case, 1024, 1024)
+    assert np.array_equal(a[:16], b[:16]) and np.all(a[16:] == 7.0) and not np.any(b == 7.0)
+
+
+def test_ringed_weights_are_refused_like_the_reference():
+    d4 = M.fc_int4_weights_desc(64, 64)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4, scale_shape=(64, 1), ring_o_offset_index=0, ring_size=64)
+    assert e.value.code == M.INVALID_ARGUMENT and "type for ringed weights" in e.value.message
+    d8 = M.fc_int8_weights_desc(64, 64)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d8, scale_shape=(64, 1), ring_i_offset_index=0, ring_size=64)
+    assert e.value.code == M.INVALID_ARGUMENT and "layout for ringed weights" in e.value.message

@@ -329,3 +329,61 @@ def run_batch_ids_int8_oracle(o, c):
 def test_batch_ids_int8_math_exact(oracle, bits, rows, row_tokens, src_rows, k, n, batch):
     c = make_batch_ids_int8_case(rows + k + bits, rows, row_tokens, src_rows, k, n, batch, bits)
     assert np.array_equal(run_batch_ids_int8_oracle(oracle, c), batch_ids_int8_exact(c))
+
+
+# ------------------------------------------------------------------------------------------
+# Runtime channel bounds (ConvRuntimeCheckDesc): the reference's FullyConnectedRuntimeChWi8Test
+# (common/kernels/tests/fully_connected_test_util.cc:1260-1300): K = 171, N = 533, int8
+# per-channel weights + bias, runtime channels {src_end 4, dst_end 8}, {src_end 8},
+# {src_end K + 4}, {dst_end 14}, against FullyConnectedReference with runtime channels
+# (common/task/testing_ref_ops.cc:961-988: sum over s < src_end_ch for d < dst_end_ch), the first
+# dst_end_ch values compared (fully_connected_test_util.cc:1208-1222).
+# ------------------------------------------------------------------------------------------
+RUNTIME_CHANNEL_CASES = [dict(src_end_ch=4, dst_end_ch=8), dict(src_end_ch=8), dict(src_end_ch=171 + 4), dict(dst_end_ch=14)]
+
+
+def test_runtime_end_slices_literals(oracle):
+    o = oracle
+    # round_up(dst_end_ch, 32) / 4, capped at the slice count; (src_end_ch + 3) / 4 after the cap at K
+    assert o.runtime_end_slices(4, 8, 171, 533, False) == (1, 8)
+    assert o.runtime_end_slices(8, None, 171, 533, False) == (2, 134)
+    assert o.runtime_end_slices(175, None, 171, 533, False) == (43, 134)
+    assert o.runtime_end_slices(None, 14, 171, 533, False) == (43, 8)
+    assert o.runtime_end_slices(None, 33, 171, 533, False) == (43, 16)
+    assert o.runtime_end_slices(None, 532, 171, 533, False) == (43, 134)   # 544 / 4 = 136 -> capped
+    assert o.runtime_end_slices(5, None, 171, 533, False) == (2, 134)
+    assert o.runtime_end_slices(5, None, 176, 533, True) == (44, 134)      # group-wise scales: all groups
+    assert o.runtime_end_slices(-3, -1, 171, 533, False) == (0, 0)
+
+
+@pytest.mark.parametrize("precision", ["f32", "f16"])
+@pytest.mark.parametrize("rc", RUNTIME_CHANNEL_CASES)
+def test_runtime_channels_reference_test(oracle, precision, rc):
+    o = oracle
+    k, n = 171, 533
+    rng = np.random.default_rng(5)
+    w = rng.integers(-128, 128, size=(n, k), dtype=np.int8)
+    scale = (rng.uniform(0.1, 1.0, size=n) / 128.0).astype(np.float32)
+    bias = rng.uniform(-1, 1, size=n).astype(np.float32)
+    src = rng.uniform(-1, 1, size=(1, k)).astype(np.float32)
+    prec = o.PREC_F32 if precision == "f32" else o.PREC_F32F16
+    if precision == "f16":
+        scale, bias, src = [x.astype(np.float16).astype(np.float32) for x in (scale, bias, src)]
+    ns = (n + 3) // 4
+    packed = o.int8_as_uint8(w, o.LAYOUT_I4O4, ns)
+    pad = lambda v: np.concatenate([v, np.zeros(ns * 4 - n, np.float32)])
+    sentinel = np.full((ns, 1, 4), 7.0, np.float32)
+    out = o.fc_kernel_runtime_check(tensor(o, o.to_slices(src), prec), packed, 1, k, n, prec, 8, o.SCALE_LINEAR,
+                                    tensor(o, pad(scale), prec), None, tensor(o, pad(bias), prec),
+                                    dst_before=tensor(o, sentinel, prec), **rc)
+    got = o.from_slices(to_f32(o, out, prec), ns * 4)[0]
+    src_end = min(rc.get("src_end_ch", k), k)
+    dst_end = rc.get("dst_end_ch", n)
+    ref = (src[0, :src_end].astype(np.float64) @ (w[:, :src_end].astype(np.float64) * scale[:, None].astype(np.float64)).T) + bias
+    eps = (1e-6 if precision == "f32" else 2e-3) * (k + 1)
+    assert np.all(np.abs(got[:dst_end] - ref[:dst_end]) <= eps)
+    # slices from dst_end_slice on are not written
+    ns_end = o.runtime_end_slices(rc.get("src_end_ch"), rc.get("dst_end_ch"), k, n, False)[1]
+    assert np.all(got[ns_end * 4:] == 7.0)
+    if ns_end < ns:
+        assert np.all(got[dst_end:ns_end * 4] != 7.0)
