@@ -454,7 +454,7 @@ static void fc_partial(const mldo_fc_params* p, const void* act, const uint8_t* 
   const int acc_half = p->precision == MLDO_PREC_F16;    /* AccType */
   const int ks = div_up(p->k, 4), ns = div_up(p->n, 4);
   const float shift = p->weight_bits == 8 ? 128.0f : 8.0f; /* fully_connected_util.cc:35-45 */
-  float w_scale[4], w_bias[4];
+  float w_scale[4] = {0, 0, 0, 0}, w_bias[4] = {0, 0, 0, 0};
   r[0] = r[1] = r[2] = r[3] = 0.0f;
 
   const int block = p->scale_kind == MLDO_SCALE_BLOCK;
@@ -518,34 +518,193 @@ static void fc_partial(const mldo_fc_params* p, const void* act, const uint8_t* 
   }
 }
 
-void mldo_fc_kernel(const mldo_fc_params* p, const void* act, const uint8_t* weights,
-                    const void* scale, const void* zp, const void* bias, void* dst) {
-  const int ns = div_up(p->n, 4);
-  const int is_half = p->precision != MLDO_PREC_F32;
-  const int acc_half = p->precision == MLDO_PREC_F16;
-  const int wg_y = p->wg_y > 0 ? p->wg_y : 1;
-  mldo_fc_params q = *p;
-  q.wg_y = wg_y;
-#ifdef _OPENMP
-  const int nthreads = p->threads > 0 ? p->threads : omp_get_max_threads();
-#pragma omp parallel for schedule(static) num_threads(nthreads)
-#endif
-  for (int dst_s = 0; dst_s < ns; ++dst_s) {
-    for (int tok = 0; tok < p->m; ++tok) {
-      float part[64][4];
-      for (int y = 0; y < wg_y; ++y) fc_partial(&q, act, weights, scale, zp, dst_s, tok, y, part[y]);
-      /* work-group tree reduction, fully_connected_util.cc:321-354 */
-      for (int stride = wg_y / 2; stride > 0; stride /= 2)
-        for (int y = 0; y < stride; ++y)
-          for (int c = 0; c < 4; ++c) part[y][c] = t_add(part[y][c], part[y + stride][c], acc_half);
-      /* fully_connected_util.cc:356-407: convert to dst type, then add bias in dst type */
-      for (int c = 0; c < 4; ++c) {
-        float res = rt(part[0][c], is_half);
-        if (p->has_bias) res = t_add(res, load_t(bias, (size_t)dst_s * 4 + c, is_half), is_half);
-        store_t(dst, ((size_t)dst_s * p->m + tok) * 4 + c, res, is_half);
+/* One (dst slice, token) of the kernel on the scalar path: the wg_y partial sums, the work-group
+ * tree reduction, the conversion and the bias. */
+static void fc_slice_token(const mldo_fc_params* q, const void* act, const uint8_t* weights,
+                           const void* scale, const void* zp, const void* bias, void* dst,
+                           int dst_s, int tok) {
+  const int is_half = q->precision != MLDO_PREC_F32;
+  const int acc_half = q->precision == MLDO_PREC_F16;
+  const int wg_y = q->wg_y;
+  float part[64][4];
+  for (int y = 0; y < wg_y; ++y) fc_partial(q, act, weights, scale, zp, dst_s, tok, y, part[y]);
+  /* work-group tree reduction, fully_connected_util.cc:321-354 */
+  for (int stride = wg_y / 2; stride > 0; stride /= 2)
+    for (int y = 0; y < stride; ++y)
+      for (int c = 0; c < 4; ++c) part[y][c] = t_add(part[y][c], part[y + stride][c], acc_half);
+  /* fully_connected_util.cc:356-407: convert to dst type, then add bias in dst type */
+  for (int c = 0; c < 4; ++c) {
+    float res = rt(part[0][c], is_half);
+    if (q->has_bias) res = t_add(res, load_t(bias, (size_t)dst_s * 4 + c, is_half), is_half);
+    store_t(dst, ((size_t)dst_s * q->m + tok) * 4 + c, res, is_half);
+  }
+}
+
+/* ---- the same operation sequence, eight output channels at a time (x86-64 AVX2 + FMA + F16C) ----
+ *
+ * Serves F32_F16 precision without zero point, wg_y = 1, per-channel or group-wise scales.  Every
+ * half operation of the scalar path (a float operation followed by a rounding to half) becomes one
+ * vector float operation followed by vcvtps2ph / vcvtph2ps, which rounds to nearest even like
+ * d2h(); the operations and their order per output channel are those of fc_partial(), so the
+ * results are bit-identical (tests compare the two paths).  The one place where the scalar path
+ * rounds once from a wider type, the fused q * scale + bias of the dequantization, is exact in
+ * float here: the path is taken only when bias = -shift * scale holds exactly for every scale
+ * (shift is a power of two, so this fails only where shift * scale leaves half's range), and then
+ * q * scale + bias = (q - shift) * scale has at most 8 + 11 significant bits. */
+#if defined(__x86_64__)
+#include <immintrin.h>
+#define MLDO_AVX2 __attribute__((target("avx2,fma,f16c")))
+
+static int g_fast_path_enabled = 1;
+
+MLDO_AVX2 static inline __m256 rt8(__m256 x) {
+  return _mm256_cvtph_ps(_mm256_cvtps_ph(x, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC));
+}
+
+/* all scales s (n_values halves) have -shift * s representable in half */
+static int scales_dequant_exactly(const uint16_t* scale, size_t n_values, float shift) {
+  for (size_t i = 0; i < n_values; ++i) {
+    const float s = mldo_f16_to_f32(scale[i]);
+    const float b = -s * shift;
+    if (!(mldo_f16_to_f32(mldo_f32_to_f16(b)) == b)) return 0; /* also false for NaN */
+  }
+  return 1;
+}
+
+/* Two adjacent dst slices (8 channels) x one K-slice: the four rows wf[i] of dequantized weights. */
+MLDO_AVX2 static inline void dequant_pair(const uint8_t* weights, size_t blk, int bits, __m256 s,
+                                          __m256 b, int use_fma, __m256 wf[4]) {
+  __m128i a0, a1; /* the 16 codes (i*4+o) of slice s and of slice s+1, one per byte */
+  if (bits == 8) {
+    a0 = _mm_loadu_si128((const __m128i*)(weights + blk * 16));
+    a1 = _mm_loadu_si128((const __m128i*)(weights + blk * 16 + 16));
+  } else {
+    const __m128i raw = _mm_loadu_si128((const __m128i*)(weights + blk * 8));
+    const __m128i m4 = _mm_set1_epi8(0x0F);
+    const __m128i lo = _mm_and_si128(raw, m4);
+    const __m128i hi = _mm_and_si128(_mm_srli_epi16(raw, 4), m4);
+    a0 = _mm_unpacklo_epi8(lo, hi); /* low nibble first, common/task/util.cc:772-790 */
+    a1 = _mm_unpackhi_epi8(lo, hi);
+  }
+  const __m128i i01 = _mm_unpacklo_epi32(a0, a1); /* [i=0: slice s, slice s+1][i=1: ...] */
+  const __m128i i23 = _mm_unpackhi_epi32(a0, a1);
+  const __m128i rows[4] = {i01, _mm_srli_si128(i01, 8), i23, _mm_srli_si128(i23, 8)};
+  for (int i = 0; i < 4; ++i) {
+    const __m256 q = _mm256_cvtepi32_ps(_mm256_cvtepu8_epi32(rows[i]));
+    wf[i] = use_fma ? rt8(_mm256_fmadd_ps(q, s, b)) : rt8(_mm256_add_ps(rt8(_mm256_mul_ps(q, s)), b));
+  }
+}
+
+/* dst slices [s0, s0 + 2*units) of token `tok`; act_f: the token's activations as float [k4]. */
+MLDO_AVX2 static inline __attribute__((always_inline)) void fc_pairs_avx2(const mldo_fc_params* p, const float* act_f, const uint8_t* weights,
+                                    const uint16_t* scale, const uint16_t* bias, uint16_t* dst, int s0,
+                                    int units, int tok) {
+  const int ks = div_up(p->k, 4), ns = div_up(p->n, 4);
+  const int block = p->scale_kind == MLDO_SCALE_BLOCK;
+  const int outer_n = block ? p->groups : 1;
+  const int group_slices = block ? ks / p->groups : ks;
+  const __m256 neg_shift = _mm256_set1_ps(p->weight_bits == 8 ? -128.0f : -8.0f);
+  __m256 acc[4], sc[4], bi[4];
+  for (int u = 0; u < units; ++u) acc[u] = _mm256_setzero_ps();
+  for (int outer = 0; outer < outer_n; ++outer) {
+    for (int u = 0; u < units; ++u) {
+      const size_t idx = ((size_t)outer * ns + s0 + 2 * u) * 4;
+      sc[u] = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(scale + idx)));
+      bi[u] = rt8(_mm256_mul_ps(sc[u], neg_shift)); /* t_mul(-s, shift) */
+    }
+    for (int sub = 0; sub < group_slices; ++sub) {
+      const int src_s = outer * group_slices + sub;
+      const __m256 v0 = _mm256_broadcast_ss(act_f + src_s * 4 + 0);
+      const __m256 v1 = _mm256_broadcast_ss(act_f + src_s * 4 + 1);
+      const __m256 v2 = _mm256_broadcast_ss(act_f + src_s * 4 + 2);
+      const __m256 v3 = _mm256_broadcast_ss(act_f + src_s * 4 + 3);
+      for (int u = 0; u < units; ++u) {
+        __m256 wf[4];
+        dequant_pair(weights, (size_t)src_s * ns + s0 + 2 * u, p->weight_bits, sc[u], bi[u], p->use_fma, wf);
+        /* r += float(v.x*w0 + v.y*w1 + v.z*w2 + v.w*w3), the sum in half */
+        __m256 t = rt8(_mm256_mul_ps(v0, wf[0]));
+        t = rt8(_mm256_add_ps(t, rt8(_mm256_mul_ps(v1, wf[1]))));
+        t = rt8(_mm256_add_ps(t, rt8(_mm256_mul_ps(v2, wf[2]))));
+        t = rt8(_mm256_add_ps(t, rt8(_mm256_mul_ps(v3, wf[3]))));
+        acc[u] = _mm256_add_ps(acc[u], t);
       }
     }
   }
+  for (int u = 0; u < units; ++u) {
+    __m256 res = rt8(acc[u]);
+    const int s = s0 + 2 * u;
+    if (p->has_bias)
+      res = rt8(_mm256_add_ps(res, _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(bias + (size_t)s * 4)))));
+    const __m128i h = _mm256_cvtps_ph(res, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC);
+    /* dst is [Ns][M][4]: the two slices of the pair are M*4 halves apart */
+    _mm_storel_epi64((__m128i*)(dst + ((size_t)s * p->m + tok) * 4), h);
+    _mm_storel_epi64((__m128i*)(dst + ((size_t)(s + 1) * p->m + tok) * 4), _mm_srli_si128(h, 8));
+  }
+}
+
+/* the full chunk of four pairs with the pair loop unrolled, the tail chunk as it comes */
+MLDO_AVX2 static void fc_chunk_avx2(const mldo_fc_params* p, const float* act_f, const uint8_t* weights,
+                                    const uint16_t* scale, const uint16_t* bias, uint16_t* dst, int s0,
+                                    int units, int tok) {
+  if (units == 4)
+    fc_pairs_avx2(p, act_f, weights, scale, bias, dst, s0, 4, tok);
+  else
+    fc_pairs_avx2(p, act_f, weights, scale, bias, dst, s0, units, tok);
+}
+
+static int fast_path_serves(const mldo_fc_params* p, const void* scale) {
+  if (!g_fast_path_enabled || p->precision != MLDO_PREC_F32F16 || p->wg_y != 1 || p->has_zero_point) return 0;
+  if (p->weight_bits != 4 && p->weight_bits != 8) return 0;
+  if (p->scale_kind != MLDO_SCALE_LINEAR && p->scale_kind != MLDO_SCALE_BLOCK) return 0;
+  if (p->scale_kind == MLDO_SCALE_BLOCK && (p->groups <= 0 || div_up(p->k, 4) % p->groups)) return 0;
+  if (!__builtin_cpu_supports("avx2") || !__builtin_cpu_supports("fma") || !__builtin_cpu_supports("f16c")) return 0;
+  const size_t n_scales = (size_t)div_up(p->n, 4) * 4 * (p->scale_kind == MLDO_SCALE_BLOCK ? p->groups : 1);
+  return scales_dequant_exactly((const uint16_t*)scale, n_scales, p->weight_bits == 8 ? 128.0f : 8.0f);
+}
+#else
+static int g_fast_path_enabled = 0;
+#endif
+
+void mldo_set_fast_path(int enabled) { g_fast_path_enabled = enabled; }
+
+int mldo_fc_kernel(const mldo_fc_params* p, const void* act, const uint8_t* weights,
+                   const void* scale, const void* zp, const void* bias, void* dst) {
+  const int ns = div_up(p->n, 4);
+  mldo_fc_params q = *p;
+  q.wg_y = p->wg_y > 0 ? p->wg_y : 1;
+#ifdef _OPENMP
+  const int nthreads = p->threads > 0 ? p->threads : omp_get_max_threads();
+#endif
+#if defined(__x86_64__)
+  if (fast_path_serves(&q, scale)) {
+    const int ks4 = div_up(p->k, 4) * 4;
+    float* act_f = (float*)malloc((size_t)p->m * ks4 * sizeof(float));
+    for (int tok = 0; tok < p->m; ++tok)
+      for (int c = 0; c < ks4; ++c)
+        act_f[(size_t)tok * ks4 + c] = mldo_f16_to_f32(((const uint16_t*)act)[((size_t)(c / 4) * p->m + tok) * 4 + c % 4]);
+    const int pairs = ns / 2;           /* an odd last slice goes through the scalar path */
+    const int chunks = div_up(pairs, 4); /* 8 slices: one 64-byte line of uint4 blocks per K-slice */
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+#endif
+    for (int ch = 0; ch < chunks; ++ch) {
+      const int units = pairs - ch * 4 < 4 ? pairs - ch * 4 : 4;
+      for (int tok = 0; tok < p->m; ++tok)
+        fc_chunk_avx2(&q, act_f + (size_t)tok * ks4, weights, (const uint16_t*)scale, (const uint16_t*)bias,
+                      (uint16_t*)dst, ch * 8, units, tok);
+    }
+    if (ns & 1)
+      for (int tok = 0; tok < p->m; ++tok) fc_slice_token(&q, act, weights, scale, zp, bias, dst, ns - 1, tok);
+    free(act_f);
+    return 1;
+  }
+#endif
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+#endif
+  for (int dst_s = 0; dst_s < ns; ++dst_s)
+    for (int tok = 0; tok < p->m; ++tok) fc_slice_token(&q, act, weights, scale, zp, bias, dst, dst_s, tok);
+  return 0;
 }
 
 static inline int32_t sat_add32(int32_t a, int64_t b) {

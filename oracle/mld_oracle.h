@@ -87,8 +87,12 @@ typedef struct {
   int threads;        /* OpenMP threads, <=0: runtime default */
 } mldo_fc_params;
 
-void mldo_fc_kernel(const mldo_fc_params* p, const void* act, const uint8_t* weights,
-                    const void* scale, const void* zero_point, const void* bias, void* dst);
+/* Returns the path taken: 0 = one output channel at a time, 1 = eight channels at a time (x86-64
+ * with AVX2, FMA and F16C, detected at run time; F32_F16 precision without zero point, wg_y = 1).
+ * The two are bit-identical; mldo_set_fast_path(0) forces path 0. */
+int mldo_fc_kernel(const mldo_fc_params* p, const void* act, const uint8_t* weights,
+                   const void* scale, const void* zero_point, const void* bias, void* dst);
+void mldo_set_fast_path(int enabled);
 void mldo_fc_int8_kernel(int m, int k, int n, int weight_bits, const int8_t* act,
                          const uint8_t* weights, int32_t* dst);
 void mldo_fc_reference_f32(int m, int k, int n, const float* src, const float* weights,

@@ -223,8 +223,17 @@ def fc_kernel(act_slices, weights, m, k, n, precision, weight_bits, scale_kind=S
     zp = None if zero_point is None else _c(zero_point, tdt)
     bi = None if bias is None else _c(bias, tdt)
     out = np.empty((div_up(n, 4), m, 4), tdt)
-    lib().mldo_fc_kernel(C.byref(p), _p(act), _p(w), _p(sc), _p(zp), _p(bi), _p(out))
+    global last_fc_path
+    last_fc_path = lib().mldo_fc_kernel(C.byref(p), _p(act), _p(w), _p(sc), _p(zp), _p(bi), _p(out))
     return out
+
+
+last_fc_path = None  # what the last fc_kernel call ran: 0 one channel at a time, 1 eight at a time (AVX2 + F16C)
+
+
+def set_fast_path(enabled):
+    """Switches the vector path of fc_kernel (bit-identical to the scalar one) on or off."""
+    lib().mldo_set_fast_path(int(bool(enabled)))
 
 
 def runtime_end_slices(src_end_ch, dst_end_ch, k, n, block_quantized):

@@ -387,3 +387,58 @@ def test_runtime_channels_reference_test(oracle, precision, rc):
     assert np.all(got[ns_end * 4:] == 7.0)
     if ns_end < ns:
         assert np.all(got[dst_end:ns_end * 4] != 7.0)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,k,n,groups,bias,use_fma", [
+    (1, 256, 128, 1, False, True), (3, 172, 536, 1, True, True), (2, 171, 533, 1, True, False), (1, 512, 68, 4, False, True),
+    (5, 1024, 260, 32, True, True), (1, 64, 4, 1, True, True), (1, 2048, 2044, 64, False, False)])
+def test_vector_path_is_bit_identical_to_scalar_path(oracle, bits, m, k, n, groups, bias, use_fma):
+    """fc_kernel's eight-channels-at-a-time path (AVX2 + F16C, used for the CPU baseline) against the
+    one-channel-at-a-time restatement: same bits, on unaligned shapes, odd slice counts, wide-range
+    scales (down to half's subnormals) and both dequantization forms."""
+    o = oracle
+    rng = np.random.default_rng(k * 7 + n + bits)
+    ks, ns = o.div_up(k, 4), o.div_up(n, 4)
+    lim = 127 if bits == 8 else 7
+    w = rng.integers(-lim - 1, lim + 1, size=(n, k), dtype=np.int8)
+    packed = (o.int8_as_uint8 if bits == 8 else o.int8_as_uint4)(w, o.LAYOUT_I4O4, ns)
+    act = o.f32_to_f16_bits(o.to_slices(rng.standard_normal((m, k)).astype(np.float32)))
+    sc = (rng.standard_normal((n, groups)) * np.exp2(rng.integers(-20, 3, size=(n, groups)))).astype(np.float32)
+    if groups == 1:
+        flat = np.zeros(ns * 4, np.float32); flat[:n] = sc[:, 0]
+        kind = o.SCALE_LINEAR
+    else:
+        flat = o.scale_to_hoio4(sc); kind = o.SCALE_BLOCK
+    flat = o.f32_to_f16_bits(flat)
+    b = o.f32_to_f16_bits(np.pad(rng.standard_normal(n).astype(np.float32), (0, ns * 4 - n))) if bias else None
+    try:
+        o.set_fast_path(False)
+        slow = o.fc_kernel(act, packed, m, k, n, o.PREC_F32F16, bits, kind, flat, None, b, groups, use_fma=use_fma)
+        assert o.last_fc_path == 0
+        o.set_fast_path(True)
+        fast = o.fc_kernel(act, packed, m, k, n, o.PREC_F32F16, bits, kind, flat, None, b, groups, use_fma=use_fma)
+        path = o.last_fc_path
+    finally:
+        o.set_fast_path(True)
+    if path != 1:
+        pytest.skip("this CPU has no AVX2 + FMA + F16C: the vector path was not taken")
+    assert np.array_equal(slow, fast)
+
+
+def test_vector_path_declines_what_it_cannot_state_exactly(oracle):
+    """A scale whose shift * scale leaves half's range (here 8 * 2^-24 is fine, 8 * 60000 overflows) and a
+    zero point both fall back to the scalar path."""
+    o = oracle
+    k, n = 64, 8
+    w = np.ones((n, k), np.int8)
+    packed = o.int8_as_uint4(w, o.LAYOUT_I4O4, 2)
+    act = o.f32_to_f16_bits(o.to_slices(np.ones((1, k), np.float32)))
+    big = o.f32_to_f16_bits(np.full(8, 60000.0, np.float32))
+    o.fc_kernel(act, packed, 1, k, n, o.PREC_F32F16, 4, o.SCALE_LINEAR, big)
+    assert o.last_fc_path == 0
+    ok = o.f32_to_f16_bits(np.full(8, 0.01, np.float32))
+    o.fc_kernel(act, packed, 1, k, n, o.PREC_F32F16, 4, o.SCALE_LINEAR, ok, zero_point=ok)
+    assert o.last_fc_path == 0
+    o.fc_kernel(act, packed, 1, k, n, o.PREC_F32, 4, o.SCALE_LINEAR, np.full(8, 0.01, np.float32))
+    assert o.last_fc_path == 0
