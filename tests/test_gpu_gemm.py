@@ -12,9 +12,17 @@ pytestmark = pytest.mark.gpu
 
 import mldhip as M
 import workloads as W
-from test_gpu_fc import check_fp, oracle_fc, textbook
+from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, textbook
 
 FP16_TOL = 2e-2
+
+
+def check_restatement(oracle, got, case, label):
+    """Against the oracle's restatement of the reference kernel: the stated tolerance, and no less
+    accurate (against float64) than that kernel itself."""
+    rest = oracle_fc(oracle, case).astype(np.float64)
+    check_fp(got, rest, case, label)
+    check_as_accurate_as(got, rest, textbook(case), case, label)
 
 
 def run_w4(case, reference_layout=None):
@@ -47,7 +55,7 @@ def test_w4_gemm_shapes(oracle, m, k, n, groups):
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
     if m * k * n <= 1 << 26:
-        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+        check_restatement(oracle, got, case, "kernel restatement")
 
 
 @pytest.mark.parametrize("m,k,n,groups", [(16, 256, 128, 8), (77, 1024, 200, 1), (128, 2048, 2048, 64)])
@@ -58,7 +66,7 @@ def test_w4_gemm_zero_points(oracle, m, k, n, groups):
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
     if m * k * n <= 1 << 26:
-        check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+        check_restatement(oracle, got, case, "kernel restatement")
 
 
 @pytest.mark.parametrize("m,k,n,groups,zp", [(2048, 64, 4096, 2, False), (2050, 96, 4000, 1, False),
@@ -71,7 +79,7 @@ def test_w4_gemm_wide_token_tile(oracle, m, k, n, groups, zp):
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
     sub = dict(case, m=64, act=case["act"][:64])
-    check_fp(got[:64], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement (first 64 tokens)")
+    check_restatement(oracle, got[:64], sub, "kernel restatement (first 64 tokens)")
 
 
 @pytest.mark.parametrize("m,k,n,groups,zp", [(16, 256, 128, 8, False), (5, 64, 8, 1, True), (128, 2048, 2048, 64, False),
@@ -88,7 +96,7 @@ def test_w8_gemm_shapes(oracle, m, k, n, groups, zp):
     small = min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
     if small * k * n <= 1 << 26:
-        check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+        check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
 @pytest.mark.parametrize("bits", [4, 8])
@@ -107,7 +115,7 @@ def test_gemm_fractional_zero_points(oracle, bits, m, k, n, groups):
     check_fp(got, textbook(case), case, "textbook")
     small = min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
-    check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+    check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
 @pytest.mark.parametrize("bits,m,k,n,groups,zp", [(4, 64, 512, 384, 4, False),    # 3 channel tiles: the last pair holds one
@@ -129,7 +137,7 @@ def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp):
     small = min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
     if small * k * n <= 1 << 26:
-        check_fp(got[:small], oracle_fc(oracle, sub).astype(np.float64), sub, "kernel restatement")
+        check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
 def test_gemm_modes_random_sweep():
