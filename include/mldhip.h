@@ -58,8 +58,12 @@ enum {
 enum {
   MLDHIP_PACKED_UINT8C4 = 1,
   MLDHIP_PACKED_INT8C4 = 2,
+  MLDHIP_PACKED_UINT8W4C4 = 3,
+  MLDHIP_PACKED_INT8W4C4 = 4,
   MLDHIP_PACKED_INT8C16 = 5,
-  MLDHIP_PACKED_UINT8C16 = 6
+  MLDHIP_PACKED_UINT8C16 = 6,
+  MLDHIP_PACKED_INT4C32 = 7,
+  MLDHIP_PACKED_UINT4C32 = 8
 };
 
 /* WeightsLayout, common/task/weights_layout.h:27-42 (same order) */
@@ -310,8 +314,16 @@ int mldhip_fc_batch_ids_create(const mldhip_fc_desc* desc, int weights_batch, in
 
 /* CreateQuantization (common/kernels/quantize_and_dequantize.h:57-73, .cc:693-842).
  * src 0 "src_tensor" [ceil(c/4)][tokens][4] (FLOAT16 or FLOAT32);
- * dst 0 "dst_tensor": codes, C4 types [ceil(c/4)][tokens][4] bytes, C16 types
- *       [ceil(c/16)][tokens][16] bytes;
+ * dst 0 "dst_tensor": codes, the tensor of GetShapeForPackedType (common/util.cc:262-277) as a
+ *       buffer (quantize_and_dequantize.cc:461-653); tokens = (y * w + x) * b + batch element:
+ *       C4   [ceil(c/4)][tokens][4] bytes;
+ *       C16  [ceil(c/16)][tokens][16] bytes (4 slices x 4 channels);
+ *       C32  [ceil(c/32)][tokens][16] bytes: 4-bit codes, channel j of the 32 in nibble j (low
+ *            nibble first, two's complement for INT4C32); code range 16 (scale abs_max / 7);
+ *       W4C4 [ceil(c/4)][h][ceil(w/4)][b][16] bytes: 4 columns x 4 channels, columns at or beyond
+ *            w repeat column w - 1 (set the shape with mldhip_op_set_shape);
+ *       slices that pad the last C16 / C32 group repeat the last slice, as in the reference's
+ *       kernel (they meet zero weights in the convolution);
  * dst 1 "dst_params": fp32 [tokens][4] = (inv_scale, offset, sum, 0), the BHWC(b,h,w,2|3)
  *       fp32 tensor the builder allocates (common/gpu_model_builder.cc:1285-1289). */
 typedef struct {

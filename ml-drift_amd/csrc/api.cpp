@@ -463,9 +463,8 @@ int mldhip_quantization_create(const mldhip_quant_desc* d, mldhip_op** out) {
   *out = nullptr;
   if (d->src_type != MLDHIP_FLOAT16 && d->src_type != MLDHIP_FLOAT32)
     return Fail(MLDHIP_INVALID_ARGUMENT, "source must be FLOAT16 or FLOAT32");
-  if (d->packed_type != MLDHIP_PACKED_UINT8C4 && d->packed_type != MLDHIP_PACKED_INT8C4 &&
-      d->packed_type != MLDHIP_PACKED_INT8C16 && d->packed_type != MLDHIP_PACKED_UINT8C16)
-    return Fail(MLDHIP_UNIMPLEMENTED, "packed type not supported");
+  if (d->packed_type < MLDHIP_PACKED_UINT8C4 || d->packed_type > MLDHIP_PACKED_UINT4C32)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "unknown packed type");
   if (d->channels <= 0 || d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad shape");
   mldhip_op* op = new (std::nothrow) mldhip_op();
   if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
@@ -590,9 +589,17 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
   } else if (op->kind == mldhip_op::kQuant) {
     const mldhip_quant_desc& d = op->q;
     const size_t s = DivUp(d.channels, 4);
-    const bool c16 = d.packed_type == MLDHIP_PACKED_INT8C16 || d.packed_type == MLDHIP_PACKED_UINT8C16;
     (*src)[0] = s * m * 4 * TypeBytes(d.src_type);
-    (*dst)[0] = c16 ? (size_t)DivUp((int)s, 4) * m * 16 : s * m * 4;
+    // GetShapeForPackedType (common/util.cc:262-277): 16 bytes per element of the packed tensor
+    switch (d.packed_type) {
+      case MLDHIP_PACKED_INT8C16:
+      case MLDHIP_PACKED_UINT8C16: (*dst)[0] = (size_t)DivUp((int)s, 4) * m * 16; break;
+      case MLDHIP_PACKED_INT4C32:
+      case MLDHIP_PACKED_UINT4C32: (*dst)[0] = (size_t)DivUp((int)s, 8) * m * 16; break;
+      case MLDHIP_PACKED_INT8W4C4:
+      case MLDHIP_PACKED_UINT8W4C4: (*dst)[0] = s * op->h * DivUp(op->w, 4) * op->b * 16; break;
+      default: (*dst)[0] = s * m * 4;
+    }
     (*dst)[1] = m * 4 * sizeof(float);
   } else {
     const mldhip_conv_int8_desc& d = op->cv;
@@ -736,6 +743,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     a.tokens = op->Tokens();
     a.channels = d.channels;
     a.batch = op->b;
+    a.width = op->w;
+    a.height = op->h;
     a.src_f16 = d.src_type == MLDHIP_FLOAT16;
     a.packed_type = d.packed_type;
     a.symmetric = d.symmetric != 0;

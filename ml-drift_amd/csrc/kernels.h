@@ -139,8 +139,9 @@ struct QuantArgs {
   void* codes = nullptr;
   float* params = nullptr;
   int tokens = 0, channels = 0, batch = 1;
+  int width = 1, height = 1;  // tokens = height * width * batch (the W4C4 types address by column)
   bool src_f16 = true;
-  int packed_type = 2;
+  int packed_type = 2;  // PackedType (common/data_type.h:48-58)
   bool symmetric = false;
   bool calculate_sum = false;
 };

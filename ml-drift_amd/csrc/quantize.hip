@@ -1,5 +1,5 @@
-// Dynamic per-token activation quantization for gfx950 (fp16/fp32 -> int8/uint8 codes plus
-// fp32 (inv_scale, offset, sum) per token), following the arithmetic of the reference's
+// Dynamic per-token activation quantization for gfx950 (fp16/fp32 -> 8-bit or 4-bit codes in the
+// C4, W4C4, C16 or C32 packing plus fp32 (inv_scale, offset, sum) per token), following the arithmetic of the reference's
 // generated kernel operation by operation: separate multiply and add (no fused
 // multiply-add), round half up through floor(x*scale + zp + 0.5) or truncation of
 // (x-min)*scale + 0.5.
@@ -31,8 +31,12 @@ struct QuantParams {
   uint8_t* codes;
   float* params;
   int tokens, channels, slices, batch;
-  int is_signed, c16, symmetric, calculate_sum;
+  int is_signed, layout, symmetric, calculate_sum;
+  int bits;           // 8, or 4 for the C32 types
+  int width, height;  // tokens = height * width * batch, token = (y * width + x) * batch + b
 };
+// where the codes of a token go
+enum : int { kCodesC4 = 0, kCodesC16 = 1, kCodesC32 = 2, kCodesW4C4 = 3 };
 
 template <typename SrcT>
 struct Raw;
@@ -71,13 +75,15 @@ __device__ __forceinline__ float RangeInSrcType(const float*, float mx, float mn
 template <bool SYM>
 struct Quantizer {
   float scale, min_value;
-  // The unsigned code of x as an integral float; the caller saturates it to [0, 255] while
-  // packing.  Asymmetric: truncation of a value >= 0.5, i.e. floor; a NaN (constant row:
-  // 0 * inf) becomes code 0.
+  float round_offset;  // symmetric: range / 2 + 0.5
+  float top;           // the largest code, range - 1
+  // The unsigned code of x as an integral float, at most `top`; the caller's conversion to a byte
+  // saturates it at 0.  Asymmetric: truncation of a value >= 0.5, i.e. floor; a NaN (constant
+  // row: 0 * inf) becomes code 0.
   __device__ __forceinline__ float Value(float x) const {
-    if (SYM) return floorf(Add(Mul(x, scale), 128.5f));
+    if (SYM) return fminf(floorf(Add(Mul(x, scale), round_offset)), top);
     const float f = floorf(Add(Mul(Sub(x, min_value), scale), 0.5f));
-    return f != f ? 0.0f : f;
+    return f != f ? 0.0f : fminf(f, top);
   }
 };
 
@@ -186,24 +192,31 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
   Quantizer<SYM> qz;
   qz.scale = 0.0f;
   qz.min_value = 0.0f;
-  const uint32_t sign_flip = p.is_signed ? 0x80808080u : 0u;  // u8 code - 128 as int8
-  const int code_shift = p.is_signed ? 128 : 0;
+  // code range: 256 values, or 16 for the 4-bit types
+  const int half_codes = p.bits == 4 ? 8 : 128;
+  const float zero_point = (float)half_codes, top = (float)(2 * half_codes - 1);
+  qz.round_offset = zero_point + 0.5f;
+  qz.top = top;
+  // unsigned code - range / 2 as a two's complement byte / nibble
+  const uint32_t sign_flip = !p.is_signed ? 0u : (p.bits == 4 ? 0x08080808u : 0x80808080u);
+  const uint32_t code_mask = p.bits == 4 ? 0x0F0F0F0Fu : 0xFFFFFFFFu;
+  const int code_shift = p.is_signed ? half_codes : 0;
   if (SYM) {
     const float abs_max = r0;
     if (abs_max > 0.0f) {
       const float min_scale = kHalf ? 6.103515625e-05f : 1.0e-30f;
-      inv_scale = fmaxf(min_scale, Div(abs_max, 127.0f));
-      if (!p.is_signed && kHalf) inv_scale = fminf(inv_scale, Div(65504.0f, 128.0f));
+      inv_scale = fmaxf(min_scale, Div(abs_max, zero_point - 1.0f));
+      if (!p.is_signed && kHalf) inv_scale = fminf(inv_scale, Div(65504.0f, zero_point));
       qz.scale = Div(1.0f, inv_scale);
-      if (!p.is_signed) offset = Mul(-inv_scale, 128.0f);
+      if (!p.is_signed) offset = Mul(-inv_scale, zero_point);
     }
   } else {
     qz.min_value = r0;
     const float src_range = RangeInSrcType(src, r1, r0);
     offset = qz.min_value;
-    qz.scale = Div(255.0f, src_range);
-    inv_scale = Div(src_range, 255.0f);
-    if (p.is_signed) offset = Add(offset, Mul(src_range, Div(128.0f, 255.0f)));
+    qz.scale = Div(top, src_range);
+    inv_scale = Div(src_range, top);
+    if (p.is_signed) offset = Add(offset, Mul(src_range, Div(zero_point, top)));
   }
 
   // pass 2: codes
@@ -217,13 +230,46 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
     for (int c = 0; c < 4; ++c) word = __builtin_amdgcn_cvt_pk_u8_f32(qz.Value(v[c]), c, word);
     const uint32_t valid = nvalid >= 4 ? 0xFFFFFFFFu : (1u << (8 * nvalid)) - 1u;
     sum = __builtin_amdgcn_udot4(word & valid, 0x01010101u, sum, false) - code_shift * nvalid;
-    return word ^ sign_flip;
+    return (word ^ sign_flip) & code_mask;
   };
+  // four bytes of 4-bit codes -> 16 bits, channel c in nibble c
+  auto nibbles = [](uint32_t w) -> uint32_t {
+    return (w & 0xFu) | ((w >> 4) & 0xF0u) | ((w >> 8) & 0xF00u) | ((w >> 12) & 0xF000u);
+  };
+  // W4C4: the token's column, row and batch element
+  int tb = 0, tx = 0, ty = 0;
+  if (p.layout == kCodesW4C4) {
+    tb = tok % p.batch;
+    tx = (tok / p.batch) % p.width;
+    ty = tok / (p.batch * p.width);
+  }
+  // packed[j]: the codes of slice 4 g + j; slices at or beyond the end hold the last slice's
   auto store_group = [&](int g, const uint32_t packed[4]) {
     if (!tok_ok) return;
-    if (p.c16) {
+    if (p.layout == kCodesC16) {
       *reinterpret_cast<uint4*>(p.codes + ((size_t)g * p.tokens + tok) * 16) =
           make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    } else if (p.layout == kCodesC32) {
+      const uint2 half = make_uint2(nibbles(packed[0]) | (nibbles(packed[1]) << 16),
+                                    nibbles(packed[2]) | (nibbles(packed[3]) << 16));
+      uint8_t* d = p.codes + ((size_t)(g >> 1) * p.tokens + tok) * 16;
+      *reinterpret_cast<uint2*>(d + (g & 1) * 8) = half;
+      if ((g & 1) == 0 && g == s16_count - 1) {  // no thread owns the upper half: the last slice again
+        const uint32_t last = nibbles(packed[3]) * 0x00010001u;
+        *reinterpret_cast<uint2*>(d + 8) = make_uint2(last, last);
+      }
+    } else if (p.layout == kCodesW4C4) {
+      const int w4 = (p.width + 3) / 4;
+      // this column, and the columns that pad the width to a multiple of 4 when it is the last one
+      const int x_end = tx == p.width - 1 ? w4 * 4 : tx + 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int s = g * 4 + j;
+        if (s >= p.slices) continue;
+        for (int x = tx; x < x_end; ++x)
+          *reinterpret_cast<uint32_t*>(p.codes + ((((size_t)s * p.height + ty) * w4 + x / 4) * p.batch + tb) * 16 +
+                                       (x % 4) * 4) = packed[j];
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -239,11 +285,7 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
     if (g < s16_count) {
       uint32_t packed[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int s = g * 4 + j;
-        const uint32_t word = encode4(cache[i][j], s);
-        packed[j] = s < p.slices ? word : 0u;
-      }
+      for (int j = 0; j < 4; ++j) packed[j] = encode4(cache[i][j], g * 4 + j);  // (the load clamped the slice)
       store_group(g, packed);
     }
   }
@@ -252,7 +294,7 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int s = g * 4 + j;
-      packed[j] = s < p.slices ? encode4(src4[(size_t)s * p.tokens + tok], s) : 0u;
+      packed[j] = encode4(src4[(size_t)min(s, p.slices - 1) * p.tokens + tok], s);
     }
     store_group(g, packed);
   }
@@ -303,8 +345,16 @@ hipError_t LaunchQuantize(const QuantArgs& a, hipStream_t stream, const char** k
   p.channels = a.channels;
   p.slices = DivUp(a.channels, 4);
   p.batch = a.batch;
-  p.is_signed = a.packed_type == 2 || a.packed_type == 5;
-  p.c16 = a.packed_type == 5 || a.packed_type == 6;
+  // PackedType: 1 uint8c4, 2 int8c4, 3 uint8w4c4, 4 int8w4c4, 5 int8c16, 6 uint8c16, 7 int4c32, 8 uint4c32
+  p.is_signed = a.packed_type == 2 || a.packed_type == 4 || a.packed_type == 5 || a.packed_type == 7;
+  p.layout = (a.packed_type == 5 || a.packed_type == 6)   ? kCodesC16
+             : (a.packed_type == 7 || a.packed_type == 8) ? kCodesC32
+             : (a.packed_type == 3 || a.packed_type == 4) ? kCodesW4C4
+                                                          : kCodesC4;
+  p.bits = p.layout == kCodesC32 ? 4 : 8;
+  p.width = a.width;
+  p.height = a.height;
+  if (p.layout == kCodesW4C4 && (long long)a.width * a.height * a.batch != a.tokens) return hipErrorInvalidValue;
   p.symmetric = a.symmetric;
   p.calculate_sum = a.calculate_sum;
   if (kernel_name) *kernel_name = "quantize_kernel";

@@ -15,6 +15,7 @@ OK, INVALID_ARGUMENT, FAILED_PRECONDITION, OUT_OF_RANGE, UNIMPLEMENTED, INTERNAL
 NOT_FOUND = 5
 FLOAT16, FLOAT32, UINT8, INT8, INT32, UINT4 = 1, 2, 5, 6, 10, 15
 PACKED_UINT8C4, PACKED_INT8C4, PACKED_INT8C16, PACKED_UINT8C16 = 1, 2, 5, 6
+PACKED_UINT8W4C4, PACKED_INT8W4C4, PACKED_INT4C32, PACKED_UINT4C32 = 3, 4, 7, 8
 LAYOUT_UNKNOWN, LAYOUT_I4O4, LAYOUT_O4I4, LAYOUT_2D_I4O4, LAYOUT_CUSTOM = 0, 1, 2, 6, 7
 PRECISION_F32, PRECISION_F32_F16, PRECISION_F16 = 0, 1, 2
 AXIS_O, AXIS_H, AXIS_W, AXIS_I = 0, 1, 2, 3

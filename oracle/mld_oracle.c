@@ -842,16 +842,35 @@ static inline int f2i_trunc(float v) { /* Convert<int4>: truncation; NaN -> 0 */
  * fp32 tensor the builder allocates (common/gpu_model_builder.cc:1285-1289), stored as
  * [tokens][4] = (inv_scale, offset, sum, 0).  `batch` is the tensor's B: the min/max
  * search of the asymmetric variant starts from the element (b, y=0, x=0, c=0) (:288).
- * codes: C4 types -> int8/uint8 [S][tokens][4]; C16 types -> [ceil(S/4)][tokens][16]. */
-void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const void* src,
-                   int packed_type, int symmetric, int calculate_sum, void* codes, float* params) {
+ * tokens are the flattened (y, x, b) index (y*W + x)*B + b.
+ * Code range (:757, 779-803): range = 2^bits (8-bit types 256, C32 types 16), dst_range = range-1,
+ * symmetric half range = range/2 - 1, zero point = range/2, rounding offset range/2 + 0.5, the
+ * unsigned cap kMaxHalf / (range/2), asymmetric middle (range/2)/(range-1).
+ * codes, as bytes in memory (:461-653, dst tensor of GetShapeForPackedType, common/util.cc:262-277,
+ * in buffer layout [slice][y][x][b][4 elements]):
+ *   C4   [S][tokens][4] one byte per channel;
+ *   W4C4 [S][H][ceil(W/4)][B][4 x][4 channels]: element (x/4, y, s) of an int32x4 tensor holds the
+ *        char4 of x, x+1, x+2, x+3; positions at or beyond W repeat column W-1 (x_clamped, :284);
+ *   C16  [ceil(S/4)][tokens][4 slices][4 channels];
+ *   C32  [ceil(S/8)][tokens][16 bytes]: channel j of the 32 in nibble j (two's complement for the
+ *        signed type), i.e. byte j/2, low nibble first;
+ *   slices at or beyond S inside the last C16 / C32 group repeat slice S-1 (s_clamped, :407). */
+void mldo_quantize_packed(int height, int width, int batch, int channels, int src_is_f16, const void* src,
+                          int packed_type, int symmetric, int calculate_sum, void* codes, float* params) {
+  const int tokens = height * width * batch;
   const int slices = div_up(channels, 4);
-  const int is_signed = packed_type == MLDO_PACKED_INT8C4 || packed_type == MLDO_PACKED_INT8C16;
+  const int is_signed = packed_type == MLDO_PACKED_INT8C4 || packed_type == MLDO_PACKED_INT8C16 ||
+                        packed_type == MLDO_PACKED_INT8W4C4 || packed_type == MLDO_PACKED_INT4C32;
   const int c16 = packed_type == MLDO_PACKED_INT8C16 || packed_type == MLDO_PACKED_UINT8C16;
-  const int dst_range = 255;
+  const int c32 = packed_type == MLDO_PACKED_INT4C32 || packed_type == MLDO_PACKED_UINT4C32;
+  const int w4 = packed_type == MLDO_PACKED_INT8W4C4 || packed_type == MLDO_PACKED_UINT8W4C4;
+  const int range = c32 ? 16 : 256;
+  const int dst_range = range - 1;
+  const float half_range = (float)(range / 2 - 1), zero_point = (float)(range / 2);
   const float kMinNormalHalf = 6.103515625e-05f, kMaxHalf = 65504.0f;
+  const int width4 = div_up(width, 4);
   uint8_t* out = (uint8_t*)codes;
-  if (c16) memset(out, 0, (size_t)div_up(slices, 4) * tokens * 16);
+  uint8_t* row = (uint8_t*)malloc((size_t)slices * 4); /* the token's codes, one byte per channel */
   for (int t = 0; t < tokens; ++t) {
     float inv_scale = 0.0f, scale = 0.0f, offset = 0.0f, min_value = 0.0f;
     if (symmetric) {
@@ -862,10 +881,10 @@ void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const vo
       }
       if (abs_max > 0.0f) { /* :363-377 */
         const float min_scale = src_is_f16 ? kMinNormalHalf : 1.0e-30f;
-        inv_scale = fmaxf(min_scale, abs_max / 127.0f);
-        if (!is_signed && src_is_f16) inv_scale = fminf(inv_scale, kMaxHalf / 128.0f);
+        inv_scale = fmaxf(min_scale, abs_max / half_range);
+        if (!is_signed && src_is_f16) inv_scale = fminf(inv_scale, kMaxHalf / zero_point);
         scale = 1.0f / inv_scale;
-        if (!is_signed) offset = -inv_scale * 128.0f;
+        if (!is_signed) offset = -inv_scale * zero_point;
       }
     } else {
       const int b = batch > 0 ? t % batch : 0;
@@ -881,7 +900,7 @@ void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const vo
       scale = (float)dst_range / src_range;
       inv_scale = src_range / (float)dst_range;
       if (is_signed) {
-        const float middle = 128.0f / 255.0f; /* :786-787 */
+        const float middle = zero_point / (float)dst_range; /* :786-787 */
         const float prod = src_range * middle;
         offset = offset + prod;
       }
@@ -893,7 +912,7 @@ void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const vo
         int q;
         if (symmetric) { /* :423-429 */
           float v = x * scale;
-          v = v + 128.5f;
+          v = v + (zero_point + 0.5f);
           v = floorf(v);
           v = fminf((float)dst_range, fmaxf(0.0f, v));
           q = f2i_trunc(v);
@@ -906,16 +925,46 @@ void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const vo
         }
         if (is_signed) q -= (dst_range + 1) / 2;
         if (calculate_sum && s * 4 + c < channels) sum += q; /* :442-459 */
-        const size_t idx = c16 ? ((size_t)(s / 4) * tokens + t) * 16 + (s % 4) * 4 + c
-                               : ((size_t)s * tokens + t) * 4 + c;
-        out[idx] = (uint8_t)q;
+        row[s * 4 + c] = (uint8_t)q;
       }
+    }
+    if (c16) {
+      for (int s = 0; s < div_up(slices, 4) * 4; ++s) {
+        const int sc = s < slices ? s : slices - 1;
+        memcpy(out + ((size_t)(s / 4) * tokens + t) * 16 + (s % 4) * 4, row + sc * 4, 4);
+      }
+    } else if (c32) {
+      for (int g = 0; g < div_up(slices, 8); ++g) {
+        uint8_t* d = out + ((size_t)g * tokens + t) * 16;
+        memset(d, 0, 16);
+        for (int j = 0; j < 32; ++j) {
+          const int s = g * 8 + j / 4, sc = s < slices ? s : slices - 1;
+          d[j / 2] |= (uint8_t)((row[sc * 4 + j % 4] & 15u) << (4 * (j & 1)));
+        }
+      }
+    } else if (w4) {
+      const int b = t % batch, x = (t / batch) % width, y = t / (batch * width);
+      for (int s = 0; s < slices; ++s) {
+        /* column x, and the columns beyond the width when x is the last one */
+        for (int xx = x; xx < (x == width - 1 ? width4 * 4 : x + 1); ++xx)
+          memcpy(out + ((((size_t)s * height + y) * width4 + xx / 4) * batch + b) * 16 + (xx % 4) * 4, row + s * 4, 4);
+      }
+    } else {
+      for (int s = 0; s < slices; ++s) memcpy(out + ((size_t)s * tokens + t) * 4, row + s * 4, 4);
     }
     params[(size_t)t * 4 + 0] = inv_scale;
     params[(size_t)t * 4 + 1] = offset;
     params[(size_t)t * 4 + 2] = calculate_sum ? (float)sum : 0.0f;
     params[(size_t)t * 4 + 3] = 0.0f;
   }
+  free(row);
+}
+
+void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const void* src,
+                   int packed_type, int symmetric, int calculate_sum, void* codes, float* params) {
+  const int b = batch > 0 ? batch : 1;
+  mldo_quantize_packed(1, tokens / b, b, channels, src_is_f16, src, packed_type, symmetric, calculate_sum, codes,
+                       params);
 }
 
 /* common/kernels/quantize_and_dequantize.cc:867-964 (CreateDequantization), fused after the

@@ -34,8 +34,12 @@ enum { MLDO_SCALE_SCALAR = 0, MLDO_SCALE_LINEAR = 1, MLDO_SCALE_BLOCK = 2 };
 enum {
   MLDO_PACKED_UINT8C4 = 1,
   MLDO_PACKED_INT8C4 = 2,
+  MLDO_PACKED_UINT8W4C4 = 3,
+  MLDO_PACKED_INT8W4C4 = 4,
   MLDO_PACKED_INT8C16 = 5,
-  MLDO_PACKED_UINT8C16 = 6
+  MLDO_PACKED_UINT8C16 = 6,
+  MLDO_PACKED_INT4C32 = 7,
+  MLDO_PACKED_UINT4C32 = 8
 };
 enum { MLDO_AXIS_O = 0, MLDO_AXIS_H = 1, MLDO_AXIS_W = 2, MLDO_AXIS_I = 3 };
 
@@ -107,6 +111,10 @@ void mldo_make_weights_from_int8(int n, int k, const int8_t* w, const float* sca
 void mldo_quantize(int tokens, int channels, int batch, int src_is_f16, const void* src,
                    int packed_type, int symmetric, int calculate_sum, void* codes,
                    float* params);
+/* every packed type; the tensor is BHWC(batch, height, width, channels), tokens = (y*W + x)*B + b */
+void mldo_quantize_packed(int height, int width, int batch, int channels, int src_is_f16,
+                          const void* src, int packed_type, int symmetric, int calculate_sum,
+                          void* codes, float* params);
 void mldo_dequantize(int tokens, int n, int k, const int32_t* acc, const float* params,
                      const int32_t* weights_sum, const float* weights_scale,
                      const float* weights_zero_point, const void* bias, int dst_is_f16,

@@ -18,6 +18,7 @@ LAYOUT_2D_I4O4 = 6
 PREC_F32, PREC_F32F16, PREC_F16 = 0, 1, 2
 SCALE_SCALAR, SCALE_LINEAR, SCALE_BLOCK = 0, 1, 2
 PACKED_UINT8C4, PACKED_INT8C4, PACKED_INT8C16, PACKED_UINT8C16 = 1, 2, 5, 6
+PACKED_UINT8W4C4, PACKED_INT8W4C4, PACKED_INT4C32, PACKED_UINT4C32 = 3, 4, 7, 8
 AXIS_O, AXIS_H, AXIS_W, AXIS_I = 0, 1, 2, 3
 
 
@@ -390,21 +391,29 @@ def make_weights_from_int8(w, scale, zero_point=None):
 
 # ---- quantization ----
 def quantize(src_slices, tokens, channels, packed_type=PACKED_INT8C4, symmetric=False,
-             calculate_sum=False, batch=1):
+             calculate_sum=False, batch=1, height=1):
+    """tokens = height * width * batch, flattened as (y * width + x) * batch + b.  Returns (codes,
+    params): codes as bytes, C4 [S][tokens][4]; C16 [ceil(S/4)][tokens][16]; C32 (4-bit codes,
+    uint8 bytes of two nibbles) [ceil(S/8)][tokens][16]; W4C4 [S][height][ceil(width/4)][batch][16]."""
     src = np.ascontiguousarray(src_slices)
     is_f16 = src.dtype == np.uint16
     assert is_f16 or src.dtype == np.float32
     slices = div_up(channels, 4)
-    assert src.size == slices * tokens * 4
-    signed = packed_type in (PACKED_INT8C4, PACKED_INT8C16)
+    assert src.size == slices * tokens * 4 and tokens % (batch * height) == 0
+    width = tokens // (batch * height)
+    signed = packed_type in (PACKED_INT8C4, PACKED_INT8C16, PACKED_INT8W4C4)
     cdt = np.int8 if signed else np.uint8
     if packed_type in (PACKED_INT8C16, PACKED_UINT8C16):
         codes = np.empty((div_up(slices, 4), tokens, 16), cdt)
+    elif packed_type in (PACKED_INT4C32, PACKED_UINT4C32):
+        codes = np.empty((div_up(slices, 8), tokens, 16), np.uint8)
+    elif packed_type in (PACKED_INT8W4C4, PACKED_UINT8W4C4):
+        codes = np.empty((slices, height, div_up(width, 4), batch, 16), cdt)
     else:
         codes = np.empty((slices, tokens, 4), cdt)
     params = np.empty((tokens, 4), np.float32)
-    lib().mldo_quantize(tokens, channels, batch, int(is_f16), _p(src), packed_type,
-                        int(symmetric), int(calculate_sum), _p(codes), _p(params))
+    lib().mldo_quantize_packed(height, width, batch, channels, int(is_f16), _p(src), packed_type,
+                               int(symmetric), int(calculate_sum), _p(codes), _p(params))
     return codes, params
 
 

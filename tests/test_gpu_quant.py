@@ -8,21 +8,29 @@ import mldhip as M
 import workloads as W
 
 
-def run_quant(src_slices_np, tokens, channels, packed_type, symmetric, calc_sum, batch=1):
+def run_quant(src_slices_np, tokens, channels, packed_type, symmetric, calc_sum, batch=1, height=1):
     import torch
     f16 = src_slices_np.dtype == np.float16
     src = torch.from_numpy(src_slices_np).cuda()
     slices = (channels + 3) // 4
-    c16 = packed_type in (M.PACKED_INT8C16, M.PACKED_UINT8C16)
-    shape = ((slices + 3) // 4, tokens, 16) if c16 else (slices, tokens, 4)
-    signed = packed_type in (M.PACKED_INT8C4, M.PACKED_INT8C16)
-    codes = torch.zeros(shape, dtype=torch.int8 if signed else torch.uint8, device="cuda")
+    width = tokens // (batch * height)
+    signed = packed_type in (M.PACKED_INT8C4, M.PACKED_INT8C16, M.PACKED_INT8W4C4)
+    if packed_type in (M.PACKED_INT8C16, M.PACKED_UINT8C16):
+        shape = ((slices + 3) // 4, tokens, 16)
+    elif packed_type in (M.PACKED_INT4C32, M.PACKED_UINT4C32):
+        shape = ((slices + 7) // 8, tokens, 16)
+    elif packed_type in (M.PACKED_INT8W4C4, M.PACKED_UINT8W4C4):
+        shape = (slices, height, (width + 3) // 4, batch, 16)
+    else:
+        shape = (slices, tokens, 4)
+    # a fill no code path leaves behind: every byte of the packed tensor must be written
+    codes = torch.full(shape, 0x5A, dtype=torch.int8 if signed else torch.uint8, device="cuda")
     params = torch.zeros((tokens, 4), dtype=torch.float32, device="cuda")
     op = M.quantization_create(M.FLOAT16 if f16 else M.FLOAT32, packed_type, channels, calc_sum,
                                symmetric, max_tokens=tokens)
     op.bind([src], [codes, params])
-    op.set_shape(batch, 1, tokens // batch)
-    print("quant", tokens, channels, packed_type, symmetric, calc_sum, flush=True)
+    op.set_shape(batch, height, width)
+    print("quant", tokens, channels, packed_type, symmetric, calc_sum, batch, height, flush=True)
     op.launch(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert op.kernel_name == "quantize_kernel"
@@ -50,7 +58,8 @@ def edge_tensor(rng, tokens, channels):
 
 @pytest.mark.parametrize("tokens,channels", [(13 * 15, 237), (35, 64), (5, 2048), (1, 16)])
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
-@pytest.mark.parametrize("packed_type", [M.PACKED_INT8C4, M.PACKED_UINT8C4, M.PACKED_INT8C16, M.PACKED_UINT8C16])
+@pytest.mark.parametrize("packed_type", [M.PACKED_INT8C4, M.PACKED_UINT8C4, M.PACKED_INT8C16, M.PACKED_UINT8C16,
+                                         M.PACKED_INT4C32, M.PACKED_UINT4C32, M.PACKED_INT8W4C4, M.PACKED_UINT8W4C4])
 @pytest.mark.parametrize("symmetric", [True, False])
 def test_quantize_bit_exact(oracle, tokens, channels, dtype, packed_type, symmetric):
     rng = np.random.default_rng(tokens + channels)
@@ -106,3 +115,32 @@ def test_symmetric_literal_tie_vector_on_gpu(dtype):
     codes, params = run_quant(src, 1, 8, M.PACKED_INT8C4, True, True)
     assert params[0, 0] == 1.0 and params[0, 1] == 0.0 and params[0, 2] == LITERAL_TIE_CODES.sum()
     assert np.array_equal(W.from_slices(codes, 8).astype(np.int32)[0], LITERAL_TIE_CODES)
+
+
+@pytest.mark.parametrize("packed_type", [M.PACKED_INT8W4C4, M.PACKED_UINT8W4C4, M.PACKED_INT4C32, M.PACKED_INT8C16])
+@pytest.mark.parametrize("b,h,w,c", [(1, 3, 7, 24), (3, 2, 5, 44), (2, 1, 1, 100), (1, 13, 15, 237), (4, 1, 64, 2048)])
+def test_packed_outputs_with_height_width_batch(oracle, packed_type, b, h, w, c):
+    """The packed tensors on BHWC shapes: W4C4 addresses by column (widths that are not multiples of 4
+    repeat the last column), C16 / C32 groups that the channels do not fill repeat the last slice."""
+    tokens = b * h * w
+    rng = np.random.default_rng(b * 1000 + h * 100 + w + c)
+    x = edge_tensor(rng, tokens, c)
+    src = W.to_slices(x).astype(np.float16)
+    osrc = oracle.f32_to_f16_bits(src.astype(np.float32))
+    for symmetric in (True, False):
+        codes, params = run_quant(src, tokens, c, packed_type, symmetric, True, batch=b, height=h)
+        rcodes, rparams = oracle.quantize(osrc, tokens, c, packed_type, symmetric, True, batch=b, height=h)
+        assert np.array_equal(params.view(np.uint32), rparams.view(np.uint32))
+        assert codes.shape == rcodes.shape and np.array_equal(codes.view(np.uint8), rcodes.view(np.uint8))
+
+
+def test_int4_literal_bytes_on_gpu():
+    """The hand-computed 4-bit vector of the oracle's tests, straight through the C-ABI."""
+    row = np.array([7.0, -7.0, 3.5, 0.5, -0.5, -3.5, 6.49, 0.0], np.float32)
+    src = W.to_slices(row[None]).astype(np.float16)
+    codes, params = run_quant(src, 1, 8, M.PACKED_INT4C32, True, True)
+    assert codes.tobytes() == bytes([0x97, 0x14, 0xD0, 0x06] + [0xD0, 0x06] * 6)
+    assert params[0].tolist() == [1.0, 0.0, 8.0, 0.0]
+    codes, params = run_quant(src, 1, 8, M.PACKED_UINT4C32, True, False)
+    assert codes.tobytes() == bytes([0x1F, 0x9C, 0x58, 0x8E] + [0x58, 0x8E] * 6)
+    assert params[0].tolist() == [1.0, -8.0, 0.0, 0.0]

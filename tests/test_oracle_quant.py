@@ -197,3 +197,133 @@ def test_symmetric_literal_tie_vector(oracle, f16):
     codes_u, params_u = o.quantize(src, 1, 8, o.PACKED_UINT8C4, symmetric=True)
     assert np.array_equal(o.from_slices(codes_u, 8).astype(np.int32)[0], LITERAL_TIE_CODES + 128)
     assert params_u[0, 0] == 1.0 and params_u[0, 1] == -128.0
+
+
+# ---- packed outputs beyond C4 / C16: 4-bit codes (C32) and four columns per element (W4C4) ----
+# hand-computed: abs_max 7 -> inv_scale 7 / 7 = 1; code = clamp(floor(x + 8.5), 0, 15) (- 8 signed)
+INT4_ROW = np.array([7.0, -7.0, 3.5, 0.5, -0.5, -3.5, 6.49, 0.0], np.float32)
+INT4_CODES = np.array([7, -7, 4, 1, 0, -3, 6, 0], np.int32)
+# nibble j of the 16 bytes = channel j, two's complement, low nibble first; the 8 channels are two
+# slices, the six slices that complete the group of 32 channels repeat the last one
+INT4_BYTES = bytes([0x97, 0x14, 0xD0, 0x06] + [0xD0, 0x06] * 6)
+UINT4_BYTES = bytes([0x1F, 0x9C, 0x58, 0x8E] + [0x58, 0x8E] * 6)
+
+
+def unpack_c32(codes, channels, signed):
+    """[G][tokens][16] bytes -> [tokens][channels] integer codes."""
+    g, tokens, _ = codes.shape
+    b = codes.astype(np.int32)
+    nib = np.stack([b & 15, b >> 4], axis=-1).reshape(g, tokens, 32)
+    flat = nib.transpose(1, 0, 2).reshape(tokens, g * 32)[:, :channels]
+    return np.where(flat >= 8, flat - 16, flat) if signed else flat
+
+
+@pytest.mark.parametrize("f16", [True, False])
+def test_int4_symmetric_literal(oracle, f16):
+    o = oracle
+    src = o.to_slices(INT4_ROW[None])
+    src = o.f32_to_f16_bits(src) if f16 else src   # 6.49 rounds to 6.4883 in half: same code
+    codes, params = o.quantize(src, 1, 8, o.PACKED_INT4C32, symmetric=True, calculate_sum=True)
+    assert codes.shape == (1, 1, 16) and codes.tobytes() == INT4_BYTES
+    assert params[0].tolist() == [1.0, 0.0, float(INT4_CODES.sum()), 0.0]
+    assert np.array_equal(unpack_c32(codes, 8, True)[0], INT4_CODES)
+    codes_u, params_u = o.quantize(src, 1, 8, o.PACKED_UINT4C32, symmetric=True)
+    assert codes_u.tobytes() == UINT4_BYTES
+    assert params_u[0, 0] == 1.0 and params_u[0, 1] == -8.0   # offset = -inv_scale * 8
+
+
+def test_int4_asymmetric_literal(oracle):
+    # [0, 15]: range 15, scale 15 / 15 = 1, code = trunc(x + 0.5): 7.4 -> 7, 7.6 -> 8
+    o = oracle
+    x = np.array([[0.0, 15.0, 7.4, 7.6]], np.float32)
+    codes, params = o.quantize(o.to_slices(x), 1, 4, o.PACKED_UINT4C32, calculate_sum=True)
+    assert unpack_c32(codes, 4, False)[0].tolist() == [0, 15, 7, 8]
+    assert params[0].tolist() == [1.0, 0.0, 30.0, 0.0]
+    codes, params = o.quantize(o.to_slices(x), 1, 4, o.PACKED_INT4C32, calculate_sum=True)
+    assert unpack_c32(codes, 4, True)[0].tolist() == [-8, 7, -1, 0]
+    # signed offset = min + range * (8 / 15), quantize_and_dequantize.cc:397-399, 786-787
+    assert params[0, 0] == 1.0 and params[0, 1] == np.float32(15.0) * (np.float32(8.0) / np.float32(15.0))
+    assert params[0, 2] == -2.0
+
+
+@pytest.mark.parametrize("signed", [True, False])
+@pytest.mark.parametrize("f16", [True, False])
+@pytest.mark.parametrize("c", [237, 64, 20])
+def test_int4_symmetric_contract_and_padding(oracle, signed, f16, c):
+    """4-bit codes on the reference's symmetric test tensor: the dequantization contract
+    x ~= q * inv_scale + offset within 0.51 step (tests/quantize_and_dequantize_test_util.cc:611-616),
+    the all-zero row (params 0, mid-point codes, :708-714), inv_scale = abs_max / 7 and the slices that
+    pad the last group of 32 channels."""
+    o = oracle
+    h, w = 5, 7
+    x = symmetric_test_tensor(np.random.default_rng(c), h, w, c)
+    tokens = h * w
+    src = o.to_slices(x)
+    src = o.f32_to_f16_bits(src) if f16 else src
+    codes, params = o.quantize(src, tokens, c, o.PACKED_INT4C32 if signed else o.PACKED_UINT4C32, symmetric=True,
+                               calculate_sum=True)
+    q = unpack_c32(codes, c, signed)
+    lo, hi = (-8, 7) if signed else (0, 15)
+    assert q.min() >= lo and q.max() <= hi
+    for t in range(tokens):
+        abs_max = np.abs(x[t]).max()
+        if abs_max == 0:
+            assert params[t, 0] == 0 and params[t, 1] == 0 and np.all(q[t] == (0 if signed else 8))
+            continue
+        inv = np.float32(abs_max) / np.float32(7)
+        if f16 and not signed:
+            inv = min(inv, np.float32(K_MAX_HALF / 8))
+        assert params[t, 0] == inv and params[t, 2] == q[t].sum()
+        deq = q[t] * params[t, 0] + params[t, 1]
+        expect = np.minimum(x[t], hi * params[t, 0] + params[t, 1])
+        assert np.all(np.abs(deq - expect) <= 0.51 * params[t, 0])
+    # padding: channels c .. 4*slices-1 are the codes of 0.0, slices beyond the last repeat it
+    slices = (c + 3) // 4
+    full = unpack_c32(codes, codes.shape[0] * 32, signed)
+    last = full[:, (slices - 1) * 4: slices * 4]
+    for s in range(slices, codes.shape[0] * 8):
+        assert np.array_equal(full[:, s * 4: s * 4 + 4], last)
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_c32_and_c16_hold_the_c4_codes_of_a_narrower_range(oracle, symmetric):
+    """Layout only: the 8-bit C16 bytes against the C4 bytes (slice s of group s / 4 at byte 4 * (s % 4),
+    the host-side packing of the reference's int8 convolution test, conv_generic_test_util.cc:1176-1200),
+    including the repeated last slice."""
+    o = oracle
+    rng = np.random.default_rng(5)
+    tokens, c = 6, 44   # 11 slices: the last C16 group holds 3 slices + 1 repeat
+    x = rng.standard_normal((tokens, c)).astype(np.float32)
+    src = o.to_slices(x)
+    c4, p4 = o.quantize(src, tokens, c, o.PACKED_INT8C4, symmetric=symmetric)
+    c16, p16 = o.quantize(src, tokens, c, o.PACKED_INT8C16, symmetric=symmetric)
+    assert np.array_equal(p4, p16)
+    for s in range(12):
+        assert np.array_equal(c16[s // 4, :, (s % 4) * 4:(s % 4) * 4 + 4], c4[min(s, 10)])
+
+
+@pytest.mark.parametrize("signed", [True, False])
+@pytest.mark.parametrize("h,w,b", [(1, 8, 1), (3, 7, 1), (2, 5, 3), (1, 1, 2)])
+def test_w4c4_layout(oracle, signed, h, w, b):
+    """W4C4: element (x / 4, y, s) of the int32x4 tensor holds the four char4 of columns x..x+3
+    (quantize_and_dequantize.cc:461-483).  With batch 1 and a width that is a multiple of 4 the bytes are
+    those of the C4 tensor (how the reference's convolution test uploads one as the other,
+    conv_generic_test_util.cc:1168-1175); columns beyond the width repeat the last one; with a batch
+    the four columns of one batch element sit together."""
+    o = oracle
+    c = 24
+    tokens = h * w * b
+    rng = np.random.default_rng(h * 100 + w * 10 + b)
+    x = rng.standard_normal((tokens, c)).astype(np.float32)
+    src = o.to_slices(x)
+    p_c4, p_w4 = (o.PACKED_INT8C4, o.PACKED_INT8W4C4) if signed else (o.PACKED_UINT8C4, o.PACKED_UINT8W4C4)
+    c4, params4 = o.quantize(src, tokens, c, p_c4, calculate_sum=True, batch=b, height=h)
+    w4, params = o.quantize(src, tokens, c, p_w4, calculate_sum=True, batch=b, height=h)
+    assert np.array_equal(params, params4)
+    assert w4.shape == (6, h, (w + 3) // 4, b, 16)
+    if b == 1 and w % 4 == 0:
+        assert w4.tobytes() == c4.tobytes()
+    c4 = c4.reshape(6, h, w, b, 4)
+    for xx in range(4 * ((w + 3) // 4)):
+        got = w4[:, :, xx // 4, :, (xx % 4) * 4:(xx % 4) * 4 + 4]
+        assert np.array_equal(got, c4[:, :, min(xx, w - 1)]), xx
