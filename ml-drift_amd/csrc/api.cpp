@@ -370,9 +370,11 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   }
   {
     const int ns = DivUp(d->o, 4);
-    const bool native = wd.type == MLDHIP_UINT4 && IsNativeGroup(wd.output_group_size) && d->o % 4 == 0 &&
-                        ns % wd.output_group_size == 0 && !batch_ids;
-    if (wd.output_group_size != ns && !native)
+    // One output group is the layout of FullyConnected (fully_connected.cc:1073-1086); groups of one
+    // slice are the layout FullyConnectedOI reads (linear_i4o4 = dst_s * src_slices + src_s,
+    // fully_connected_oi.cc:122-133); any other whole number of groups is addressed the same way.
+    const bool whole_groups = wd.output_group_size > 0 && ns % wd.output_group_size == 0 && !batch_ids;
+    if (wd.output_group_size != ns && !whole_groups)
       return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
   }
   if (d->precision < MLDHIP_PRECISION_F32 || d->precision > MLDHIP_PRECISION_F16)
@@ -702,7 +704,9 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       const int8_t* act = static_cast<const int8_t*>(op->src_ptr[0]);
       const uint8_t* weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
       int32_t* dst = static_cast<int32_t*>(op->dst_ptr[0]);
-      if (GetTuning().force_generic <= 0 && op->idx_params < 0 && FcInt8MathStreamSupported(tokens, d.i, d.o, bits))
+      const int group = EffectiveGroup(batch.group, DivUp(d.o, 4));
+      if (GetTuning().force_generic <= 0 && op->idx_params < 0 && FcInt8MathStreamSupported(tokens, d.i, d.o, bits) &&
+          (bits == 8 || group % 2 == 0))
         e = LaunchFcInt8MathStream(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
       else
         e = LaunchFcInt8Math(act, weights, dst, tokens, d.i, d.o, bits, stream, &op->last_kernel, batch);
@@ -722,7 +726,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       } else
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
       // on the vector-ALU kernel; the tuning knob gemv_mfma = 1 forces the matrix-core one there too)
-      if (!force_generic && (a.m >= 2 || GetTuning().gemv_mfma > 0) && FcW4MfmaStreamSupported(a)) {
+      if (!force_generic && (a.m >= 2 || GetTuning().gemv_mfma > 0 || !FcW4StreamSupported(a)) &&
+          FcW4MfmaStreamSupported(a)) {
         e = LaunchFcW4MfmaStream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4StreamSupported(a)) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);

@@ -896,6 +896,8 @@ bool FcW4StreamSupported(const FcArgs& a) {
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   const int ks = DivUp(a.k, 4), ns = DivUp(a.n, 4);
   if (ns % 2 != 0) return false;  // 16-byte loads need an even number of 8-byte blocks per row
+  const int group = EffectiveGroup(a.group, ns);
+  if (ns % group != 0 || group % 2 != 0) return false;  // ... per row of one output group
   if (a.scale_kind == kScaleScalar) return false;
   if (a.scale_kind == kScaleBlock) {
     if (a.groups <= 0 || ks % a.groups != 0) return false;

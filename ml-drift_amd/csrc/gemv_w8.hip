@@ -242,6 +242,7 @@ hipError_t LaunchT(const W8Params& p, int lpr, int waves, hipStream_t stream) {
 
 bool FcW8StreamSupported(const FcArgs& a) {
   if (a.weight_bits != 8 || a.act_f16 != a.dst_f16) return false;
+  if (EffectiveGroup(a.group, DivUp(a.n, 4)) != DivUp(a.n, 4)) return false;  // one output group only
   if (a.m < 1 || a.m > kGemvMaxTokens) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   if (a.scale_kind == kScaleScalar) return false;

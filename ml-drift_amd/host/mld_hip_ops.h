@@ -7,6 +7,7 @@
 //   ExternalWeights                            common/task/gpu_operation.h:354-363
 //   CreateFullyConnectedExternalWeights        common/kernels/fully_connected.h:155-161
 //   CreateFullyConnectedWeightsBatchIds        common/kernels/fully_connected.cc:1174-1216
+//   CreateFullyConnectedOI                     common/kernels/fully_connected_oi.h:80-86
 //   CreateQuantization                         common/kernels/quantize_and_dequantize.h:68-73
 //   ClOperation::{SetSrcTensor, SetDstTensor, UpdateParams, AddToQueue}   cl/cl_operation.h:44-129
 //   GpuModelBuilder::FullyConnectedInt4/8ExternalWeights (dispatcher)     common/gpu_model_builder.cc:1548-1725
@@ -39,7 +40,9 @@ struct BHWC {
 };
 enum class CalculationsPrecision { kF32 = 0, kF32F16 = 1, kF16 = 2 };
 enum class DataType { kFloat16 = 1, kFloat32 = 2, kUint8 = 5, kInt8 = 6, kInt32 = 10, kUint4 = 15 };
-enum class PackedType { kUint8C4 = 1, kInt8C4 = 2, kInt8C16 = 5, kUint8C16 = 6 };
+enum class PackedType {  // common/data_type.h:48-58
+  kUint8C4 = 1, kInt8C4 = 2, kUint8W4C4 = 3, kInt8W4C4 = 4, kInt8C16 = 5, kUint8C16 = 6, kInt4C32 = 7, kUint4C32 = 8
+};
 
 using WeightsDescription = mldhip_weights_desc;
 
@@ -185,6 +188,19 @@ inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precisio
   if (rc != MLDHIP_OK) return Status::FromCode(rc);
   *result = HipOperation(op);
   return {};
+}
+
+// CreateFullyConnectedOI (common/kernels/fully_connected_oi.cc:530-583): the FullyConnected over
+// weights with the output slice outermost, linear_i4o4 = dst_s * src_slices + src_s (:122-133),
+// which is kOSpatialIOGroupI4O4 with output_group_size = 1 (what the reference's tests pass,
+// tests/fully_connected_oi_test_util.cc:109-111, 256-258).  Same objects and arithmetic as
+// CreateFullyConnectedExternalWeights; a description with another group size is refused here.
+inline Status CreateFullyConnectedOI(CalculationsPrecision precision, DataType src_type, DataType dst_type,
+                                     const ExternalWeights& weights, bool has_bias, int max_tokens,
+                                     HipOperation* result, const ConvRuntimeCheckDesc& runtime_check = {}) {
+  if (weights.desc.output_group_size != 1) return Status::FromCode(MLDHIP_INVALID_ARGUMENT);
+  return CreateFullyConnectedExternalWeights(precision, src_type, dst_type, weights, has_bias, max_tokens, result,
+                                             runtime_check);
 }
 
 inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,

@@ -57,14 +57,19 @@ def make_fc_case(seed, m, k, n, weight_bits, tensor_dtype, groups=1, with_bias=F
     return case
 
 
-def pack_fc_weights(case, reference_layout=False):
+def pack_fc_weights(case, reference_layout=False, output_group=None):
     """Packs the case's weights for the FullyConnected op: in the layout the library asks for, or
-    with `reference_layout` in the reference's own FullyConnected layout (one output group)."""
+    with `reference_layout` in the reference's own FullyConnected layout (one output group), or
+    in output groups of `output_group` slices (1: the layout FullyConnectedOI reads)."""
     n, k = case["n"], case["k"]
     if case["weight_bits"] == 4:
-        desc = M.fc_int4_weights_desc(n, k, reference=reference_layout)
+        desc = M.fc_int4_weights_desc(n, k, reference=reference_layout or output_group is not None)
+        if output_group is not None:
+            desc.output_group_size = output_group
         return desc, M.rearrange_int8_as_uint4(case["w"], desc)
     desc = M.fc_int8_weights_desc(n, k)
+    if output_group is not None:
+        desc.output_group_size = output_group
     return desc, M.rearrange_int8_as_uint8(case["w"], desc)
 
 
@@ -75,14 +80,15 @@ def mld_type(np_dtype):
 class FcDevice:
     """An FC op with its device buffers (torch tensors) for one synthetic case."""
 
-    def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None, reference_layout=False):
+    def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None, reference_layout=False,
+                 output_group=None):
         import torch
         self.torch = torch
         self.case = case
         m, k, n = case["m"], case["k"], case["n"]
         td = case["tensor_dtype"]
         tt = torch.float16 if td == np.float16 else torch.float32
-        self.desc, packed = pack_fc_weights(case, reference_layout)
+        self.desc, packed = pack_fc_weights(case, reference_layout, output_group)
         self.packed_host = packed
         self.weights = torch.from_numpy(packed).to(device)
         self.act = torch.from_numpy(to_slices(case["act"]).astype(td)).to(device)

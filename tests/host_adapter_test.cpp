@@ -53,7 +53,7 @@ int main() {
   EXPECT(fc.UpdateParams(BHWC{1, 1, 5, 4096}).code == MLDHIP_OUT_OF_RANGE);
   EXPECT(fc.AddToQueue(nullptr).code == MLDHIP_FAILED_PRECONDITION);  // nothing bound: refused before any GPU call
 
-  w.desc.output_group_size = 7;
+  w.desc.output_group_size = 5;  // does not divide the slices
   HipOperation bad;
   st = CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
                                            false, 1, &bad);
@@ -76,6 +76,19 @@ int main() {
   st = CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
                                            false, 1, &ringed, rc_desc);
   EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !ringed.valid());
+
+  // FullyConnectedOI: the same op over output groups of one slice (fully_connected_oi_test_util.cc:109-111)
+  ExternalWeights woi = w;
+  woi.desc.output_group_size = 1;
+  HipOperation oi;
+  EXPECT(CreateFullyConnectedOI(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, woi,
+                                /*has_bias=*/true, 4, &oi)
+             .ok());
+  names = oi.GetSrcTensorsNames();
+  EXPECT(names.size() == 4 && names[1] == "weights" && names[3] == "biases");
+  HipOperation not_oi;
+  EXPECT(CreateFullyConnectedOI(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w, true, 4, &not_oi)
+             .code == MLDHIP_INVALID_ARGUMENT);
 
   // the mixture-of-experts FullyConnected: fully_connected.cc:1203-1213 registers batch_ids before the weights
   ExternalWeights we;
