@@ -291,6 +291,17 @@ typedef struct {
   int32_t has_runtime_check;
   int32_t src_end_ch_index, dst_end_ch_index;
   int32_t ring_o_offset_index, ring_i_offset_index, ring_size;
+  /* ConvRuntimeCheckDesc::PackedGroups (common/task/gpu_operation.h:396-406), read when
+   * has_runtime_check != 0 and packed_num_groups > 0: the grouped FullyConnected of a
+   * mixture-of-experts prefill (MakeConvWithPackedGroups, common/gpu_model_builder_moe_util.cc:119-230).
+   * ExternalWeights::shape = OHWI(o, packed_num_groups, 1, i): the matrices packed one after the other
+   * in the one-group layout, scales [scale_i][packed_num_groups][ceil(o/4)][4], as for
+   * mldhip_fc_batch_ids_create.  The source is one row of tokens sorted by matrix; matrix g multiplies
+   * the params[packed_params_offset + g] tokens that start at token
+   * params[packed_params_offset + packed_num_groups + g] (fully_connected_util.cc:263-277), at most
+   * packed_max_group_size of them; dst tokens that belong to no group are not written.  "params" is
+   * the last src object; mldhip_op_set_shape(op, 1, 1, tokens). */
+  int32_t packed_params_offset, packed_num_groups, packed_max_group_size;
 } mldhip_fc_desc;
 
 int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);

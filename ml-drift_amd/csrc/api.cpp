@@ -398,7 +398,7 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     if (d->has_zero_point_tensor && d->scale_o * d->scale_i == 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "a zero-point tensor needs a scale tensor of the same shape");
   }
-  bool runtime_bounds = false;
+  bool runtime_bounds = false, packed_groups = false;
   if (d->has_runtime_check) {
     // ringed weights: refused as the reference refuses them for these weights (fully_connected.cc:1087-1097)
     if (d->ring_o_offset_index >= 0 || d->ring_i_offset_index >= 0) {
@@ -409,12 +409,24 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     runtime_bounds = d->src_end_ch_index >= 0 || d->dst_end_ch_index >= 0;
     if (runtime_bounds && batch_ids)
       return Fail(MLDHIP_UNIMPLEMENTED, "runtime channel bounds with batched weights are not supported");
+    if (d->packed_num_groups > 0) {
+      if (batch_ids) return Fail(MLDHIP_INVALID_ARGUMENT, "packed groups and batch ids exclude each other");
+      if (int8_math) return Fail(MLDHIP_UNIMPLEMENTED, "packed groups: floating-point FullyConnected only");
+      if (d->packed_params_offset < 0 || d->packed_max_group_size < 1)
+        return Fail(MLDHIP_INVALID_ARGUMENT, "packed groups need a params offset >= 0 and a positive max_group_size");
+      if (wd.output_group_size != DivUp(d->o, 4))
+        return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
+      packed_groups = true;
+      weights_batch = d->packed_num_groups;
+    }
   }
   mldhip_op* op = new (std::nothrow) mldhip_op();
   if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
   op->kind = mldhip_op::kFc;
   op->fc = *d;
   if (!d->has_runtime_check) op->fc.src_end_ch_index = op->fc.dst_end_ch_index = -1;
+  if (!packed_groups) op->fc.packed_num_groups = 0;
+  if (packed_groups) op->weights_batch = weights_batch;
   op->max_tokens = d->max_tokens;
   op->AddSrc("src_tensor");
   if (batch_ids) {  // registered before the weights objects (fully_connected.cc:1203-1208)
@@ -437,7 +449,7 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     op->idx_bias = (int)op->src_names.size();
     op->AddSrc("biases");
   }
-  if (runtime_bounds) {
+  if (runtime_bounds || packed_groups) {
     op->idx_params = (int)op->src_names.size();
     op->AddSrc("params");
   }
@@ -585,8 +597,11 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
     if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
-    if (op->idx_params >= 0)
-      (*src)[op->idx_params] = (size_t)(std::max(d.src_end_ch_index, d.dst_end_ch_index) + 1) * sizeof(int32_t);
+    if (op->idx_params >= 0) {
+      int values = std::max(d.src_end_ch_index, d.dst_end_ch_index) + 1;
+      if (d.packed_num_groups > 0) values = std::max(values, d.packed_params_offset + 2 * d.packed_num_groups);
+      (*src)[op->idx_params] = (size_t)values * sizeof(int32_t);
+    }
     (*dst)[0] = ns * m * 4 * TypeBytes(d.dst_type);
   } else if (op->kind == mldhip_op::kQuant) {
     const mldhip_quant_desc& d = op->q;
@@ -672,6 +687,11 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
     a.params = static_cast<const int32_t*>(op->src_ptr[op->idx_params]);
     a.src_end_ch_index = d.src_end_ch_index;
     a.dst_end_ch_index = d.dst_end_ch_index;
+    if (d.packed_num_groups > 0) {
+      a.packed_params_offset = d.packed_params_offset;
+      a.packed_max_group_size = d.packed_max_group_size;
+      a.weights_batch = op->weights_batch;
+    }
   }
   *out = a;
   return MLDHIP_OK;

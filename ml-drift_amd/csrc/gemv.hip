@@ -58,6 +58,9 @@ struct GenericParams {
   const int32_t* params;
   int src_end_ch_index, dst_end_ch_index;
   int k_channels;
+  // packed groups (fully_connected_util.cc:263-277; fully_connected.cc:706-710, 810-816): blockIdx.z =
+  // weight matrix g; its tokens are params[off + g] many from token params[off + weights_batch + g]
+  int packed_params_offset, packed_max_group_size;
 };
 
 // K-slices the loop covers and dst slices that are written, with runtime channel bounds
@@ -90,8 +93,19 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
   const int row = blockIdx.z;
   int wb = p.batch_ids ? p.batch_ids[row] : 0;
   wb = min(max(wb, 0), p.weights_batch - 1);
-  const size_t act_stride = (size_t)p.src_rows * p.m, dst_stride = (size_t)p.rows * p.m;
-  const size_t act_tok0 = (size_t)min(row, p.src_rows - 1) * p.m, dst_tok0 = (size_t)row * p.m;
+  size_t act_stride = (size_t)p.src_rows * p.m, dst_stride = (size_t)p.rows * p.m;
+  size_t act_tok0 = (size_t)min(row, p.src_rows - 1) * p.m, dst_tok0 = (size_t)row * p.m;
+  int tok_count = p.m;  // tokens of this row: tok0 + t < tok_count
+  if (p.packed_params_offset >= 0) {
+    // one row of p.m tokens; this work-group's matrix owns tok_count of them from token dst_tok0 on
+    wb = row;
+    const int size = p.params[p.packed_params_offset + row];
+    const int offset = p.params[p.packed_params_offset + p.weights_batch + row];
+    tok_count = min(min(size, p.packed_max_group_size), p.m - offset);
+    act_stride = dst_stride = (size_t)p.m;
+    act_tok0 = dst_tok0 = (size_t)max(offset, 0);
+    if (offset < 0 || tok0 >= tok_count) return;  // (the whole work-group: no barrier is left waiting)
+  }
   const uint8_t* weights = p.weights + (size_t)wb * p.ks * p.ns * (WBITS == 8 ? 16 : 8);
 
   float acc[TB][4];
@@ -148,7 +162,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 #pragma unroll
       for (int t = 0; t < TB; ++t) {
         const int tok = tok0 + t;
-        if (tok < p.m) {
+        if (tok < tok_count) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const float a = LoadF(act, ((size_t)ks * act_stride + act_tok0 + tok) * 4 + i);
@@ -170,7 +184,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
       const int tok = tok0 + t;
-      if (tok >= p.m) continue;
+      if (tok >= tok_count) continue;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         float r = 0.0f;
@@ -186,6 +200,7 @@ template <typename ActT, typename DstT, int WBITS>
 hipError_t LaunchGenericT(const GenericParams& p, hipStream_t stream) {
   constexpr int TB = 4;
   dim3 grid(DivUp(p.ns, kSl), DivUp(p.m, TB), p.rows);
+  if (p.packed_params_offset >= 0) grid = dim3(DivUp(p.ns, kSl), DivUp(std::min(p.m, p.packed_max_group_size), TB), p.weights_batch);
   dim3 block(kSl, kKl);
   hipLaunchKernelGGL((fc_generic_kernel<ActT, DstT, WBITS, TB>), grid, block, 0, stream, p);
   return hipGetLastError();
@@ -325,6 +340,10 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
   p.src_end_ch_index = a.src_end_ch_index;
   p.dst_end_ch_index = a.dst_end_ch_index;
   p.k_channels = a.k;
+  p.packed_params_offset = a.params ? a.packed_params_offset : -1;
+  p.packed_max_group_size = a.packed_max_group_size;
+  if (p.packed_params_offset >= 0 && (a.batch_ids != nullptr || a.packed_max_group_size < 1 || a.weights_batch < 1))
+    return hipErrorInvalidValue;
   if (kernel_name) *kernel_name = "fc_generic_kernel";
   const bool w8 = a.weight_bits == 8;
   if (a.act_f16 && a.dst_f16)

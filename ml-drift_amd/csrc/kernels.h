@@ -64,6 +64,10 @@ struct FcArgs {
   // kernel; an index < 0 = not set.  Served by the unspecialised kernels.
   const int32_t* params = nullptr;
   int src_end_ch_index = -1, dst_end_ch_index = -1;
+  // Packed groups (ConvRuntimeCheckDesc::PackedGroups, common/task/gpu_operation.h:396-406): the
+  // tokens of the one source row are sorted by weight matrix; params[offset + g] tokens starting at
+  // token params[offset + weights_batch + g] are multiplied with matrix g.  offset < 0 = not set.
+  int packed_params_offset = -1, packed_max_group_size = 0;
 };
 
 // Split-K workspace sizing for the streaming GEMV.

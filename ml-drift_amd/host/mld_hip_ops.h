@@ -116,6 +116,14 @@ struct ConvRuntimeCheckDesc {
   int ring_i_offset_index = -1;
   int ring_size = 0;
   bool HasValues() const { return src_end_ch_index >= 0 || dst_end_ch_index >= 0; }
+  // for batched weights: the tokens of the source row are sorted by weight matrix, sizes and offsets
+  // of the groups are read from the params object (gpu_operation.h:396-406); num_groups == 0 = not set
+  struct PackedGroups {
+    int params_offset = 0;  // [num_groups] sizes, then [num_groups] offsets
+    int num_groups = 0;     // the batch size of the weights (ExternalWeights::shape.h)
+    int max_group_size = 0;
+  };
+  PackedGroups packed_groups;
 };
 
 // A node executor: what ClOperation is to a GPUOperation in the reference.
@@ -213,6 +221,9 @@ inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType
   d.ring_o_offset_index = runtime_check.ring_o_offset_index;
   d.ring_i_offset_index = runtime_check.ring_i_offset_index;
   d.ring_size = runtime_check.ring_size;
+  d.packed_params_offset = runtime_check.packed_groups.params_offset;
+  d.packed_num_groups = runtime_check.packed_groups.num_groups;
+  d.packed_max_group_size = runtime_check.packed_groups.max_group_size;
   d.precision = (int)precision;
   d.src_type = (int)src_type;
   d.dst_type = (int)dst_type;

@@ -52,7 +52,9 @@ class FcDesc(C.Structure):
                 ("scalar_zero_point", C.c_float), ("has_bias", C.c_int32),
                 ("max_tokens", C.c_int32), ("has_runtime_check", C.c_int32),
                 ("src_end_ch_index", C.c_int32), ("dst_end_ch_index", C.c_int32),
-                ("ring_o_offset_index", C.c_int32), ("ring_i_offset_index", C.c_int32), ("ring_size", C.c_int32)]
+                ("ring_o_offset_index", C.c_int32), ("ring_i_offset_index", C.c_int32), ("ring_size", C.c_int32),
+                ("packed_params_offset", C.c_int32), ("packed_num_groups", C.c_int32),
+                ("packed_max_group_size", C.c_int32)]
 
 
 class QuantDesc(C.Structure):
@@ -382,9 +384,11 @@ def fc_launch_gated(gate, up, activation, dst, stream=0):
 def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1, 1),
               scalar_scale=1.0, has_zero_point_tensor=False, scalar_zero_point=None,
               has_bias=False, max_tokens=1, weights_batch=None, shared_src=False, src_end_ch_index=None,
-              dst_end_ch_index=None, ring_o_offset_index=None, ring_i_offset_index=None, ring_size=0):
+              dst_end_ch_index=None, ring_o_offset_index=None, ring_i_offset_index=None, ring_size=0,
+              packed_groups=None):
     """weights_batch: number of weight matrices of a batch-ids op (mldhip_fc_batch_ids_create).
-    src_end_ch_index / dst_end_ch_index: ConvRuntimeCheckDesc indices into the "params" object."""
+    src_end_ch_index / dst_end_ch_index: ConvRuntimeCheckDesc indices into the "params" object.
+    packed_groups: (params_offset, num_groups, max_group_size) of ConvRuntimeCheckDesc::PackedGroups."""
     d = FcDesc()
     d.precision, d.src_type, d.dst_type, d.o, d.i = precision, src_type, dst_type, o, i
     d.weights = weights_desc
@@ -396,7 +400,9 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
     d.has_bias = int(has_bias)
     d.max_tokens = max_tokens
     checks = (src_end_ch_index, dst_end_ch_index, ring_o_offset_index, ring_i_offset_index)
-    d.has_runtime_check = int(any(v is not None for v in checks))
+    d.has_runtime_check = int(any(v is not None for v in checks) or packed_groups is not None)
+    if packed_groups is not None:
+        d.packed_params_offset, d.packed_num_groups, d.packed_max_group_size = packed_groups
     d.src_end_ch_index, d.dst_end_ch_index, d.ring_o_offset_index, d.ring_i_offset_index = [
         -1 if v is None else v for v in checks]
     d.ring_size = ring_size

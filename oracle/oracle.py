@@ -312,6 +312,38 @@ def fc_batch_ids_kernel(act_slices, ids, weights, rows, row_tokens, src_rows, we
     return out
 
 
+def fc_packed_groups_kernel(act_slices, sizes, offsets, weights, tokens, k, n, precision, weight_bits,
+                            scale_kind=SCALE_LINEAR, scale=None, zero_point=None, bias=None, groups=1,
+                            max_group_size=None, dst_before=None):
+    """The generated kernel with ConvRuntimeCheckDesc::PackedGroups (common/kernels/fully_connected_util.cc:
+    263-277: w_group_size / w_group_offset read per weight matrix, work-groups beyond the size return;
+    fully_connected.cc:810-816: source and destination token = w_group_offset + local token, row 0;
+    fully_connected_util.cc:382-386: written only below w_group_offset + w_group_size): matrix g on the
+    `sizes[g]` tokens from token `offsets[g]`, i.e. `fc_kernel` on that run of tokens with matrix g of
+    the batched buffers.  Tokens in no group keep `dst_before` (zeros when not given).
+    act [Ks][tokens][4] -> [Ns][tokens][4]; weights / scale / zero_point as for fc_batch_ids_kernel."""
+    tdt = np.float32 if precision == PREC_F32 else np.uint16
+    ks, ns = div_up(k, 4), div_up(n, 4)
+    nb = len(sizes)
+    act = _c(act_slices, tdt).reshape(ks, tokens, 4)
+    w = _c(weights, np.uint8).reshape(nb, -1)
+    sc = None if scale is None else _c(scale, tdt).reshape(groups, nb, ns * 4)
+    zp = None if zero_point is None else _c(zero_point, tdt).reshape(groups, nb, ns * 4)
+    out = np.zeros((ns, tokens, 4), tdt) if dst_before is None else _c(dst_before, tdt).reshape(ns, tokens, 4).copy()
+    for g in range(nb):
+        size, off = int(sizes[g]), int(offsets[g])
+        if max_group_size is not None:
+            size = min(size, max_group_size)
+        size = min(size, tokens - off)
+        if size <= 0 or off < 0:
+            continue
+        a = np.ascontiguousarray(act[:, off:off + size, :])
+        out[:, off:off + size, :] = fc_kernel(a, w[g], size, k, n, precision, weight_bits, scale_kind,
+                                              None if sc is None else np.ascontiguousarray(sc[:, g, :]),
+                                              None if zp is None else np.ascontiguousarray(zp[:, g, :]), bias, groups)
+    return out
+
+
 def fc_batch_ids_int8_kernel(act_slices_i8, ids, weights, rows, row_tokens, src_rows, weights_batch, k, n, weight_bits):
     """The integer-math variant with batched weights (the same generator with int8 sources:
     common/kernels/fully_connected.cc:543-621 with the w_batch_id offsets of :549-557, rows as in

@@ -90,6 +90,25 @@ int main() {
   EXPECT(CreateFullyConnectedOI(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w, true, 4, &not_oi)
              .code == MLDHIP_INVALID_ARGUMENT);
 
+  // packed groups (gpu_model_builder_moe_util.cc:133-141, 214-224): batched weights, "params" last
+  {
+    ExternalWeights wp;
+    wp.shape = OHWI{768, 128, 1, 2048};
+    mldhip_fc_int4_weights_desc_reference(768, 2048, &wp.desc);
+    wp.scale_zp_shape = OHWI{768, 128, 1, 64};
+    wp.has_scale_tensor = true;
+    ConvRuntimeCheckDesc rc_packed;
+    rc_packed.packed_groups.params_offset = 0;
+    rc_packed.packed_groups.num_groups = 128;
+    rc_packed.packed_groups.max_group_size = 64;
+    HipOperation grouped;
+    EXPECT(CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, wp,
+                                               /*has_bias=*/false, 512, &grouped, rc_packed)
+               .ok());
+    names = grouped.GetSrcTensorsNames();
+    EXPECT(names.size() == 4 && names[1] == "weights" && names[2] == "weights_scale" && names[3] == "params");
+  }
+
   // the mixture-of-experts FullyConnected: fully_connected.cc:1203-1213 registers batch_ids before the weights
   ExternalWeights we;
   we.shape = OHWI{768, 128, 1, 2048};

@@ -1,0 +1,107 @@
+"""GPU parity of the FullyConnected with packed groups (ConvRuntimeCheckDesc::PackedGroups: the
+tokens of the source row sorted by weight matrix, group sizes and offsets read on the device - the
+grouped FullyConnected of a mixture-of-experts prefill, MakeConvWithPackedGroups,
+common/gpu_model_builder_moe_util.cc:119-230), through the C-ABI: the reference test's own flow
+(common/kernels/tests/fully_connected_test_util.cc:2487-2597) against the per-token float64 products,
+and against the oracle's restatement of the kernel."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+import mldhip as M
+import workloads as W
+from test_oracle_fc import (make_packed_groups_case, packed_groups_expected, run_packed_groups_oracle, unpack_groups)
+
+FP16_TOL = 2e-2
+
+
+def run_device(c, td, sizes=None, offsets=None, max_group_size=None, params_offset=0, fill=None):
+    import torch
+    tt = torch.float16 if td == np.float16 else torch.float32
+    mt = M.FLOAT16 if td == np.float16 else M.FLOAT32
+    n, k, batch = c["n"], c["k"], c["batch"]
+    ns = W.div_up(n, 4)
+    tokens = c["packed_src"].shape[0]
+    desc = M.fc_int8_weights_desc(n, k) if c["bits"] == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    packed = (M.rearrange_int8_as_uint8 if c["bits"] == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
+
+    def tensor(v):
+        t = M.scale_to_tensor_batched(v, mt)
+        return torch.from_numpy(t.view(td) if td == np.float16 else t).cuda()
+    sizes = c["sizes"] if sizes is None else sizes
+    offsets = c["offsets"] if offsets is None else offsets
+    params = np.concatenate([np.full(params_offset, -12345, np.int32), sizes, offsets]).astype(np.int32)
+    srcs = [torch.from_numpy(W.to_slices(c["packed_src"]).astype(td)).cuda(), torch.from_numpy(packed).cuda(),
+            tensor(c["scale"])]
+    if c["zp"] is not None:
+        srcs.append(tensor(c["zp"]))
+    srcs.append(torch.from_numpy(params).cuda())
+    out = torch.full((ns, tokens, 4), 0.0 if fill is None else fill, dtype=tt, device="cuda")
+    op = M.fc_create(M.PRECISION_F32 if td == np.float32 else M.PRECISION_F32_F16, mt, mt, n, k, desc,
+                     scale_shape=(n, c["groups"]), has_zero_point_tensor=c["zp"] is not None, max_tokens=tokens,
+                     packed_groups=(params_offset, batch, max_group_size or tokens))
+    assert op.src_names[-1] == "params" and op.src_names[1] == "weights"
+    op.bind(srcs, [out])
+    op.set_shape(1, 1, tokens)
+    print("packed groups", c["bits"], tokens, k, n, batch, c["groups"], td.__name__, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert op.kernel_name == "fc_generic_kernel", op.kernel_name
+    return W.from_slices(out.cpu().numpy().astype(np.float32), n)
+
+
+def check(got, ref, td, k):
+    err = np.abs(got - ref).max()
+    if td == np.float16:
+        rms = np.sqrt(np.mean(ref ** 2))
+        assert err <= FP16_TOL * rms, (err, rms)
+    else:
+        tol = 1.1920929e-7 * (k + 1) * max(1.0, np.abs(ref).max())
+        assert err <= tol, (err, tol)
+
+
+@pytest.mark.parametrize("td", [np.float32, np.float16])
+@pytest.mark.parametrize("bits,groups,zp", [(8, 1, False), (4, 2, True)])
+def test_reference_test_flow(oracle, td, bits, groups, zp):
+    c = make_packed_groups_case(3 + bits, 64, 4, 64, 32, 16, bits, groups, zp)
+    got = unpack_groups(c, run_device(c, td))
+    assert not np.isnan(got).any()
+    check(got, packed_groups_expected(oracle, c, td), td, c["k"])
+
+
+@pytest.mark.parametrize("bits,width,per_item,k,n,batch,groups,zp,td", [
+    (4, 512, 8, 2048, 768, 128, 64, False, np.float16),   # a mixture layer's prefill: 4096 routed tokens, 128 experts
+    (4, 96, 2, 768, 2048, 8, 24, False, np.float16),      # its down projections
+    (8, 33, 3, 171, 533, 5, 1, True, np.float32),         # the reference's odd sizes
+    (4, 7, 1, 64, 20, 4, 2, True, np.float16),            # fewer tokens than a token block, ragged channels
+])
+def test_mixture_prefill_shapes(oracle, bits, width, per_item, k, n, batch, groups, zp, td):
+    c = make_packed_groups_case(width + n, width, per_item, k, n, batch, bits, groups, zp)
+    rows = run_device(c, td, params_offset=3)
+    got = unpack_groups(c, rows)
+    check(got, packed_groups_expected(oracle, c, td), td, k)
+    if width * per_item * k * n <= 1 << 28:
+        rest = run_packed_groups_oracle(oracle, c, oracle.PREC_F32 if td == np.float32 else oracle.PREC_F32F16)
+        check(rows, rest.astype(np.float64), td, k)
+
+
+def test_tokens_outside_every_group_are_not_written(oracle):
+    c = make_packed_groups_case(11, 16, 2, 32, 8, 4)
+    sizes = np.array([5, 0, 9, 40], np.int32)
+    offsets = np.array([2, 7, 10, 28], np.int32)
+    got = run_device(c, np.float32, sizes=sizes, offsets=offsets, max_group_size=6, fill=7.0)
+    before = np.full((2, 32, 4), 7.0, np.float32)
+    ref = run_packed_groups_oracle(oracle, c, oracle.PREC_F32, max_group_size=6, dst_before=before, sizes=sizes, offsets=offsets)
+    assert np.array_equal(got == 7.0, ref == 7.0)
+    assert np.abs(got - ref).max() <= 1e-5
+
+
+def test_packed_groups_arguments():
+    d = M.fc_int4_weights_desc(64, 64, reference=True)
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d, scale_shape=(64, 1), packed_groups=(0, 4, 0))
+    assert e.value.code == M.INVALID_ARGUMENT
+    with pytest.raises(M.MldhipError) as e:
+        M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 64, 64, d, packed_groups=(0, 4, 8))
+    assert e.value.code == M.UNIMPLEMENTED

@@ -442,3 +442,97 @@ def test_vector_path_declines_what_it_cannot_state_exactly(oracle):
     assert o.last_fc_path == 0
     o.fc_kernel(act, packed, 1, k, n, o.PREC_F32, 4, o.SCALE_LINEAR, np.full(8, 0.01, np.float32))
     assert o.last_fc_path == 0
+
+
+# ---- packed groups (the grouped FullyConnected of a mixture-of-experts prefill) ----
+def make_packed_groups_case(seed, width, per_item, k, n, batch, bits=8, groups=1, with_zp=False):
+    """The set-up of FullyConnectedPackedGroupsTest (fully_connected_test_util.cc:2487-2530): every one of
+    `width` tokens goes to `per_item` distinct matrices of `batch`; GroupsMapReference /
+    PackedGroupsMapReference (common/task/testing_ref_ops.cc:2765-2816) sort the (slot, token) pairs by
+    matrix (tokens ascending, slots inner), RemapToReference (:2819-2833) gathers the source rows in that
+    order.  Returns the batch-ids style case plus ids [width][per_item], the packed (slot, token) list,
+    sizes and offsets."""
+    c = make_batch_ids_case(seed, 1, 1, 1, k, n, batch, bits, groups, with_zp)
+    rng = np.random.default_rng(seed + 1)
+    src = rng.uniform(-1, 1, size=(width, k)).astype(np.float32)
+    ids = np.stack([rng.permutation(batch)[:per_item] for _ in range(width)]).astype(np.int32)
+    lists = [[] for _ in range(batch)]
+    for w in range(width):
+        for slot in range(per_item):
+            lists[int(ids[w, slot])].append((slot, w))
+    sizes = np.array([len(l) for l in lists], np.int32)
+    offsets = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(np.int32)
+    packed_map = [p for l in lists for p in l]
+    c.update(tokens_src=src, ids2=ids, packed_map=packed_map, sizes=sizes, offsets=offsets, width=width, per_item=per_item,
+             packed_src=np.stack([src[w] for _, w in packed_map]))
+    return c
+
+
+def packed_groups_expected(o, c, dtype=np.float32):
+    """ConvolutionWithIds (common/task/testing_ref_ops.cc:2853-2880) in float64 over the dequantized
+    matrices: result[slot][token] = W[ids[token][slot]] . src[token]."""
+    wf = batch_ids_float_weights(o, c).astype(np.float64)
+    src = c["tokens_src"].astype(dtype).astype(np.float64)
+    out = np.empty((c["per_item"], c["width"], c["n"]))
+    for w in range(c["width"]):
+        for slot in range(c["per_item"]):
+            out[slot, w] = wf[:, int(c["ids2"][w, slot]), :] @ src[w]
+    return out
+
+
+def unpack_groups(c, packed_rows):
+    """RemapFromReference (common/task/testing_ref_ops.cc:2835-2851)."""
+    out = np.full((c["per_item"], c["width"], packed_rows.shape[1]), np.nan)
+    for i, (slot, w) in enumerate(c["packed_map"]):
+        out[slot, w] = packed_rows[i]
+    return out
+
+
+def run_packed_groups_oracle(o, c, precision, max_group_size=None, dst_before=None, sizes=None, offsets=None):
+    ns = (c["n"] + 3) // 4
+    pack = o.int8_as_uint8 if c["bits"] == 8 else o.int8_as_uint4
+    packed = pack(c["w"], I4O4, ns)
+    tokens = c["packed_src"].shape[0]
+    act = tensor(o, o.to_slices(c["packed_src"]), precision)
+    kind = o.SCALE_LINEAR if c["groups"] == 1 else o.SCALE_BLOCK
+    sc = tensor(o, o.scale_to_hoio4_batched(c["scale"]), precision)
+    zp = None if c["zp"] is None else tensor(o, o.scale_to_hoio4_batched(c["zp"]), precision)
+    out = o.fc_packed_groups_kernel(act, c["sizes"] if sizes is None else sizes, c["offsets"] if offsets is None else offsets,
+                                    packed, tokens, c["k"], c["n"], precision, c["bits"], kind, sc, zp, None, c["groups"],
+                                    max_group_size, dst_before)
+    return o.from_slices(to_f32(o, out, precision), c["n"])
+
+
+@pytest.mark.parametrize("bits,groups,zp", [(8, 1, False), (4, 2, True)])
+def test_packed_groups_reference_test_flow(oracle, bits, groups, zp):
+    """The reference test's shape (64 -> 32 channels, 64 tokens, 16 matrices, 4 per token) through the
+    reference test's own flow: pack by matrix, run the grouped kernel, unpack, compare with the
+    per-token products; its tolerance eps * 2 * K (fully_connected_test_util.cc:2594-2595)."""
+    o = oracle
+    c = make_packed_groups_case(3 + bits, 64, 4, 64, 32, 16, bits, groups, zp)
+    assert c["sizes"].sum() == 64 * 4 and c["packed_src"].shape == (256, 64)
+    got = unpack_groups(c, run_packed_groups_oracle(o, c, o.PREC_F32))
+    ref = packed_groups_expected(o, c)
+    assert not np.isnan(got).any()
+    assert np.abs(got - ref).max() <= 1e-6 * 2.0 * 64 * max(1.0, np.abs(ref).max())
+
+
+def test_packed_groups_leaves_other_tokens_alone(oracle):
+    """Tokens that no group covers keep what the tensor held; a group is cut at max_group_size and at
+    the end of the tensor; a group of size 0 writes nothing."""
+    o = oracle
+    c = make_packed_groups_case(11, 16, 2, 32, 8, 4)
+    tokens = c["packed_src"].shape[0]  # 32
+    sizes = np.array([5, 0, 9, 40], np.int32)
+    offsets = np.array([2, 7, 10, 28], np.int32)
+    before = np.full((2, tokens, 4), 7.0, np.float32)
+    got = run_packed_groups_oracle(o, c, o.PREC_F32, max_group_size=6, dst_before=before, sizes=sizes, offsets=offsets)
+    written = np.zeros(tokens, bool)
+    written[2:7] = True      # group 0: 5 tokens
+    written[10:16] = True    # group 2: 9 cut to max_group_size 6
+    written[28:32] = True    # group 3: cut at the end of the tensor
+    assert np.all(got[~written] == 7.0) and not np.any(got[written] == 7.0)
+    wf = batch_ids_float_weights(o, c).astype(np.float64)
+    for g, (a, b) in {0: (2, 7), 2: (10, 16), 3: (28, 32)}.items():
+        ref = c["packed_src"][a:b].astype(np.float64) @ wf[:, g, :].T
+        assert np.abs(got[a:b] - ref).max() <= 1e-5
