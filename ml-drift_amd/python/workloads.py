@@ -81,7 +81,7 @@ class FcDevice:
     """An FC op with its device buffers (torch tensors) for one synthetic case."""
 
     def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None, reference_layout=False,
-                 output_group=None):
+                 output_group=None, precision=None):
         import torch
         self.torch = torch
         self.case = case
@@ -111,7 +111,8 @@ class FcDevice:
             self.bias = torch.from_numpy(b).to(device)
             srcs.append(self.bias)
         self.out = torch.zeros((div_up(n, 4), m, 4), dtype=tt, device=device)
-        precision = M.PRECISION_F32 if td == np.float32 else M.PRECISION_F32_F16
+        if precision is None:
+            precision = M.PRECISION_F32 if td == np.float32 else M.PRECISION_F32_F16
         self.op = M.fc_create(precision, mt, mt, n, k, self.desc, scale_shape=scale_shape,
                               scalar_scale=1.0 if scalar_scale is None else scalar_scale,
                               has_zero_point_tensor=scalar_scale is None and case["zero_point"] is not None,

@@ -474,3 +474,25 @@ def test_fc_tensor_batch(oracle, bits, k, n, groups, b, w):
     check_fp(batched, textbook(case), case, "textbook")
     if m * k * n <= 1 << 27:
         check_fp(batched, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
+
+
+@pytest.mark.parametrize("bits,m,k,n,groups", [(4, 1, 4096, 2048, 1), (4, 3, 1024, 1032, 32), (8, 1, 2048, 2048, 16),
+                                               (4, 64, 512, 384, 4), (8, 5, 171, 533, 1)])
+def test_precision_f16_runs_with_float_accumulators(oracle, bits, m, k, n, groups):
+    """CalculationsPrecision::kF16 (all arithmetic in half in the reference,
+    common/kernels/fully_connected_util.cc:167-203) is accepted and computed like kF32_F16, with fp32
+    accumulators: bit-identical to the op created with kF32_F16, hence inside the tolerance, and
+    closer to the float64 result than the reference's all-half kernel as the oracle restates it."""
+    case = W.make_fc_case(seed=bits + m + k, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                          with_bias=True)
+    print("precision F16", bits, m, k, n, groups, flush=True)
+    a = W.FcDevice(case, precision=M.PRECISION_F16)
+    a.run()
+    b = W.FcDevice(case, precision=M.PRECISION_F32_F16)
+    b.run()
+    got = a.result()
+    assert a.op.kernel_name == b.op.kernel_name and np.array_equal(got, b.result())
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    half = oracle_fc(oracle, case, precision=oracle.PREC_F16).astype(np.float64)
+    assert np.sqrt(np.mean((got - ref) ** 2)) <= np.sqrt(np.mean((half - ref) ** 2)) + 2.0 ** -12 * np.sqrt(np.mean(ref ** 2))
