@@ -42,9 +42,11 @@ def parse():
                    help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
                         "kernels away from the launch-bound regime)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
-    p.add_argument("--layout", default="library", choices=["library", "reference"],
+    p.add_argument("--layout", default="default", choices=["default", "library", "reference"],
                    help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
-                        "slices) or in the reference's own FullyConnected layout (one output group)")
+                        "slices; the default) or in the reference's own FullyConnected layout (one output group). "
+                        "c5-decode: the weights as mldhip_fc_int4_weights_desc_decode asks for them (the default) or, "
+                        "with 'library', in the one layout that serves decode and prefill ops alike")
     p.add_argument("--tune", default="", help="tuning knobs for the run, e.g. gemv_ksplit=1,gemm_dual=0 (mldhip_set_tuning)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
@@ -285,13 +287,16 @@ def run_other(args, torch, M, W):
     else:
         from decoder_stack import DecoderStack
         tokens = 1 if args.workload == "c5-decode" else max(5, args.tokens)
-        st = DecoderStack(max_tokens=max(128, tokens), keep_host=False)
+        # a decode step runs over the weights as a decode graph's ops ask for them (--layout library:
+        # the one layout that serves both graphs)
+        decode_layout = tokens == 1 and args.layout != "library"
+        st = DecoderStack(max_tokens=max(128, tokens), keep_host=False, decode_layout=decode_layout)
         st.set_tokens(tokens)
         wall, us, reg = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
         wb, fl = st.weight_bytes(), st.flops(tokens)
         if tokens == 1:
             out = dict(base, metric="int4_decoder_stack_decode_hbm_bandwidth", value=round(wb / wall / 1e9, 1),
-                       unit="GB/s", roofline={"bound": "hbm", "kernel": "fc_w4_stream_kernel (126 FCs per step; q/k/v and gate/up share a launch)",
+                       unit="GB/s", roofline={"bound": "hbm", "kernel": "%s (126 FCs per step; q/k/v and gate/up share a launch)" % " + ".join(sorted(set(st.kernel_names()))),
                                               "achieved": round(wb / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                               "frac": round(wb / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
                                               "avg_step_us": round(us, 1)})
@@ -303,7 +308,9 @@ def run_other(args, torch, M, W):
                                                  "avg_step_us": round(us, 1)})
         out.update(ms_per_step=round(wall * 1e3, 6), dtype="u4 weights x f16 activations, f32 accumulate",
                    config=dict({"workload": "c5: 18 layers x (q,k,v,o,gate,up,down) int4 group-32, hidden 2048, %d token(s) "
-                                            "per step" % tokens, "weight_bytes_per_step": wb, "flops_per_step": fl}, **reg))
+                                            "per step" % tokens, "weight_bytes_per_step": wb, "flops_per_step": fl,
+                                "weights_layout": "decode ops' layout (mldhip_fc_int4_weights_desc_decode)" if decode_layout
+                                else "mldhip_fc_int4_weights_desc"}, **reg))
     print(json.dumps(out))
 
 

@@ -126,6 +126,14 @@ int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc);
 /* The reference's own GetFullyConnectedInt4WeightsDesc choice (one output group,
  * output_group_size = ceil(o/4)), for weights that were packed for the reference's kernel. */
 int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* desc);
+/* The layout for an op that only ever runs one token per launch (the FullyConnected nodes of a
+ * decode graph, where a builder keeps a second packed copy of the weights for the prefill graph):
+ * as mldhip_fc_int4_weights_desc, except that layers of fewer than 8192 output channels, which
+ * have too few 64-channel strips to occupy the chip, take output groups of 2 slices (8 channels,
+ * 16-byte K rows): every CU then streams the whole K of a strip and no second kernel adds partial
+ * sums.  Ops over this layout run any number of tokens, but more than one token is served by the
+ * slower general kernels. */
+int mldhip_fc_int4_weights_desc_decode(int o, int i, mldhip_weights_desc* desc);
 
 /* The weights layout the int8 x int8 MFMA convolution asks for, the counterpart of the
  * conv_weights_desc that SelectConvolutionInt8 returns to the builder

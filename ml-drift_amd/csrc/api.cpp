@@ -155,13 +155,20 @@ int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc) {
 int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* desc) {
   return FcDesc(o, i, MLDHIP_UINT4, false, desc);
 }
+int mldhip_fc_int4_weights_desc_decode(int o, int i, mldhip_weights_desc* desc) {
+  if (int rc = FcDesc(o, i, MLDHIP_UINT4, true, desc)) return rc;
+  // fewer than 128 strips of 64 channels: strips of 8 channels (output groups of 2 slices), which the
+  // one-token kernel reads with the whole K inside a work-group
+  if (o % 8 == 0 && o / 64 < 128 && GetTuning().fc_group <= 0) desc->output_group_size = 2;
+  return MLDHIP_OK;
+}
 
 int mldhip_set_tuning(const char* name, int value) {
   if (!name) return Fail(MLDHIP_INVALID_ARGUMENT, "null name");
   Tuning& t = GetTuning();
   const struct { const char* name; int* field; } knobs[] = {
       {"force_generic", &t.force_generic}, {"gemv_mfma", &t.gemv_mfma}, {"gemv_fast", &t.gemv_fast},
-      {"fc_group", &t.fc_group},
+      {"fc_group", &t.fc_group}, {"gemv_rows_rpt", &t.gemv_rows_rpt},
       {"gemv_lpr", &t.gemv_lpr}, {"gemv_waves", &t.gemv_waves}, {"gemv_ksplit", &t.gemv_ksplit},
       {"gemv_narrow_max_mb", &t.gemv_narrow_max_mb}, {"gemm_fm", &t.gemm_fm}, {"gemm_ksplit", &t.gemm_ksplit},
       {"gemm_no_pair", &t.gemm_no_pair}, {"gemm_dual", &t.gemm_dual}, {"gemm_xcd_m", &t.gemm_xcd_m},

@@ -600,6 +600,7 @@ __device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
   // narrower rows: the lanes 4 (and 2) apart hold further rows of the same channels
   if (LPR <= 4) v += __shfl_xor(v, 4, 64);
   if (LPR <= 2) v += __shfl_xor(v, 2, 64);
+  if (LPR <= 1) v += __shfl_xor(v, 1, 64);
   return v;
 }
 
@@ -888,6 +889,201 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// One token over weights packed in output groups of 2 slices (8 channels): the whole K of a strip
+// of 8 channels is one contiguous run of 16-byte rows, so layers of a few thousand channels, which
+// have too few 64-channel strips to occupy the chip, give every CU a strip without splitting K
+// across work-groups (no second kernel for the sums).  Lane l of the work-group reads rows
+// l, l + T, l + 2T, ... (T threads): every load instruction of a wave covers 1 KB of contiguous
+// memory.  The rows of a thread lie in different scale groups, so with group-wise scales a row's
+// sums are scaled as they are added (scale vectors come from cache: 8 lanes share one).
+// K reduction: the 8 channel sums of the 64 lanes by the register exchanges of the strip kernel
+// (all lanes hold rows of the same 8 channels), across waves through LDS in wave order.
+// ------------------------------------------------------------------------------------------
+template <int WAVES, bool GROUPED, bool ZP, bool MULTI>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
+  constexpr int T = WAVES * 64;
+  __shared__ float red[WAVES][8];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  // Work-groups go round-robin to the 8 XCDs.  The scales of 8 neighbouring strips share a 128-byte
+  // line per scale group, so neighbouring strips are given to work-groups of one XCD (whose L2 then
+  // fetches the line once): of every 64 work-groups, XCD x takes strips 8x .. 8x + 7.
+  int si = 0, strip = blockIdx.x;
+  if (strip < (int)(gridDim.x & ~63u)) strip = (strip & ~63) + ((strip & 7) << 3) + ((strip >> 3) & 7);
+  if (MULTI && p.segments > 1 && strip >= p.seg[0].strip_end) {
+    si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
+    strip -= p.seg[si - 1].strip_end;
+  }
+  const StripSegment& sg = p.seg[MULTI ? si : 0];
+  struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
+  const u32x4* wstrip = sg.weights + (size_t)strip * p.ks;  // row r of the strip: K-slice r, 2 slices x 8 bytes
+  const u32x2* act2 = reinterpret_cast<const u32x2*>(p.act);
+  const __half* scale = sg.scale;
+  const __half* zero_point = sg.zero_point;
+  const int ks = p.ks, n_pad = sg.n_pad;
+  const int group_shift = p.group_chunks;  // log2 of the K-slices per scale group (grouped only)
+  const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+
+  float acc[8], asum_all = 0.0f;
+#pragma unroll
+  for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
+  u32x4 zv_lin = {0u, 0u, 0u, 0u};
+  if (ZP && !GROUPED) zv_lin = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * 8);
+
+  for (int r0 = tid; r0 < ks; r0 += 8 * T) {
+    u32x4 w[8], sv[8], zv[8];
+    u32x2 a[8];
+    // small loads that come from cache first, then the eight weight loads back to back
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = r0 + T * j;
+      const u32x2 v = act2[min(r, ks - 1)];
+      a[j] = u32x2{r < ks ? v[0] : 0u, r < ks ? v[1] : 0u};
+    }
+    if (GROUPED) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const size_t so = (size_t)(min(r0 + T * j, ks - 1) >> group_shift) * n_pad + (size_t)strip * 8;
+        sv[j] = *reinterpret_cast<const u32x4*>(scale + so);
+        if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(zero_point + so);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wstrip + min(r0 + T * j, ks - 1));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const half2_t a01 = AsHalf2(a[j][0]), a23 = AsHalf2(a[j][1]);
+      float asum = __builtin_amdgcn_fdot2(a01, ones, 0.0f, false);
+      asum = __builtin_amdgcn_fdot2(a23, ones, asum, false);
+      float t[8];
+#pragma unroll
+      for (int h = 0; h < 4; h += 2) {  // words h, h + 1: inputs (0, 1) and (2, 3) of outputs 4 * (h >> 1) .. + 3
+        const uint32_t lo0 = w[j][h], hi0 = lo0 >> 8, lo1 = w[j][h + 1], hi1 = lo1 >> 8;
+        const int ob = 4 * (h >> 1);
+        t[ob + 0] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(lo0, up.mask_lo, up.magic_lo)), a01, 0.0f, false);
+        t[ob + 1] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(lo0, up.mask_hi, up.magic_hi)), a01, 0.0f, false);
+        t[ob + 2] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(hi0, up.mask_lo, up.magic_lo)), a01, 0.0f, false);
+        t[ob + 3] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(hi0, up.mask_hi, up.magic_hi)), a01, 0.0f, false);
+        t[ob + 0] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(lo1, up.mask_lo, up.magic_lo)), a23, t[ob + 0], false);
+        t[ob + 1] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(lo1, up.mask_hi, up.magic_hi)), a23, t[ob + 1], false);
+        t[ob + 2] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(hi1, up.mask_lo, up.magic_lo)), a23, t[ob + 2], false);
+        t[ob + 3] = __builtin_amdgcn_fdot2(AsHalf2(AndOr(hi1, up.mask_hi, up.magic_hi)), a23, t[ob + 3], false);
+      }
+      if (GROUPED) {
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+          float centre = (o & 1) ? -72.0f : -1032.0f;  // the unpacked code carries +64 / +1024; its centre is 8
+          if (ZP) centre -= (float)AsHalf2(zv[j][o >> 1])[o & 1];
+          acc[o] = fmaf((float)AsHalf2(sv[j][o >> 1])[o & 1], fmaf(centre, asum, t[o]), acc[o]);
+        }
+      } else {
+        asum_all += asum;
+#pragma unroll
+        for (int o = 0; o < 8; ++o) acc[o] += t[o];
+      }
+    }
+  }
+  if (!GROUPED) {
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+      float centre = (o & 1) ? -72.0f : -1032.0f;
+      if (ZP) centre -= (float)AsHalf2(zv_lin[o >> 1])[o & 1];
+      acc[o] = fmaf(centre, asum_all, acc[o]);
+    }
+  }
+  // every lane holds sums of the same 8 channels: lane l ends with channel (l / 8) % 8
+  float v = WaveStripSum<1>(acc, lane);
+  const int ch = (lane >> 3) & 7;
+  if (WAVES > 1) {
+    if ((lane & 7) == 0) red[wave][ch] = v;
+    __syncthreads();
+    if (tid >= 64) return;
+    v = 0.0f;
+#pragma unroll
+    for (int q = 0; q < WAVES; ++q) v += red[q][ch];
+  }
+  if ((lane & 7) != 0) return;
+  const int n_out = strip * 8 + ch;
+  if (!GROUPED) v *= __half2float(scale[n_out]);
+  __half h = __float2half_rn(v);
+  if (sg.bias) h = __hadd(h, sg.bias[n_out]);
+  sg.dst[n_out] = h;
+}
+
+template <int WAVES>
+hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+  const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
+  const dim3 block(WAVES * 64);
+#define MLD_ROWS(G, Z, MU) hipLaunchKernelGGL((fc_w4_rows_kernel<WAVES, G, Z, MU>), grid, block, 0, stream, p)
+  if (grouped) {
+    if (zp) { if (multi) MLD_ROWS(true, true, true); else MLD_ROWS(true, true, false); }
+    else    { if (multi) MLD_ROWS(true, false, true); else MLD_ROWS(true, false, false); }
+  } else {
+    if (zp) { if (multi) MLD_ROWS(false, true, true); else MLD_ROWS(false, true, false); }
+    else    { if (multi) MLD_ROWS(false, false, true); else MLD_ROWS(false, false, false); }
+  }
+#undef MLD_ROWS
+  return hipGetLastError();
+}
+
+// The row-interleaved kernel serves: one token, every matrix of the launch packed in output groups
+// of 2 slices, scale groups of a power-of-two number of K-slices.
+bool RowsKernelServes(const FcArgs* args, int count) {
+  if (GetTuning().gemv_fast == 0) return false;
+  if (args[0].m != 1 || args[0].batch_ids != nullptr || args[0].k % 4 != 0) return false;
+  for (int i = 0; i < count; ++i) {
+    const int ns = DivUp(args[i].n, 4);
+    if (args[i].n % 8 != 0 || EffectiveGroup(args[i].group, ns) != 2) return false;
+  }
+  if (args[0].scale_kind == kScaleBlock) {
+    const int group_slices = DivUp(args[0].k, 4) / args[0].groups;
+    if (group_slices < 1 || (group_slices & (group_slices - 1)) != 0) return false;
+  }
+  return true;
+}
+
+hipError_t LaunchRows(const StreamParams& p, const FcArgs* args, int count, bool grouped, hipStream_t stream) {
+  StripParams sp;
+  sp.act = p.act;
+  sp.partial = nullptr;
+  sp.ks = p.ks;
+  sp.chunks = p.chunks;
+  sp.chunks_per_split = p.chunks;
+  sp.ksplit = 1;
+  sp.group_chunks = 0;  // here: log2 of the K-slices per scale group
+  if (grouped)
+    for (int gs = p.ks / p.groups; gs > 1; gs >>= 1) ++sp.group_chunks;
+  sp.n_total = p.n_total;
+  sp.segments = p.segments;
+  sp.reserved = 0;
+  sp.mask_lo = p.mask_lo;
+  sp.mask_hi = p.mask_hi;
+  sp.magic_lo = p.magic_lo;
+  sp.magic_hi = p.magic_hi;
+  int strips = 0;
+  for (int i = 0; i < kMaxSegments; ++i) {
+    const StreamSegment& g = p.seg[i];
+    if (i < count) strips += g.ns / 2;
+    sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, strips, g.n_off, 0};
+  }
+  // eight rows per thread where K allows: all of a thread's loads are in flight at once
+  const int rpt = GetTuning().gemv_rows_rpt > 0 ? GetTuning().gemv_rows_rpt : 8;
+  int waves = 1;
+  while (waves < 16 && waves * 64 * rpt < p.ks) waves *= 2;
+  if (GetTuning().gemv_waves > 0) waves = GetTuning().gemv_waves;
+  const dim3 grid(strips);
+  switch (waves) {
+    case 1: return LaunchRowsW<1>(sp, grouped, grid, stream);
+    case 2: return LaunchRowsW<2>(sp, grouped, grid, stream);
+    case 4: return LaunchRowsW<4>(sp, grouped, grid, stream);
+    case 8: return LaunchRowsW<8>(sp, grouped, grid, stream);
+    default: return LaunchRowsW<16>(sp, grouped, grid, stream);
+  }
+}
+
 }  // namespace
 
 bool FcW4StreamSupported(const FcArgs& a) {
@@ -963,6 +1159,10 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     return wide ? LaunchBatchedM<8, 8>(p, grouped, grid_b, stream) : LaunchBatchedM<4, 4>(p, grouped, grid_b, stream);
   }
 
+  if (RowsKernelServes(args, count)) {
+    if (kernel_name) *kernel_name = "fc_w4_rows_kernel";
+    return LaunchRows(p, args, count, grouped, stream);
+  }
   if (StripKernelServes(args, count)) {
     if (kernel_name) *kernel_name = "fc_w4_strip_kernel";
     return LaunchStrip(p, args, count, grouped, stream);

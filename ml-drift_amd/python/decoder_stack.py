@@ -19,7 +19,8 @@ import workloads as W
 
 
 class DecoderStack:
-    def __init__(self, layers=W.C5_LAYERS, max_tokens=128, seed=5, layer_shapes=None, device="cuda", keep_host=True):
+    def __init__(self, layers=W.C5_LAYERS, max_tokens=128, seed=5, layer_shapes=None, device="cuda", keep_host=True,
+                 decode_layout=False):
         import torch
         self.torch = torch
         self.layers = layers
@@ -47,7 +48,9 @@ class DecoderStack:
                 case["name"] = name
                 case["m"] = max_tokens
                 case["act"] = self.inputs[k]
-                desc, w = W.pack_fc_weights(case)
+                # decode_layout: the weights as a decode graph's ops ask for them (the prefill graph keeps
+                # its own packed copy)
+                desc, w = W.pack_fc_weights(case, decode_layout=decode_layout)
                 sc = M.scale_to_tensor(case["scale"], M.FLOAT16).view(np.float16)
                 w_dev = torch.from_numpy(w).to(device)
                 s_dev = torch.from_numpy(sc).to(device)

@@ -33,7 +33,7 @@ SYMBOLS = [
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
-    "mldhip_fc_int4_weights_desc_reference", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
+    "mldhip_fc_int4_weights_desc_reference", "mldhip_fc_int4_weights_desc_decode", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
     "mldhip_probe_launch",
 ]
 
@@ -143,11 +143,13 @@ def fc_int8_weights_desc(o, i):
     return d
 
 
-def fc_int4_weights_desc(o, i, reference=False):
-    """The layout this library asks for (output groups of 16 slices where the shape allows), or with
-    `reference` the reference's own choice (one output group)."""
+def fc_int4_weights_desc(o, i, reference=False, decode=False):
+    """The layout this library asks for (output groups of 16 slices where the shape allows), with
+    `reference` the reference's own choice (one output group), with `decode` the layout for ops that
+    run one token per launch (output groups of 2 slices for layers of a few thousand channels)."""
     d = WeightsDesc()
-    fn = lib().mldhip_fc_int4_weights_desc_reference if reference else lib().mldhip_fc_int4_weights_desc
+    fn = (lib().mldhip_fc_int4_weights_desc_reference if reference else
+          lib().mldhip_fc_int4_weights_desc_decode if decode else lib().mldhip_fc_int4_weights_desc)
     check(fn(o, i, C.byref(d)))
     return d
 

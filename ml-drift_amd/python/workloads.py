@@ -57,13 +57,13 @@ def make_fc_case(seed, m, k, n, weight_bits, tensor_dtype, groups=1, with_bias=F
     return case
 
 
-def pack_fc_weights(case, reference_layout=False, output_group=None):
+def pack_fc_weights(case, reference_layout=False, output_group=None, decode_layout=False):
     """Packs the case's weights for the FullyConnected op: in the layout the library asks for, or
     with `reference_layout` in the reference's own FullyConnected layout (one output group), or
     in output groups of `output_group` slices (1: the layout FullyConnectedOI reads)."""
     n, k = case["n"], case["k"]
     if case["weight_bits"] == 4:
-        desc = M.fc_int4_weights_desc(n, k, reference=reference_layout or output_group is not None)
+        desc = M.fc_int4_weights_desc(n, k, reference=reference_layout or output_group is not None, decode=decode_layout)
         if output_group is not None:
             desc.output_group_size = output_group
         return desc, M.rearrange_int8_as_uint4(case["w"], desc)

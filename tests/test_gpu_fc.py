@@ -447,7 +447,30 @@ def test_strip_kernel_group_sizes(oracle, group, k, n, groups, zp, bias):
                           with_bias=bias, with_zero_point=zp)
     with M.tuning(fc_group=group):
         assert M.fc_int4_weights_desc(n, k).output_group_size == group
-        run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
+        got = run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
+    # K split across work-groups (a second kernel adds the sums in split order): inside the bar too
+    for ksplit in (4, 7):
+        if k // 32 >= ksplit:
+            with M.tuning(fc_group=group, gemv_ksplit=ksplit):
+                run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
+
+
+def test_split_k_launches_repeat_bit_for_bit(oracle):
+    """50 launches in a row of a K-split GEMV (the down projection of the decoder stack): the same
+    bits every time."""
+    case = W.make_fc_case(seed=77, m=1, k=16384, n=2048, weight_bits=4, tensor_dtype=np.float16, groups=512)
+    dev = W.FcDevice(case)
+    dev.run()
+    assert dev.op.kernel_name == "fc_w4_strip_kernel"
+    first = dev.result()
+    check_fp(first, textbook(case), case, "textbook")
+    import torch
+    stream = torch.cuda.current_stream().cuda_stream
+    for i in range(50):
+        dev.out.zero_()
+        dev.op.launch(stream)
+        if i % 10 == 9:
+            assert np.array_equal(dev.result(), first), i
 
 
 @pytest.mark.parametrize("bits,k,n,groups", [(4, 4096, 2048, 1), (4, 1024, 1032, 32), (8, 2048, 2048, 1), (4, 171, 533, 1)])
@@ -496,3 +519,35 @@ def test_precision_f16_runs_with_float_accumulators(oracle, bits, m, k, n, group
     check_fp(got, ref, case, "textbook")
     half = oracle_fc(oracle, case, precision=oracle.PREC_F16).astype(np.float64)
     assert np.sqrt(np.mean((got - ref) ** 2)) <= np.sqrt(np.mean((half - ref) ** 2)) + 2.0 ** -12 * np.sqrt(np.mean(ref ** 2))
+
+
+@pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 64, False, True), (16384, 2048, 512, False, False),
+                                               (4096, 1536, 1, True, True), (512, 256, 16, True, False),
+                                               (2048, 16384, 64, False, False), (100, 72, 1, False, True),
+                                               (171 * 4, 536, 1, False, False), (8192, 2048, 64, False, True),
+                                               (40000, 64, 1, False, False)])
+def test_rows_kernel(oracle, k, n, groups, zp, bias):
+    """One token on the row-interleaved kernel over weights packed in output groups of 2 slices:
+    per-channel and group-wise scales, zero points, K shorter than a work-group's rows, K that needs
+    several passes, K that is no multiple of the rows per pass."""
+    case = W.make_fc_case(seed=k + n, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    print("rows kernel", k, n, groups, zp, bias, flush=True)
+    dev = W.FcDevice(case, output_group=2)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_rows_kernel", dev.op.kernel_name
+    dev.out.zero_()
+    dev.run()
+    assert np.array_equal(got, dev.result())
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    if k * n <= 1 << 27:
+        rest = oracle_fc(oracle, case).astype(np.float64)
+        check_fp(got, rest, case, "kernel restatement")
+        check_as_accurate_as(got, rest, ref, case, "fc_w4_rows_kernel")
+    for waves in (1, 4, 16):
+        with M.tuning(gemv_waves=waves):
+            dev.out.zero_()
+            dev.run()
+            check_fp(dev.result(), ref, case, "waves %d" % waves)

@@ -19,6 +19,12 @@ def stack():
     return DecoderStack(layers=LAYERS, max_tokens=128)
 
 
+@pytest.fixture(scope="module")
+def decode_stack():
+    """The same stack with the weights packed as the ops of a decode graph ask for them."""
+    return DecoderStack(layers=LAYERS, max_tokens=128, decode_layout=True)
+
+
 @pytest.mark.parametrize("tokens", [1, 128, 7])
 def test_stack_parity(stack, tokens):
     print("decoder stack, tokens =", tokens, flush=True)
@@ -36,6 +42,34 @@ def test_stack_parity(stack, tokens):
     stack.launch()
     for (layer, idx), got in first.items():
         assert np.array_equal(got, stack.result(layer, idx))
+
+
+@pytest.mark.parametrize("tokens", [1, 3, 128])
+def test_decode_layout_stack_parity(decode_stack, tokens):
+    """The decode layout: the 2048- and 256-channel layers in output groups of 2 slices (the
+    row-interleaved kernel at one token), the 16384-channel ones in groups of 16 (the strip kernel);
+    more tokens run on the general kernels over the same buffers."""
+    import mldhip as M
+    st = decode_stack
+    assert [M.fc_int4_weights_desc(n, k, decode=True).output_group_size for _, k, n in W.C5_LAYER] == [2, 2, 2, 2, 16, 16, 2]
+    st.set_tokens(tokens)
+    for fused in (True, False):
+        for out in st.outs:
+            out.zero_()
+        st.launch(fused=fused)
+        for layer in range(LAYERS):
+            for idx, case in enumerate(st.cases):
+                got = st.result(layer, idx)
+                check_fp(got, textbook(st.case(idx, layer=layer)), st.case(idx, layer=layer),
+                         "decode layout layer %d %s" % (layer, case["name"]))
+        if tokens == 1:
+            names = st.kernel_names()[:7]
+            assert names == ["fc_w4_rows_kernel"] * 4 + ["fc_w4_strip_kernel"] * 2 + ["fc_w4_rows_kernel"], names
+    first = [st.result(layer, idx) for layer in range(LAYERS) for idx in range(len(st.cases))]
+    st.launch(fused=False)
+    again = [st.result(layer, idx) for layer in range(LAYERS) for idx in range(len(st.cases))]
+    for a, b in zip(first, again):
+        assert np.array_equal(a, b)
 
 
 def test_stack_accounting(stack):
