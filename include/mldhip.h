@@ -443,7 +443,8 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
  * statically on every GPU it runs on (until the process ends).  Calls no hipMalloc / hipFree.
  * Same kernels and same results as mldhip_op_launch on an op of the same description.
  * Limits: o <= 65536 (MLDHIP_OUT_OF_RANGE beyond), an even number of 4-channel slices,
- * output_group_size = ceil(o/4) or 16 as mldhip_fc_create takes it.  All calls on one GPU share
+ * output_group_size = any even number of slices that divides ceil(o/4) (the reference's one group,
+ * 16, the decode layout's 2, ...).  All calls on one GPU share
  * that GPU's array: calls that overlap in time on one GPU (different streams) race; calls on
  * one stream are ordered.  The array needs no clearing between calls.
  *   src [ceil(i/4)][tokens][4] halfs, weights packed uint4, weights_scale [scale_groups][ceil(o/4)][4]

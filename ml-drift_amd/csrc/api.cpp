@@ -877,8 +877,8 @@ int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const vo
   if (ns % 2 != 0) return Fail(MLDHIP_UNIMPLEMENTED, "an odd number of 4-channel output slices is not served here");
   if (scale_groups < 1 || ks % scale_groups != 0 || (scale_groups > 1 && (ks / scale_groups) % 8 != 0))
     return Fail(MLDHIP_INVALID_ARGUMENT, "scale groups must be whole multiples of 32 input channels");
-  const bool native = IsNativeGroup(output_group_size) && o % 4 == 0 && ns % output_group_size == 0;
-  if (output_group_size != ns && !native)
+  // whole groups of an even number of slices (16-byte items of the packed rows), as the streaming kernels read them
+  if (output_group_size < 1 || ns % output_group_size != 0 || output_group_size % 2 != 0)
     return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
   const void* ptrs[5] = {src, weights, weights_scale, biases, dst};
   for (const void* ptr : ptrs)

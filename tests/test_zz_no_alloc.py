@@ -10,9 +10,9 @@ import mldhip as M
 import workloads as W
 
 
-def run_pair(case, reference_layout):
+def run_pair(case, reference_layout, output_group=None):
     import torch
-    dev = W.FcDevice(case, reference_layout=reference_layout)
+    dev = W.FcDevice(case, reference_layout=reference_layout, output_group=output_group)
     dev.run()
     ref = dev.result()
     kernel = dev.op.kernel_name
@@ -39,6 +39,17 @@ def test_no_alloc_matches_op_launch(reference_layout):
     two = W.make_fc_case(seed=73, m=2, k=4096, n=1536, weight_bits=4, tensor_dtype=np.float16, groups=1, with_bias=True)
     print("no-alloc", two["k"], two["n"], reference_layout, flush=True)
     run_pair(two, reference_layout)
+
+
+def test_no_alloc_decode_layout():
+    """Weights in output groups of 2 slices (the decode ops' layout) through the same entry point: the
+    row-interleaved kernel, which needs no scratch; 8 slices per group on the streaming kernel."""
+    case = W.make_fc_case(seed=74, m=1, k=16384, n=2048, weight_bits=4, tensor_dtype=np.float16, groups=512, with_bias=True)
+    print("no-alloc, groups of 2 slices", flush=True)
+    assert run_pair(case, False, output_group=2) == "fc_w4_rows_kernel"
+    three = W.make_fc_case(seed=75, m=3, k=2048, n=1024, weight_bits=4, tensor_dtype=np.float16, groups=64)
+    run_pair(three, False, output_group=2)
+    run_pair(three, False, output_group=8)
 
 
 def test_no_alloc_rejects():
