@@ -742,6 +742,10 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       if (int rc = BuildFcArgs(op, &a)) return rc;
       // runtime channel bounds are served by the unspecialised kernel
       const bool force_generic = GetTuning().force_generic > 0 || a.params != nullptr;
+      // packed groups: the matrix-core GEMM with one launch plane per matrix where it serves the shape
+      if (GetTuning().force_generic <= 0 && FcW4MfmaPackedSupported(a)) {
+        e = LaunchFcW4Mfma(a, stream, &op->last_kernel);
+      } else
       // batched weights by runtime ids: the streaming GEMVs, else the unspecialised kernel
       if (a.batch_ids != nullptr) {
         if (!force_generic && FcW4StreamSupported(a))

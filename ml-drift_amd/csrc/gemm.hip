@@ -87,6 +87,11 @@ struct GemmParams {
   int xcd_m;        // fp16 path: the 8 XCDs form an xcd_m x (8 / xcd_m) grid over (token tiles, channel tiles)
   int gate_activation;  // gated fp16 launch: MLDHIP_GATE_*
   int dual;             // fp16 path: a work-group owns two neighbouring channel tiles
+  // fp16 path, packed groups (ConvRuntimeCheckDesc::PackedGroups): blockIdx.z = weight matrix g of
+  // pg_groups; its tokens are min(pg_params[pg_offset + g], pg_max) many from token
+  // pg_params[pg_offset + pg_groups + g] of the one source row.  pg_groups = 0: not set.
+  const int32_t* pg_params;
+  int pg_offset, pg_groups, pg_max;
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -591,7 +596,18 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // same few activation tiles while the weights stream through.
   const int tiles_n_all = p.seg[MULTI ? p.segments - 1 : 0].tile_end;  // channel tiles of all matrices of the launch
   const int tiles_n = DUAL ? (tiles_n_all + 1) / 2 : tiles_n_all;        // channel tiles of the grid
-  const int tiles_m = (p.m + BM - 1) / BM;
+  // Packed groups: this work-group's matrix and the run of tokens it multiplies (else: all tokens).
+  int m_lo = 0, m_hi = p.m, pg_e = 0;
+  int tiles_m = (p.m + BM - 1) / BM;
+  if (p.pg_groups > 0) {
+    pg_e = blockIdx.z;
+    const int size = min(p.pg_params[p.pg_offset + pg_e], p.pg_max);
+    const int off = p.pg_params[p.pg_offset + p.pg_groups + pg_e];
+    if (off < 0) return;
+    m_lo = off;
+    m_hi = min(off + size, p.m);
+    tiles_m = (p.pg_max + BM - 1) / BM;
+  }
   const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
   const int xm = p.xcd_m, xn = 8 / xm;
   const int rect_m = (tiles_m + xm - 1) / xm, rect_n = (tiles_n + xn - 1) / xn;
@@ -615,7 +631,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int si = locate(tn);
   const W4Segment& sg = p.seg[GATED ? half : (MULTI ? si : 0)];
   const int slice0 = tn * (BN / 4);  // first output slice of the tile
-  const int m0 = tm * BM;
+  const int m0 = m_lo + tm * BM;
+  if (m0 >= m_hi) return;  // (packed groups: a tile beyond the group's size; the whole work-group leaves)
   const int nsi = slice0 + i32;
   const bool n_ok = tile_ok && nsi < sg.ns;
 
@@ -639,8 +656,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const uint32_t x_end = min((uint64_t)p.b_bytes, (uint64_t)k_slices_end * row_x);
 
   constexpr uint32_t kOob = 0x7FFFFFF0u;
+  // packed groups: matrix pg_e of the batched buffers (weights one matrix after the other, scales
+  // [group][matrix][Ns][4])
+  const uint8_t* w_base = sg.w4 + (size_t)pg_e * sg.a_bytes;
+  const __half* s_base = sg.scale + (size_t)pg_e * sg.ns * 4;
+  const __half* z_base = (ZP ? sg.zp : sg.scale) + (size_t)pg_e * sg.ns * 4;
+  const uint32_t s_bytes = sg.s_bytes - (uint32_t)pg_e * (uint32_t)sg.ns * 8u;
   const __amdgpu_buffer_rsrc_t rsrc_w =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sg.w4), 0, w_end, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(w_base), 0, w_end, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_x =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, x_end, 0x00020000);
   // Second descriptors, one K-slice row further: the loads of rows 2q and 2q+1 share an offset.
@@ -652,12 +675,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   };
   const uint32_t w1_bytes = __builtin_amdgcn_readfirstlane(w_end > row_w ? w_end - row_w : 0u);
   const uint32_t x1_bytes = __builtin_amdgcn_readfirstlane(x_end > row_x ? x_end - row_x : 0u);
-  const __amdgpu_buffer_rsrc_t rsrc_w1 = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(sg.w4, row_w), 0, w1_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w1 = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(w_base, row_w), 0, w1_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_x1 = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.act, row_x), 0, x1_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_s =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(sg.scale), 0, sg.s_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(s_base), 0, s_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_z =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(ZP ? sg.zp : sg.scale), 0, sg.s_bytes, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(z_base), 0, s_bytes, 0x00020000);
 
   // Per-lane byte offsets of the next step to fetch; each fetch advances them by one step.
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
@@ -674,9 +697,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
 #pragma unroll
   for (int i = 0; i < NX; ++i) {
     const int mi = token(PAIR ? 2 * i : i);
-    vx[i] = mi < p.m ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
+    vx[i] = mi < m_hi ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_x + (uint32_t)mi * 8u : kOob;
   }
-  const uint32_t group_bytes = (uint32_t)sg.ns * 8u;  // one scale group: [Ns][4] halfs
+  const uint32_t group_bytes = (uint32_t)sg.ns * 8u * (uint32_t)max(p.pg_groups, 1);  // one scale group: [matrices][Ns][4] halfs
 
   wblk_t rw[U][2];
   u32x2 rsc[U], rzp[U], rx[U][NX][2];
@@ -880,9 +903,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
             sum_b.w += o.w;
           }
           if (DUAL) {
-            if (mi < p.m && slice0_a + slice_l < sga.ns) store(sga, slice0_a + slice_l, mi, sum);
-            if (mi < p.m && tile_b_ok && slice0_b + slice_l < sgb.ns) store(sgb, slice0_b + slice_l, mi, sum_b);
-          } else if (mi < p.m && slice0 + slice_l < sga.ns) {
+            if (mi < m_hi && slice0_a + slice_l < sga.ns) store(sga, slice0_a + slice_l, mi, sum);
+            if (mi < m_hi && tile_b_ok && slice0_b + slice_l < sgb.ns) store(sgb, slice0_b + slice_l, mi, sum_b);
+          } else if (mi < m_hi && slice0 + slice_l < sga.ns) {
             const int slice = slice0 + slice_l;
             const float g[4] = {sum.x, sum.y, sum.z, sum.w}, up[4] = {sum_b.x, sum_b.y, sum_b.z, sum_b.w};
             __half h[4];
@@ -898,7 +921,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
             o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
             *reinterpret_cast<u32x2*>(sga.dst + ((size_t)slice * p.m + mi) * 4) = o;
           }
-        } else if (mi < p.m && slice0 + slice_l < sg.ns) {
+        } else if (mi < m_hi && slice0 + slice_l < sg.ns) {
           store(sg, slice0 + slice_l, mi, sum);
         }
       }
@@ -1070,6 +1093,9 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
   const bool gated = gate_activation != 0;
   if (gated && count != 2) return hipErrorInvalidValue;
   const FcArgs& a = args[0];
+  // packed groups: one launch plane per weight matrix, token tiles sized for the largest group
+  const bool packed = a.params != nullptr && a.packed_params_offset >= 0;
+  if (packed && (count != 1 || gated || a.weights_batch < 1 || a.packed_max_group_size < 1)) return hipErrorInvalidValue;
   GemmParams p = {};
   p.gate_activation = gate_activation;
   p.segments = count;
@@ -1108,7 +1134,7 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     if (sg.ns % sg.group != 0) return hipErrorInvalidValue;  // whole groups only
     if (args[i].weight_bits != a.weight_bits) return hipErrorInvalidValue;
     sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * (a.weight_bits == 8 ? 16 : 8));
-    sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8);
+    sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8 * (packed ? a.weights_batch : 1));
     if (gated) {
       tiles_n = DivUp(args[i].n, 128);  // a tile holds the same 128 channels of both matrices
       if (args[i].n != a.n) return hipErrorInvalidValue;
@@ -1123,9 +1149,28 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
   if (kernel_name)
     *kernel_name = gated ? (a.weight_bits == 8 ? "fc_w8_gated_mfma_gemm_kernel" : "fc_w4_gated_mfma_gemm_kernel")
                          : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
+  const Tuning& tune = GetTuning();
+  if (packed) {
+    p.pg_params = a.params;
+    p.pg_offset = a.packed_params_offset;
+    p.pg_groups = a.weights_batch;
+    p.pg_max = std::min(a.packed_max_group_size, a.m);
+    p.ksplit = 1;
+    int fm = p.pg_max <= 32 ? 1 : 2;
+    if (tune.gemm_fm == 1 || tune.gemm_fm == 2) fm = tune.gemm_fm;
+    const int tiles_m = DivUp(p.pg_max, fm * 32);
+    p.xcd_m = 1;  // few token tiles per matrix: the XCDs share the channel tiles
+    if (tune.gemm_xcd_m == 1 || tune.gemm_xcd_m == 2 || tune.gemm_xcd_m == 4 || tune.gemm_xcd_m == 8) p.xcd_m = tune.gemm_xcd_m;
+    const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), 1, a.weights_batch);
+    const bool zp = p.seg[0].zp != nullptr;
+    if (fm == 2)
+      LaunchDirect<2, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);
+    else
+      LaunchDirect<1, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);
+    return hipGetLastError();
+  }
   // token tile and K split follow the launch as a whole (all channels of all matrices)
   int fm = W4TokenBlocks(a.m, n_total);
-  const Tuning& tune = GetTuning();
   if (tune.gemm_fm > 0) fm = tune.gemm_fm == 1 ? 1 : (tune.gemm_fm == 4 && a.m % 2 == 0 ? 4 : 2);
   p.ksplit = 1;
   if (fm == W4TokenBlocks(a.m, n_total)) p.ksplit = W4KSplit(a.m, a.k, n_total);
@@ -1170,6 +1215,16 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
 }  // namespace
 
 bool FcW4MfmaSupported(const FcArgs& a) { return a.m > kGemvMaxTokens && DirectGemmShapeOk(a); }
+
+// Packed groups on the matrix cores: batched weights in the one-group layout, no channel bounds.
+bool FcW4MfmaPackedSupported(const FcArgs& a) {
+  if (a.params == nullptr || a.packed_params_offset < 0 || a.batch_ids != nullptr) return false;
+  if (a.src_end_ch_index >= 0 || a.dst_end_ch_index >= 0) return false;
+  if (EffectiveGroup(a.group, DivUp(a.n, 4)) != DivUp(a.n, 4)) return false;
+  // 32-bit offsets into the scale tensor of all matrices
+  if ((size_t)(a.scale_kind == kScaleBlock ? a.groups : 1) * a.weights_batch * DivUp(a.n, 4) * 8 >= 0x7FFFFFF0u) return false;
+  return DirectGemmShapeOk(a);
+}
 
 hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name) {
   return LaunchDirectGemm(args, count, 0, nullptr, stream, kernel_name);

@@ -168,6 +168,7 @@ hipError_t LaunchConvInt8(const ConvInt8Args& a, hipStream_t stream, const char*
 
 // Multi-token FullyConnected with uint4 or uint8 weights on the MFMA units (fp16 tensors).
 bool FcW4MfmaSupported(const FcArgs& a);
+bool FcW4MfmaPackedSupported(const FcArgs& a);  // packed groups: launched through LaunchFcW4Mfma
 hipError_t LaunchFcW4Mfma(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
 hipError_t LaunchFcW4MfmaFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);

@@ -154,6 +154,14 @@ def fc_int4_weights_desc(o, i, reference=False, decode=False):
     return d
 
 
+_forced_generic = [False]
+
+
+def get_tuning_forced_generic():
+    """True inside a `tuning(force_generic=1)` block."""
+    return _forced_generic[0]
+
+
 class tuning:
     """Context manager: overrides launch heuristics (mldhip_set_tuning) inside the block."""
 
@@ -163,11 +171,15 @@ class tuning:
     def __enter__(self):
         for name, value in self.knobs.items():
             check(lib().mldhip_set_tuning(name.encode(), int(value)))
+        if int(self.knobs.get("force_generic", 0)) > 0:
+            _forced_generic[0] = True
         return self
 
     def __exit__(self, *exc):
         for name in self.knobs:
             check(lib().mldhip_set_tuning(name.encode(), -1))
+        if "force_generic" in self.knobs:
+            _forced_generic[0] = False
         return False
 
 

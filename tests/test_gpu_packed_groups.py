@@ -47,7 +47,13 @@ def run_device(c, td, sizes=None, offsets=None, max_group_size=None, params_offs
     print("packed groups", c["bits"], tokens, k, n, batch, c["groups"], td.__name__, flush=True)
     op.launch(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert op.kernel_name == "fc_generic_kernel", op.kernel_name
+    # fp16 tensors run on the matrix cores (one launch plane per matrix), fp32 on the unspecialised kernel
+    want = "fc_generic_kernel" if td == np.float32 or M.get_tuning_forced_generic() else "fc_w%d_mfma_gemm_kernel" % c["bits"]
+    assert op.kernel_name == want, op.kernel_name
+    first = out.clone()
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(first, out)
     return W.from_slices(out.cpu().numpy().astype(np.float32), n)
 
 
@@ -84,6 +90,28 @@ def test_mixture_prefill_shapes(oracle, bits, width, per_item, k, n, batch, grou
     if width * per_item * k * n <= 1 << 28:
         rest = run_packed_groups_oracle(oracle, c, oracle.PREC_F32 if td == np.float32 else oracle.PREC_F32F16)
         check(rows, rest.astype(np.float64), td, k)
+    if td == np.float16:  # the same op on the unspecialised kernel
+        with M.tuning(force_generic=1):
+            slow = unpack_groups(c, run_device(c, td, params_offset=3))
+        check(slow, packed_groups_expected(oracle, c, td), td, k)
+
+
+@pytest.mark.parametrize("fm", [1, 2])
+def test_groups_of_every_size_on_the_matrix_cores(oracle, fm):
+    """Group sizes 0, 1, odd, one token tile exactly, several tiles, beyond max_group_size; offsets that
+    are odd and that leave gaps; both token tiles (32 and 64 tokens).  fp16, against the restatement."""
+    c = make_packed_groups_case(21, 300, 1, 256, 136, 8, 4, 8, True)
+    sizes = np.array([0, 1, 33, 64, 65, 100, 7, 40], np.int32)
+    # (runs that do not overlap; the last one is cut at the end of the tensor)
+    offsets = np.array([0, 1, 3, 40, 110, 177, 258, 266], np.int32)
+    with M.tuning(gemm_fm=fm):
+        got = run_device(c, np.float16, sizes=sizes, offsets=offsets, max_group_size=80, fill=7.0)
+    before = oracle.f32_to_f16_bits(np.full(((136 + 3) // 4, 300, 4), 7.0, np.float32))
+    ref = run_packed_groups_oracle(oracle, c, oracle.PREC_F32F16, max_group_size=80, dst_before=before, sizes=sizes, offsets=offsets)
+    assert np.array_equal(got == 7.0, ref == 7.0)
+    written = ref != 7.0
+    rms = np.sqrt(np.mean(ref[written] ** 2))
+    assert np.abs(got - ref)[written].max() <= FP16_TOL * rms
 
 
 def test_tokens_outside_every_group_are_not_written(oracle):
