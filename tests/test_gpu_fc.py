@@ -66,6 +66,14 @@ def check_fp(got, ref, case, label=""):
     return err / rms
 
 
+def restatement_affordable(case, tokens=None):
+    """The oracle's eight-channel path (fp16 tensors, no zero points) restates about 5e9 multiply-adds
+    per second on 8 cores, the one-channel path 30 times fewer."""
+    work = (case["m"] if tokens is None else tokens) * case["k"] * case["n"]
+    fast = case["tensor_dtype"] == np.float16 and case["zero_point"] is None
+    return work <= (1 << 33 if fast else 1 << 27)
+
+
 def check_as_accurate_as(got, restatement, exact, case, label=""):
     """The sharp bar beside the stated tolerance: measured against the float64 result, the GPU's
     error (RMS and maximum over the outputs) is no larger than 1.5 x the error of the reference's own
@@ -113,7 +121,7 @@ def run_case(oracle, case, expect_kernel=None, tune=None, layouts=None):
             assert np.array_equal(got, dev.result())
         ref_tb = textbook(case)
         check_fp(got, ref_tb, case, "textbook")
-        if case["m"] * case["k"] * case["n"] <= 1 << 27:
+        if restatement_affordable(case):
             rest = oracle_fc(oracle, case).astype(np.float64)
             check_fp(got, rest, case, "kernel restatement")
             check_as_accurate_as(got, rest, ref_tb, case, dev.op.kernel_name)

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 import mldhip as M
 import workloads as W
 from refmath import textbook
-from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc
+from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, restatement_affordable
 
 
 def synthetic(shape, index_offset=0):
@@ -38,7 +38,7 @@ def run_grouped(oracle, case, group, expect_kernel=None):
     assert np.array_equal(got, dev.result())
     ref = textbook(case)
     check_fp(got, ref, case, "textbook")
-    if case["m"] * case["k"] * case["n"] <= 1 << 27:
+    if restatement_affordable(case):
         rest = oracle_fc(oracle, case).astype(np.float64)
         check_fp(got, rest, case, "kernel restatement")
         check_as_accurate_as(got, rest, ref, case, dev.op.kernel_name)

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 import mldhip as M
 import workloads as W
-from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, textbook
+from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, restatement_affordable, textbook
 
 FP16_TOL = 2e-2
 
@@ -54,7 +54,7 @@ def test_w4_gemm_shapes(oracle, m, k, n, groups):
                           with_bias=(m % 2 == 1))
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
-    if m * k * n <= 1 << 26:
+    if restatement_affordable(case):
         check_restatement(oracle, got, case, "kernel restatement")
 
 
@@ -65,7 +65,7 @@ def test_w4_gemm_zero_points(oracle, m, k, n, groups):
                           with_bias=True, with_zero_point=True)
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
-    if m * k * n <= 1 << 26:
+    if restatement_affordable(case):
         check_restatement(oracle, got, case, "kernel restatement")
 
 
@@ -93,9 +93,9 @@ def test_w8_gemm_shapes(oracle, m, k, n, groups, zp):
                           with_bias=(m % 2 == 1), with_zero_point=zp)
     got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
-    small = min(m, 64)
+    small = m if restatement_affordable(case) else min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
-    if small * k * n <= 1 << 26:
+    if restatement_affordable(sub):
         check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
@@ -134,9 +134,9 @@ def test_gemm_two_tiles_per_work_group(oracle, bits, m, k, n, groups, zp):
     with M.tuning(gemm_dual=1):
         got = run_w4(case)
     check_fp(got, textbook(case), case, "textbook")
-    small = min(m, 64)
+    small = m if restatement_affordable(case) else min(m, 64)
     sub = dict(case, m=small, act=case["act"][:small])
-    if small * k * n <= 1 << 26:
+    if restatement_affordable(sub):
         check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
@@ -250,11 +250,10 @@ def test_config3_prefill_gemm(oracle):
     got = run_w4(case)
     rel = check_fp(got, textbook(case), case, "textbook")
     print("c3 max|err|/rms = %.3e" % rel)
-    # a slab of outputs against the restatement of the generated kernel
-    sub = dict(case, n=64, w=case["w"][:64], scale=case["scale"][:64])
-    ref = oracle_fc(oracle, sub).astype(np.float64)
-    rms = np.sqrt(np.mean(ref ** 2))
-    assert np.abs(got[:, :64] - ref).max() <= FP16_TOL * rms
+    # every output of every tile against the restatement of the generated kernel (8.6e9 multiply-adds:
+    # a few seconds on the oracle's eight-channel path), to the stated tolerance and to the bar "no less
+    # accurate than the reference's kernel"
+    check_restatement(oracle, got, case, "kernel restatement, all 512 x 4096 outputs")
 
 
 def test_config5_prefill_shapes(oracle):
