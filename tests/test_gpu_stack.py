@@ -119,13 +119,15 @@ def test_fused_launch_matches_single_launches(stack):
                 pos += 1
 
 
-def test_graph_replays_match_eager():
+@pytest.mark.parametrize("decode_layout", [False, True])
+def test_graph_replays_match_eager(decode_layout):
     """A decode step and a prefill step captured into a graph: several replays, with eager work
     and synchronisations in between, must reproduce the eager results bit for bit (launches
-    allocate nothing after the first eager pass and record no memset nodes)."""
+    allocate nothing and record no memset nodes); in the layout for both graphs and in the decode
+    ops' layout."""
     import torch
     from decoder_stack import DecoderStack
-    st = DecoderStack(layers=2, max_tokens=128)
+    st = DecoderStack(layers=2, max_tokens=128, decode_layout=decode_layout)
     for tokens in (1, 128):
         st.set_tokens(tokens)
         st.launch()
