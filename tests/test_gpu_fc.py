@@ -443,6 +443,39 @@ def test_random_shapes_sweep(oracle):
     assert len(seen) >= 4
 
 
+def test_random_layouts_sweep(oracle):
+    """Seeded sweep over the weights layouts the op accepts (output groups of any size that divides
+    the output slices: 1 is the FullyConnectedOI layout, 2 the decode layout, all slices the
+    reference's FullyConnected layout), crossed with token counts, ragged K / N and scale
+    groupings: every result against the textbook reference at the fp16 bar."""
+    rng = np.random.default_rng(77)
+    seen = {}
+    for it in range(40):
+        m = int(rng.choice([1, 1, 1, 2, 3, 4, 5, 16, 33, 64, 130]))
+        bits = int(rng.choice([4, 4, 4, 8]))
+        k = int(rng.choice([64, 100, 171, 512, 1000, 2048, 4096]))
+        n = int(rng.choice([8, 24, 64, 152, 536, 1024, 2056, 4096, 8200]))
+        ns = -(-n // 4)
+        divisors = [g for g in range(1, ns + 1) if ns % g == 0]
+        group = int(rng.choice([1, 2, ns, divisors[int(rng.integers(len(divisors)))]]))
+        groups = 1
+        if k % 32 == 0 and rng.random() < 0.6:
+            groups = k // int(rng.choice([32, 64, k])) if k >= 64 else 1
+        zp = bool(rng.random() < 0.3)
+        bias = bool(rng.random() < 0.5)
+        case = W.make_fc_case(seed=3000 + it, m=m, k=k, n=n, weight_bits=bits, tensor_dtype=np.float16, groups=groups,
+                              with_zero_point=zp, with_bias=bias)
+        print("layout sweep", it, dict(m=m, k=k, n=n, bits=bits, group=group, of=ns, groups=groups, zp=zp, bias=bias),
+              flush=True)
+        dev = W.FcDevice(case, output_group=group)
+        dev.run()
+        got = dev.result()
+        seen[dev.op.kernel_name] = seen.get(dev.op.kernel_name, 0) + 1
+        check_fp(got, textbook(case), case, "layout sweep %d (group %d, %s)" % (it, group, dev.op.kernel_name))
+    print("kernels exercised:", seen)
+    assert len(seen) >= 4
+
+
 @pytest.mark.parametrize("group", [4, 8, 16])
 @pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 64, False, True), (16384, 2048, 512, False, False),
                                                (4096, 1536, 1, True, True), (512, 256, 1, False, False),
