@@ -105,6 +105,9 @@ struct mldhip_op {
   float* partial = nullptr;
   size_t partial_floats = 0;
   const char* last_kernel = "";
+  // bytes every object needs at the current shape (kept up to date by create and set_shape, so that
+  // a launch checks its bindings without touching the heap)
+  std::vector<size_t> need_src, need_dst;
 
   void AddSrc(const char* name) {
     src_names.emplace_back(name);
@@ -120,6 +123,8 @@ struct mldhip_op {
 };
 
 extern "C" {
+
+static void UpdateRequiredSizes(mldhip_op* op);
 
 const char* mldhip_last_error(void) { return g_error.c_str(); }
 const char* mldhip_version(void) { return "mldhip 0.1 (gfx950)"; }
@@ -400,7 +405,7 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
       return Fail(MLDHIP_INVALID_ARGUMENT, "scale_zp_shape.o must be 1 or the output channel count");
     if (d->scale_o == 1 && d->scale_i != 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "group-wise scales need one row per output channel");
-    if (d->scale_i > 1 && (d->i % (4 * d->scale_i)) != 0)
+    if (d->scale_i > 1 && (d->scale_i > d->i / 4 || (d->i % (4 * d->scale_i)) != 0))
       return Fail(MLDHIP_INVALID_ARGUMENT, "input channels must split into scale groups of whole 4-channel slices");
     if (d->has_zero_point_tensor && d->scale_o * d->scale_i == 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "a zero-point tensor needs a scale tensor of the same shape");
@@ -469,6 +474,7 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
       return rc;
     }
   }
+  UpdateRequiredSizes(op);
   *out = op;
   return MLDHIP_OK;
 }
@@ -495,6 +501,7 @@ int mldhip_quantization_create(const mldhip_quant_desc* d, mldhip_op** out) {
   op->AddSrc("src_tensor");
   op->AddDst("dst_tensor");
   op->AddDst("dst_params");
+  UpdateRequiredSizes(op);
   *out = op;
   return MLDHIP_OK;
 }
@@ -539,6 +546,7 @@ int mldhip_conv_int8_create(const mldhip_conv_int8_desc* d, mldhip_op** out) {
     }
   }
   op->AddDst("dst_tensor");
+  UpdateRequiredSizes(op);
   *out = op;
   return MLDHIP_OK;
 }
@@ -584,6 +592,7 @@ int mldhip_op_set_shape(mldhip_op* op, int b, int h, int w) {
   op->b = b;
   op->h = h;
   op->w = w;
+  UpdateRequiredSizes(op);
   return MLDHIP_OK;
 }
 
@@ -641,9 +650,10 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
   }
 }
 
+static void UpdateRequiredSizes(mldhip_op* op) { RequiredSizes(op, &op->need_src, &op->need_dst); }
+
 static int CheckBindings(const mldhip_op* op) {
-  std::vector<size_t> need_src, need_dst;
-  RequiredSizes(op, &need_src, &need_dst);
+  const std::vector<size_t>&need_src = op->need_src, &need_dst = op->need_dst;
   for (size_t i = 0; i < need_src.size(); ++i) {
     if (!op->src_ptr[i]) return Fail(MLDHIP_FAILED_PRECONDITION, "src object '" + op->src_names[i] + "' is not bound");
     if (op->src_bytes[i] < need_src[i])
@@ -858,6 +868,7 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
                 "type, symmetric weights and scale groups the gated kernels serve (int8 weights: above 4 tokens)");
   const size_t need = (size_t)DivUp(args[0].n, 4) * 4 * args[0].m * sizeof(uint16_t);
   if (dst_bytes < need) return Fail(MLDHIP_INVALID_ARGUMENT, "dst is too small for the gated output");
+  if (reinterpret_cast<uintptr_t>(dst) % 16 != 0) return Fail(MLDHIP_INVALID_ARGUMENT, "dst is not 16-byte aligned");
   const char* name = nullptr;
   hipStream_t stream = static_cast<hipStream_t>(stream_ptr);
   // 1..2 tokens: the streaming GEMV pair; more: the matrix-core GEMM with the gated epilogue
