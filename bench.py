@@ -42,11 +42,12 @@ def parse():
                    help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
                         "kernels away from the launch-bound regime)")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
-    p.add_argument("--layout", default="default", choices=["default", "library", "reference"],
+    p.add_argument("--layout", default="default", choices=["default", "library", "reference", "decode"],
                    help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
                         "slices; the default) or in the reference's own FullyConnected layout (one output group). "
                         "c5-decode: the weights as mldhip_fc_int4_weights_desc_decode asks for them (the default) or, "
-                        "with 'library', in the one layout that serves decode and prefill ops alike")
+                        "with 'library', in the layout mldhip_fc_int4_weights_desc asks for; c5-prefill with 'decode': "
+                        "the prefill step over the decode ops' layout (one copy of the weights for both graphs)")
     p.add_argument("--tune", default="", help="tuning knobs for the run, e.g. gemv_ksplit=1,gemm_dual=0 (mldhip_set_tuning)")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-graph", action="store_true", help="time an eager launch loop instead of a graph replay")
@@ -289,7 +290,7 @@ def run_other(args, torch, M, W):
         tokens = 1 if args.workload == "c5-decode" else max(5, args.tokens)
         # a decode step runs over the weights as a decode graph's ops ask for them (--layout library:
         # the one layout that serves both graphs)
-        decode_layout = tokens == 1 and args.layout != "library"
+        decode_layout = (tokens == 1 and args.layout != "library") or args.layout == "decode"
         st = DecoderStack(max_tokens=max(128, tokens), keep_host=False, decode_layout=decode_layout)
         st.set_tokens(tokens)
         wall, us, reg = time_graph(torch, stream, lambda s, i: st.launch(s), args.steps, args.warmup)
