@@ -206,7 +206,9 @@ def run_other(args, torch, M, W):
         # weights exist twice, so a matrix comes back after 470 MB of other weights.
         m, k, n, experts, top = 1, 4096, 14336, 8, 2
         ns = (n + 3) // 4
-        desc = M.fc_int4_weights_desc(n, k, reference=True)  # batched weights: one output group
+        # the matrices in the layout mldhip_fc_int4_weights_desc asks for (--layout reference: one output
+        # group, one matrix after the other, as the reference's kernel reads them)
+        desc = M.fc_int4_weights_desc(n, k, reference=args.layout == "reference")
         rng = np.random.default_rng(0)
         act = torch.from_numpy(W.to_slices(rng.standard_normal((m, k)).astype(np.float16))).cuda()
         scale = torch.from_numpy(M.scale_to_tensor_batched(
@@ -231,6 +233,7 @@ def run_other(args, torch, M, W):
                    dtype="u4 weights x f16 activations, f32 accumulate",
                    config=dict({"workload": "moe: FullyConnected with batched weights by runtime ids, 1 token, 2 of 8 "
                                             "matrices K=4096 N=14336 int4 per-channel, fp16 act/out",
+                                "weights_layout": "kOSpatialIOGroupI4O4, output_group_size %d" % desc.output_group_size,
                                 "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes}, **reg),
                    roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),

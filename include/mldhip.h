@@ -316,8 +316,11 @@ int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);
 
 /* CreateFullyConnectedWeightsBatchIds (common/kernels/fully_connected.cc:1174-1216): the
  * FullyConnected of a mixture-of-experts layer (common/gpu_model_builder_moe_util.cc:232-291).
- * ExternalWeights::shape = OHWI(o, weights_batch, 1, i): `weights_batch` matrices packed one
- * after the other (pack OHWI(o, weights_batch, 1, i) with the same WeightsDescription);
+ * ExternalWeights::shape = OHWI(o, weights_batch, 1, i): `weights_batch` matrices, packed as the
+ * rearrange functions pack OHWI(o, weights_batch, 1, i) with the op's WeightsDescription: one
+ * matrix after the other when the description has one output group (what the reference's kernel
+ * reads, fully_connected.cc:493-496), else the matrices of an output group one after the other
+ * ([o / (4 * group)][weights_batch][ceil(i/4)][group] blocks, weights_conversion.cc:139-185);
  * scale_zp_shape = OHWI(scale_o, weights_batch, 1, scale_i), as a tensor
  * [scale_i][weights_batch][ceil(o/4)][4] (mldhip_scale_to_tensor_batched).  Row y of the dst
  * tensor (h rows of w tokens; mldhip_op_set_shape(op, 1, h, w)) is the FullyConnected of source

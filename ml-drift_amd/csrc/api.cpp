@@ -385,7 +385,9 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     // One output group is the layout of FullyConnected (fully_connected.cc:1073-1086); groups of one
     // slice are the layout FullyConnectedOI reads (linear_i4o4 = dst_s * src_slices + src_s,
     // fully_connected_oi.cc:122-133); any other whole number of groups is addressed the same way.
-    const bool whole_groups = wd.output_group_size > 0 && ns % wd.output_group_size == 0 && !batch_ids;
+    // Batched weights: as the packers lay out an OHWI shape whose height is the batch (the matrices
+    // of an output group one after the other; with one group, one matrix after the other).
+    const bool whole_groups = wd.output_group_size > 0 && ns % wd.output_group_size == 0;
     if (wd.output_group_size != ns && !whole_groups)
       return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
   }

@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
     act_tok0 = dst_tok0 = (size_t)max(offset, 0);
     if (offset < 0 || tok0 >= tok_count) return;  // (the whole work-group: no barrier is left waiting)
   }
-  const uint8_t* weights = p.weights + (size_t)wb * p.ks * p.ns * (WBITS == 8 ? 16 : 8);
+  const uint8_t* weights = p.weights;  // (matrix wb: through the block index)
 
   float acc[TB][4];
 #pragma unroll
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
           if (zp) z[c] = LoadF(zp, sidx + c);
         }
       }
-      const size_t blk = BlockIndex(ks, ds, p.ks, p.ns, p.wgroup);
+      const size_t blk = BatchedBlockIndex(ks, ds, wb, p.weights_batch, p.ks, p.ns, p.wgroup);
       float wf[4][4];
       if (WBITS == 8) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(weights + blk * 16);
@@ -222,7 +222,6 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
   const int row = blockIdx.z;
   int wb = batch.ids ? batch.ids[row] : 0;
   wb = min(max(wb, 0), batch.weights_batch - 1);
-  weights += (size_t)wb * ks_n * ns * (WBITS == 8 ? 16 : 8);
   const size_t act_stride = (size_t)batch.src_rows * m, dst_stride = (size_t)batch.rows * m;
   const size_t act_tok0 = (size_t)min(row, batch.src_rows - 1) * m, dst_tok0 = (size_t)row * m;
   int acc[TB][4];
@@ -235,7 +234,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
   if (ds < ns_end) {
 #pragma unroll 4
     for (int ks = ty; ks < ks_end; ks += kKl) {
-      const size_t blk = BlockIndex(ks, ds, ks_n, ns, batch.group);
+      const size_t blk = BatchedBlockIndex(ks, ds, wb, batch.weights_batch, ks_n, ns, batch.group);
       uint32_t w0, w1, w2, w3;  // per output channel: the 4 input-channel values, one per byte
       if (WBITS == 4) {
         const u32x2 w = *reinterpret_cast<const u32x2*>(weights + blk * 8);

@@ -69,8 +69,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
   int wb = BATCHED ? p.batch.ids[brow] : 0;
   if (BATCHED) wb = min(max(wb, 0), p.batch.weights_batch - 1);
   // column of this lane: with output groups, the rows of a group lie one after the other
-  const u32x4* weights = p.weights + (BATCHED ? (size_t)wb * p.ks * p.row_u4 : 0) +
-                         ((size_t)(item / p.gu4) * p.ks * p.gu4 + item % p.gu4);
+  // (batched: the matrices of an output group lie one after the other)
+  const u32x4* weights = p.weights + ((size_t)(item / p.gu4) * (BATCHED ? p.batch.weights_batch : 1) + wb) * p.ks * p.gu4 +
+                         item % p.gu4;
   const int act_stride = BATCHED ? p.batch.src_rows * M : M, act_tok0 = BATCHED ? min(brow, p.batch.src_rows - 1) * M : 0;
   const int dst_stride = BATCHED ? p.batch.rows * M : M, dst_tok0 = BATCHED ? brow * M : 0;
 

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   const int brow = BATCHED ? (int)blockIdx.z : 0;
   int wb = BATCHED ? p.batch_ids[brow] : 0;
   if (BATCHED) wb = __builtin_amdgcn_readfirstlane(min(max(wb, 0), p.weights_batch - 1));
-  const u32x4* weights = sg.weights + (BATCHED ? (size_t)wb * p.ks * row_u4 : 0);
+  const u32x4* weights = sg.weights;
   const __half* scale_base = sg.scale + (BATCHED ? (size_t)wb * sg.n_pad : 0);
   const __half* zp_base = ZP ? sg.zero_point + (BATCHED ? (size_t)wb * sg.n_pad : 0) : nullptr;
   const size_t group_stride = (size_t)sg.n_pad * (BATCHED ? p.weights_batch : 1);  // elements per scale group
@@ -198,8 +198,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   const int pcol_raw = strip * LPR + col;  // uint4 column = output channels 8*pcol .. +7
   const bool col_ok = pcol_raw < row_u4;
   const int pcol = col_ok ? pcol_raw : row_u4 - 1;  // clamp: loads stay in range, result unused
-  // with output groups, the rows of a group lie one after the other
-  const u32x4* wcol = weights + ((size_t)(pcol / sg.gu4) * p.ks * sg.gu4 + pcol % sg.gu4);
+  // with output groups, the rows of a group lie one after the other (batched: of its matrices, one
+  // after the other)
+  const u32x4* wcol = weights + ((size_t)(pcol / sg.gu4) * (BATCHED ? p.weights_batch : 1) + wb) * p.ks * sg.gu4 + pcol % sg.gu4;
   const int rstride = sg.gu4;
   const int ky = blockIdx.y;
   const int c_begin = ky * p.chunks_per_split;
@@ -624,10 +625,17 @@ struct StripParams {
   int group_chunks, n_total, segments, reserved;
   uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
   StripSegment seg[kMaxSegments];
+  // batched weights selected by runtime ids (BATCHED instantiations only): dst row blockIdx.z
+  const int32_t* batch_ids;
+  int rows, src_rows, weights_batch;
 };
 
-template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI>
+// BATCHED: batched weights selected by runtime ids, one dst row of one token per blockIdx.z (no K
+// split, one matrix list entry): the strip of matrix b is the b-th of its output group's runs,
+// scales are [group][matrix][channel], the token of source row r is every src_rows-th 8 bytes.
+template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) {
+  static_assert(!BATCHED || !MULTI, "a batched launch has one matrix list entry");
   constexpr int ROWS = WAVES * 64 / LPR;  // chunks of 8 K-slices the work-group covers per pass
   constexpr int STRIP = LPR * 8;          // channels of a strip (one output group of the layout)
   __shared__ float red[WAVES][STRIP];
@@ -647,10 +655,22 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
   const u32x4* weights = sg.weights;
   const u32x4* astrip = reinterpret_cast<const u32x4*>(p.act);  // chunk c: 4 uint4 (8 slices x 4 halfs)
-  const __half* scale = sg.scale;
-  const __half* zero_point = sg.zero_point;
   int ks = p.ks, group_chunks = p.group_chunks, n_pad = sg.n_pad;
   asm volatile("" : "+s"(up.mask_lo), "+s"(up.mask_hi), "+s"(ks), "+s"(group_chunks), "+s"(n_pad));
+  // BATCHED: this row's matrix (an id outside the batch is clamped into it) and its source row (one
+  // shared row is broadcast)
+  const int brow = BATCHED ? (int)blockIdx.z : 0;
+  int wb = 0, nb = 1, src_rows = 1, arow = 0;
+  if (BATCHED) {
+    nb = p.weights_batch;
+    src_rows = p.src_rows;
+    wb = __builtin_amdgcn_readfirstlane(min(max(p.batch_ids[brow], 0), nb - 1));
+    arow = min(brow, src_rows - 1);
+  }
+  const u32x2* arows = reinterpret_cast<const u32x2*>(p.act) + arow;  // BATCHED: K-slice s of the row at s * src_rows
+  const __half* scale = sg.scale + (size_t)wb * n_pad;
+  const __half* zero_point = ZP ? sg.zero_point + (size_t)wb * n_pad : nullptr;
+  const size_t group_stride = (size_t)n_pad * nb;  // elements per scale group
   // (the pointers are left to the compiler: through an asm operand they would lose their address
   // space and turn every load into a flat one)
   const int ky = blockIdx.y;
@@ -668,18 +688,24 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
   u32x4 zv = {0u, 0u, 0u, 0u};
   // row r of the strip: LPR uint4; chunk c: 8 rows
-  const u32x4* wstrip = weights + (size_t)strip * ks * LPR + col;
+  const u32x4* wstrip = weights + ((size_t)strip * nb + wb) * ks * LPR + col;
   // Loads of one chunk, in the order the memory pipeline returns them (loads return in order): the
   // small ones that come from cache first (activations, group scales), then the eight weight loads
   // back to back.
   u32x4 w[8], a4[4], sv;
+  u32x2 ab[8];
   auto issue = [&](int c) {
     const u32x4* wp = wstrip + (size_t)c * (8 * LPR);
+    if (BATCHED) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) a4[j] = astrip[c * 4 + j];
+      for (int j = 0; j < 8; ++j) ab[j] = arows[(size_t)(c * 8 + j) * src_rows];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a4[j] = astrip[c * 4 + j];
+    }
     if (GROUPED) {
       const int g = c / group_chunks;
-      const size_t so = (size_t)g * n_pad + (size_t)strip * STRIP + col * 8;
+      const size_t so = (size_t)g * group_stride + (size_t)strip * STRIP + col * 8;
       sv = *reinterpret_cast<const u32x4*>(scale + so);
       if (ZP) zv = *reinterpret_cast<const u32x4*>(zero_point + so);
     }
@@ -689,7 +715,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   auto consume = [&]() {
     u32x2 a[8][1];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) a[j][0] = u32x2{a4[j >> 1][2 * (j & 1)], a4[j >> 1][2 * (j & 1) + 1]};
+    for (int j = 0; j < 8; ++j) a[j][0] = BATCHED ? ab[j] : u32x2{a4[j >> 1][2 * (j & 1)], a4[j >> 1][2 * (j & 1) + 1]};
     float t[1][8], asum[1] = {0.0f};
 #pragma unroll
     for (int o = 0; o < 8; ++o) t[0][o] = 0.0f;
@@ -740,7 +766,10 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
     if (!GROUPED) v *= __half2float(__ushort_as_half(out_scale_raw));
     __half h = __float2half_rn(v);
     if (sg.bias) h = __hadd(h, __ushort_as_half(out_bias_raw));
-    sg.dst[n_out] = h;
+    if (BATCHED)
+      sg.dst[((size_t)(n_out >> 2) * p.rows + brow) * 4 + (n_out & 3)] = h;
+    else
+      sg.dst[n_out] = h;
   } else {
     p.partial[(size_t)ky * p.n_total + sg.n_off + n_out] = v;
   }
@@ -779,6 +808,16 @@ template <int LPR, int WAVES>
 hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
   const dim3 block(WAVES * 64);
+  if (p.batch_ids != nullptr) {  // batched weights: strips of 64 channels only
+    if constexpr (LPR == 8) {
+#define MLD_STRIP_B(G, Z) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, Z, false, true>), grid, block, 0, stream, p)
+      if (grouped) { if (zp) MLD_STRIP_B(true, true); else MLD_STRIP_B(true, false); }
+      else         { if (zp) MLD_STRIP_B(false, true); else MLD_STRIP_B(false, false); }
+#undef MLD_STRIP_B
+      return hipGetLastError();
+    }
+    return hipErrorInvalidValue;
+  }
 #define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
     if (zp) { if (multi) MLD_STRIP(true, true, true); else MLD_STRIP(true, true, false); }
@@ -806,10 +845,12 @@ hipError_t LaunchStripL(const StripParams& p, int waves, bool grouped, dim3 grid
 // groups of the same size (16, 8 or 4 slices), K a multiple of 32 channels (whole chunks).
 bool StripKernelServes(const FcArgs* args, int count) {
   if (GetTuning().gemv_fast == 0) return false;
-  if (args[0].m != 1 || args[0].batch_ids != nullptr) return false;
+  if (args[0].m != 1) return false;
   if (DivUp(args[0].k, 4) % 8 != 0 || args[0].k % 4 != 0) return false;
   const int group = EffectiveGroup(args[0].group, DivUp(args[0].n, 4));
   if (!IsNativeGroup(group)) return false;
+  // batched weights: one matrix list entry, strips of 64 channels
+  if (args[0].batch_ids != nullptr && (count != 1 || group != kNativeGroup)) return false;
   for (int i = 0; i < count; ++i) {
     const int ns = DivUp(args[i].n, 4);
     if (args[i].n % 4 != 0 || ns % group != 0 || EffectiveGroup(args[i].group, ns) != group) return false;
@@ -833,12 +874,13 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   size_t weight_bytes = 0;
   for (int i = 0; i < count; ++i) weight_bytes += (size_t)p.ks * p.seg[i].ns * 8;
   int cps = p.chunks;
-  if (strips < 128 && p.chunks > 64 / lpr && weight_bytes > ((size_t)6 << 20)) {
+  const bool batched = p.batch_ids != nullptr;  // (no K split: a dst row's sums stay in its work-group)
+  if (!batched && strips < 128 && p.chunks > 64 / lpr && weight_bytes > ((size_t)6 << 20)) {
     const int want = DivUp(256, strips);
     cps = 64 / lpr;
     while (cps * 2 * want <= p.chunks) cps *= 2;
   }
-  if (tune.gemv_ksplit > 0) cps = std::max(1, DivUp(p.chunks, tune.gemv_ksplit));
+  if (tune.gemv_ksplit > 0 && !batched) cps = std::max(1, DivUp(p.chunks, tune.gemv_ksplit));
   int ksplit = DivUp(p.chunks, cps);
   if (ksplit > kGemvMaxKSplit) {
     ksplit = kGemvMaxKSplit;
@@ -854,9 +896,16 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   p.ksplit = ksplit;
   int waves = 1;
   while (waves < 16 && waves * 64 / lpr < cps) waves *= 2;
+  // more work-groups than CUs (several dst rows): 512 threads, so that two work-groups share a CU and
+  // the second round starts while the first still streams (two c2-shaped matrices: 12.3 -> 11.4 us)
+  if (batched && (long)strips * p.rows > 256) waves = std::min(waves, 8);
   if (tune.gemv_waves > 0) waves = tune.gemv_waves;
-  const dim3 grid(strips, ksplit);
+  const dim3 grid(strips, ksplit, batched ? p.rows : 1);
   StripParams sp;
+  sp.batch_ids = p.batch_ids;
+  sp.rows = p.rows;
+  sp.src_rows = p.src_rows;
+  sp.weights_batch = p.weights_batch;
   sp.act = p.act;
   sp.partial = p.partial;
   sp.ks = p.ks;
@@ -1150,8 +1199,13 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
     // together still give most CUs a work-group, else 64-byte ones.
     if (count != 1) return hipErrorInvalidValue;
     p.ksplit = 1;
-    if (kernel_name) *kernel_name = "fc_w4_stream_kernel";
     const bool wide = (long)DivUp(p.seg[0].row_u4, 8) * a.rows >= 192;
+    // one token per row over output groups of 16 slices: the contiguous-strip kernel
+    if (wide && StripKernelServes(args, count)) {
+      if (kernel_name) *kernel_name = "fc_w4_strip_kernel";
+      return LaunchStrip(p, args, count, grouped, stream);
+    }
+    if (kernel_name) *kernel_name = "fc_w4_stream_kernel";
     const int lpr_b = wide ? 8 : 4, rows_b = wide ? 64 : 64;
     p.chunks_per_split = DivUp(p.chunks, rows_b) * rows_b;
     p.seg[0].strip_end = DivUp(p.seg[0].row_u4, lpr_b);

@@ -19,6 +19,14 @@ __host__ __device__ inline size_t BlockIndex(int ks, int s, int ks_total, int ns
   const int g = group > 0 && group < ns ? group : ns;
   return ((size_t)(s / g) * ks_total + ks) * g + s % g;
 }
+// Batched weights (matrix b of `batch` matrices): the reference packs them as the height of the
+// OHWI shape, and a spatial position lies between the output group and the K-slice
+// ([Og][HW][Is][G] blocks, weights_conversion.cc:139-185); with one output group that is one matrix
+// after the other, which is what fully_connected.cc:493-496 reads.
+__host__ __device__ inline size_t BatchedBlockIndex(int ks, int s, int b, int batch, int ks_total, int ns, int group) {
+  const int g = group > 0 && group < ns ? group : ns;
+  return (((size_t)(s / g) * batch + b) * ks_total + ks) * g + s % g;
+}
 inline int EffectiveGroup(int group, int ns) { return group > 0 && group < ns ? group : ns; }
 // Output group size (slices) of the layout mldhip_fc_int4_weights_desc asks for: 16 (64-channel
 // strips, 128-byte rows).  The kernels also read groups of 8 and 4 slices (narrower strips, more of

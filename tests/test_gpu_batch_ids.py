@@ -15,14 +15,17 @@ from test_oracle_fc import (batch_ids_float_weights, batch_ids_int8_exact, make_
 FP16_TOL = 2e-2
 
 
-def run_device(c, td, bias=None, max_tokens=None):
+def run_device(c, td, bias=None, max_tokens=None, group=None):
     import torch
     tt = torch.float16 if td == np.float16 else torch.float32
     mt = M.FLOAT16 if td == np.float16 else M.FLOAT32
     n, k, batch = c["n"], c["k"], c["batch"]
     ns = W.div_up(n, 4)
-    # batched weights come in the reference's layout (one output group, the batch outermost)
+    # batched weights come in the reference's layout (one output group, the batch outermost) or, with
+    # `group`, in output groups of that many slices (the matrices of a group one after the other)
     desc = M.fc_int8_weights_desc(n, k) if c["bits"] == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    if group is not None:
+        desc.output_group_size = group
     packed = (M.rearrange_int8_as_uint8 if c["bits"] == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
     src2 = c["src"].reshape(c["src_rows"] * c["row_tokens"], k)
     act = torch.from_numpy(W.to_slices(src2).astype(td)).cuda()
@@ -118,6 +121,32 @@ def test_mixture_shapes(oracle, bits, rows, row_tokens, src_rows, k, n, batch, g
     assert name == expect, (name, expect)
 
 
+@pytest.mark.parametrize("bits,rows,row_tokens,src_rows,k,n,batch,groups,zp,group,td", [
+    (4, 8, 1, 1, 2048, 768, 8, 64, False, 16, np.float16),    # mixture decode over the library's groups of 16 slices
+    (4, 8, 1, 8, 768, 2048, 8, 24, False, 16, np.float16),    # its down projections: one input row per matrix
+    (4, 2, 1, 1, 4096, 1024, 8, 1, False, 16, np.float16),    # per-channel scales
+    (4, 4, 1, 1, 1024, 4096, 6, 1, True, 16, np.float16),     # 256 strips: per-channel scales and zero points, shared input
+    (4, 7, 1, 7, 512, 2048, 5, 16, True, 16, np.float16),     # 224 strips: group-wise zero points, one input row per matrix
+    (4, 2, 1, 1, 4096, 14336, 3, 1, False, 16, np.float16),   # two matrices of the c2 shape
+    (4, 3, 4, 3, 1000, 1032, 5, 1, True, 6, np.float16),      # 4 tokens per row, zero points, groups of 6 of 258 slices
+    (4, 4, 7, 4, 352, 200, 128, 11, False, 25, np.float16),   # many tokens per row, odd group (unspecialised kernel)
+    (4, 5, 3, 5, 64, 20, 4, 2, True, 1, np.float32),          # groups of one slice, fp32
+    (8, 6, 2, 1, 171, 536, 3, 1, True, 2, np.float32),        # uint8 weights in groups
+    (8, 8, 1, 1, 2048, 768, 16, 64, True, 16, np.float16),    # uint8 group-wise, shared input
+])
+def test_mixture_shapes_in_output_groups(oracle, bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, group, td):
+    """Batched weights packed in output groups (the packers put the matrices of a group one after the
+    other): same results as the float reference over the same weights."""
+    c = make_batch_ids_case(rows * 5 + n + group, rows, row_tokens, src_rows, k, n, batch, bits, groups, zp)
+    print("batch ids in groups", bits, rows, row_tokens, src_rows, k, n, batch, groups, zp, group, td.__name__, flush=True)
+    got, name = run_device(c, td, group=group)
+    check(c, td, got, oracle)
+    if bits == 4 and td == np.float16 and row_tokens <= 4 and group % 2 == 0:
+        # one token per row over at least 192 strips of 64 channels: the contiguous-strip kernel
+        strip = row_tokens == 1 and group == 16 and k % 32 == 0 and (n // 64) * rows >= 192
+        assert name == ("fc_w4_strip_kernel" if strip else "fc_w4_stream_kernel"), name
+
+
 def test_repeated_and_out_of_range_ids(oracle):
     """The same matrix for several rows; an id outside the batch is clamped into it."""
     c = make_batch_ids_case(1, rows=6, row_tokens=2, src_rows=6, k=64, n=32, batch=4)
@@ -183,7 +212,8 @@ def test_random_sweep(oracle):
     (8, 3, 4, 3, 1000, 1032, 5), (4, 5, 3, 5, 171, 20, 3),     # ragged K, odd uint4 slice count (tiled kernel)
     (8, 2, 9, 1, 256, 64, 4),                                   # more than 4 tokens per row (tiled kernel)
 ])
-def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, batch):
+@pytest.mark.parametrize("group", [None, 2])
+def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, batch, group):
     """The integer-math FullyConnected over batched weights: int32 results bit for bit against the
     closed form and the oracle's kernel restatement."""
     import torch
@@ -191,6 +221,10 @@ def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, bat
     print("batch ids int8", bits, rows, row_tokens, src_rows, k, n, batch, flush=True)
     ns = W.div_up(n, 4)
     desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    if group is not None:  # output groups: the matrices of a group one after the other
+        if ns % group != 0:
+            pytest.skip("the group does not divide the slices")
+        desc.output_group_size = group
     packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
     act = torch.from_numpy(W.to_slices(c["src"].reshape(-1, k))).cuda()
     ids = torch.from_numpy(c["ids"]).cuda()

@@ -248,6 +248,23 @@ def test_batched_packing_is_one_matrix_after_the_other(oracle):
         assert np.array_equal(whole, parts)
 
 
+def test_batched_packing_in_output_groups(oracle):
+    """With output groups of G slices the spatial index lies between the output group and the K-slice
+    ([Og][HW][Is][G] blocks, weights_conversion.cc:139-185): the run of output group g of matrix b in
+    the batched buffer is that group's run of matrix b packed alone, at run index g * batch + b."""
+    rng = np.random.default_rng(6)
+    for bits, n, k, batch, group in ((4, 128, 64, 3, 16), (8, 32, 20, 4, 2), (4, 24, 40, 5, 3), (8, 16, 8, 2, 1)):
+        lim = 127 if bits == 8 else 7
+        w = rng.integers(-lim, lim + 1, size=(n, batch, 1, k), dtype=np.int8)
+        ns, ks = (n + 3) // 4, (k + 3) // 4
+        pack = oracle.int8_as_uint8 if bits == 8 else oracle.int8_as_uint4
+        run = ks * group * (16 if bits == 8 else 8)  # bytes of one output group of one matrix
+        whole = pack(w, I4O4, group).reshape(ns // group, batch, run)
+        for e in range(batch):
+            single = pack(np.ascontiguousarray(w[:, e, 0, :]), I4O4, group).reshape(ns // group, run)
+            assert np.array_equal(whole[:, e, :], single), (bits, n, k, batch, group, e)
+
+
 def test_batched_scale_tensor_layout(oracle):
     """[group][batch][slice][4], zero padded: element (o, b, g) found where the kernel reads it
     (weights_scale.Read(o_slice, w_batch_id, group), fully_connected_util.cc:80-98)."""
