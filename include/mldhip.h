@@ -302,9 +302,9 @@ typedef struct {
   /* ConvRuntimeCheckDesc::PackedGroups (common/task/gpu_operation.h:396-406), read when
    * has_runtime_check != 0 and packed_num_groups > 0: the grouped FullyConnected of a
    * mixture-of-experts prefill (MakeConvWithPackedGroups, common/gpu_model_builder_moe_util.cc:119-230).
-   * ExternalWeights::shape = OHWI(o, packed_num_groups, 1, i): the matrices packed one after the other
-   * in the one-group layout, scales [scale_i][packed_num_groups][ceil(o/4)][4], as for
-   * mldhip_fc_batch_ids_create.  The source is one row of tokens sorted by matrix; matrix g multiplies
+   * ExternalWeights::shape = OHWI(o, packed_num_groups, 1, i): the matrices packed with the op's
+   * WeightsDescription and the scales [scale_i][packed_num_groups][ceil(o/4)][4], both as for
+   * mldhip_fc_batch_ids_create (the two ops of a layer read the same buffers).  The source is one row of tokens sorted by matrix; matrix g multiplies
    * the params[packed_params_offset + g] tokens that start at token
    * params[packed_params_offset + packed_num_groups + g] (fully_connected_util.cc:263-277), at most
    * packed_max_group_size of them; dst tokens that belong to no group are not written.  "params" is

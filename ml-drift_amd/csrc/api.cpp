@@ -428,8 +428,6 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
       if (int8_math) return Fail(MLDHIP_UNIMPLEMENTED, "packed groups: floating-point FullyConnected only");
       if (d->packed_params_offset < 0 || d->packed_max_group_size < 1)
         return Fail(MLDHIP_INVALID_ARGUMENT, "packed groups need a params offset >= 0 and a positive max_group_size");
-      if (wd.output_group_size != DivUp(d->o, 4))
-        return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription output_group_size.");
       packed_groups = true;
       weights_batch = d->packed_num_groups;
     }

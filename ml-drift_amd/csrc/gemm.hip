@@ -652,13 +652,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const uint32_t row_w = (uint32_t)sg.group * kBlk;  // bytes per K-slice row of the weights
   const uint32_t row_x = (uint32_t)p.m * 8u;   // bytes per K-slice row of the activations
   const uint32_t k_slices_end = (uint32_t)(t_begin + per_wave) * 4u;
-  const uint32_t w_end = one_group ? (uint32_t)min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w) : sg.a_bytes;
+  // (packed groups over output groups: the buffer of all matrices, see w_base)
+  const uint32_t w_end = one_group ? (uint32_t)min((uint64_t)sg.a_bytes, (uint64_t)k_slices_end * row_w)
+                                   : sg.a_bytes * (uint32_t)max(p.pg_groups, 1);
   const uint32_t x_end = min((uint64_t)p.b_bytes, (uint64_t)k_slices_end * row_x);
 
   constexpr uint32_t kOob = 0x7FFFFFF0u;
-  // packed groups: matrix pg_e of the batched buffers (weights one matrix after the other, scales
-  // [group][matrix][Ns][4])
-  const uint8_t* w_base = sg.w4 + (size_t)pg_e * sg.a_bytes;
+  // packed groups: matrix pg_e of the batched buffers (weights one matrix after the other, or, with
+  // output groups, the matrices of a group one after the other; scales [group][matrix][Ns][4])
+  const uint8_t* w_base = sg.w4 + (one_group ? (size_t)pg_e * sg.a_bytes : 0);
   const __half* s_base = sg.scale + (size_t)pg_e * sg.ns * 4;
   const __half* z_base = (ZP ? sg.zp : sg.scale) + (size_t)pg_e * sg.ns * 4;
   const uint32_t s_bytes = sg.s_bytes - (uint32_t)pg_e * (uint32_t)sg.ns * 8u;
@@ -687,7 +689,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // address lives there.
   const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
   const uint32_t col_w = one_group ? (uint32_t)nsi * kBlk
-                                   : ((uint32_t)(nsi / sg.group) * (uint32_t)p.ks * (uint32_t)sg.group + (uint32_t)(nsi % sg.group)) * kBlk;
+                                   : (((uint32_t)(nsi / sg.group) * (uint32_t)max(p.pg_groups, 1) + (uint32_t)pg_e) * (uint32_t)p.ks *
+                                          (uint32_t)sg.group +
+                                      (uint32_t)(nsi % sg.group)) * kBlk;
   uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + col_w : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
   // token of this lane in MFMA token block fm
@@ -1220,9 +1224,9 @@ bool FcW4MfmaSupported(const FcArgs& a) { return a.m > kGemvMaxTokens && DirectG
 bool FcW4MfmaPackedSupported(const FcArgs& a) {
   if (a.params == nullptr || a.packed_params_offset < 0 || a.batch_ids != nullptr) return false;
   if (a.src_end_ch_index >= 0 || a.dst_end_ch_index >= 0) return false;
-  if (EffectiveGroup(a.group, DivUp(a.n, 4)) != DivUp(a.n, 4)) return false;
-  // 32-bit offsets into the scale tensor of all matrices
+  // 32-bit offsets into the scale tensor of all matrices and, with output groups, into their weights
   if ((size_t)(a.scale_kind == kScaleBlock ? a.groups : 1) * a.weights_batch * DivUp(a.n, 4) * 8 >= 0x7FFFFFF0u) return false;
+  if ((size_t)a.weights_batch * DivUp(a.k, 4) * DivUp(a.n, 4) * (a.weight_bits == 8 ? 16 : 8) >= 0x7FFFFFF0u) return false;
   return DirectGemmShapeOk(a);
 }
 

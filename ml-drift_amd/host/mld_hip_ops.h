@@ -53,12 +53,9 @@ inline WeightsDescription GetFullyConnectedInt8WeightsDesc(const OHWI& shape) {
 }
 inline WeightsDescription GetFullyConnectedInt4WeightsDesc(const OHWI& shape) {
   WeightsDescription d;
-  // batched weights (h = the weights batch) keep the reference's single output group, with which
-  // the matrices of the batch lie one after the other
-  if (shape.h * shape.w != 1)
-    mldhip_fc_int4_weights_desc_reference(shape.o, shape.i, &d);
-  else
-    mldhip_fc_int4_weights_desc(shape.o, shape.i, &d);
+  // (batched weights, h = the weights batch, take the same description: the packers put the matrices
+  // of an output group one after the other)
+  mldhip_fc_int4_weights_desc(shape.o, shape.i, &d);
   return d;
 }
 inline WeightsDescription GetConvolutionInt8WeightsDesc(const OHWI& shape) {

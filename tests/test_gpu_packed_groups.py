@@ -16,7 +16,7 @@ from test_oracle_fc import (make_packed_groups_case, packed_groups_expected, run
 FP16_TOL = 2e-2
 
 
-def run_device(c, td, sizes=None, offsets=None, max_group_size=None, params_offset=0, fill=None):
+def run_device(c, td, sizes=None, offsets=None, max_group_size=None, params_offset=0, fill=None, group=None):
     import torch
     tt = torch.float16 if td == np.float16 else torch.float32
     mt = M.FLOAT16 if td == np.float16 else M.FLOAT32
@@ -24,6 +24,8 @@ def run_device(c, td, sizes=None, offsets=None, max_group_size=None, params_offs
     ns = W.div_up(n, 4)
     tokens = c["packed_src"].shape[0]
     desc = M.fc_int8_weights_desc(n, k) if c["bits"] == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    if group is not None:  # output groups of `group` slices: the matrices of a group one after the other
+        desc.output_group_size = group
     packed = (M.rearrange_int8_as_uint8 if c["bits"] == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
 
     def tensor(v):
@@ -94,6 +96,24 @@ def test_mixture_prefill_shapes(oracle, bits, width, per_item, k, n, batch, grou
         with M.tuning(force_generic=1):
             slow = unpack_groups(c, run_device(c, td, params_offset=3))
         check(slow, packed_groups_expected(oracle, c, td), td, k)
+
+
+@pytest.mark.parametrize("bits,width,per_item,k,n,batch,groups,zp,td,group", [
+    (4, 512, 8, 2048, 768, 128, 64, False, np.float16, 16),  # the mixture layer's prefill over groups of 16 slices
+    (4, 96, 2, 768, 2048, 8, 24, True, np.float16, 16),      # its down projections, zero points
+    (8, 40, 3, 256, 536, 5, 1, False, np.float16, 2),        # uint8 weights in groups of 2 slices
+    (4, 33, 3, 171, 536, 5, 1, True, np.float32, 67),        # fp32 tensors (unspecialised kernel), odd group
+    (4, 7, 1, 64, 20, 4, 2, True, np.float16, 1),            # groups of one slice
+])
+def test_mixture_prefill_shapes_in_output_groups(oracle, bits, width, per_item, k, n, batch, groups, zp, td, group):
+    """The batched weights packed in output groups (the layout the batch-ids op of the same layer
+    streams fastest): same results."""
+    c = make_packed_groups_case(width + n + group, width, per_item, k, n, batch, bits, groups, zp)
+    rows = run_device(c, td, params_offset=2, group=group)
+    check(unpack_groups(c, rows), packed_groups_expected(oracle, c, td), td, k)
+    if width * per_item * k * n <= 1 << 28:
+        rest = run_packed_groups_oracle(oracle, c, oracle.PREC_F32 if td == np.float32 else oracle.PREC_F32F16)
+        check(rows, rest.astype(np.float64), td, k)
 
 
 @pytest.mark.parametrize("fm", [1, 2])
