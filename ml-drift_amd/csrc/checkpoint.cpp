@@ -15,6 +15,7 @@
 // [o][i / block].
 #include <cstdio>
 #include <cstring>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -132,10 +133,9 @@ extern "C" int mldhip_checkpoint_fc_probe(const char* directory, const char* wei
   return MLDHIP_OK;
 }
 
-extern "C" int mldhip_checkpoint_fc_read(const char* directory, const char* weights_name, const char* base_name,
-                                         const mldhip_checkpoint_fc* info, int swap_dims, int tensor_type,
-                                         uint8_t* weights, size_t weights_bytes, void* scale, void* zero_point,
-                                         size_t scale_bytes, int32_t* weights_sum_i) {
+static int ReadFc(const char* directory, const char* weights_name, const char* base_name, const mldhip_checkpoint_fc* info,
+                  int swap_dims, int tensor_type, uint8_t* weights, size_t weights_bytes, void* scale, void* zero_point,
+                  size_t scale_bytes, int32_t* weights_sum_i) {
   if (!directory || !weights_name || !base_name || !info || !weights || !scale || !weights_sum_i)
     return FailWith(MLDHIP_INVALID_ARGUMENT, "null argument");
   if (tensor_type != MLDHIP_FLOAT16 && tensor_type != MLDHIP_FLOAT32)
@@ -190,4 +190,16 @@ extern "C" int mldhip_checkpoint_fc_read(const char* directory, const char* weig
     if (int rc = mldhip_scale_to_tensor(z_host.data(), o, info->scale_i, tensor_type, zero_point, scale_bytes)) return rc;
   }
   return MLDHIP_OK;
+}
+
+extern "C" int mldhip_checkpoint_fc_read(const char* directory, const char* weights_name, const char* base_name,
+                                         const mldhip_checkpoint_fc* info, int swap_dims, int tensor_type,
+                                         uint8_t* weights, size_t weights_bytes, void* scale, void* zero_point,
+                                         size_t scale_bytes, int32_t* weights_sum_i) {
+  try {  // (the staging buffers are as large as the layer: no exception may cross the C boundary)
+    return ReadFc(directory, weights_name, base_name, info, swap_dims, tensor_type, weights, weights_bytes, scale, zero_point,
+                  scale_bytes, weights_sum_i);
+  } catch (const std::bad_alloc&) {
+    return FailWith(MLDHIP_INTERNAL, "out of host memory while reading the layer");
+  }
 }
