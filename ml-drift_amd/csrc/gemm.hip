@@ -1160,14 +1160,18 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     p.pg_groups = a.weights_batch;
     p.pg_max = std::min(a.packed_max_group_size, a.m);
     p.ksplit = 1;
-    int fm = p.pg_max <= 32 ? 1 : 2;
-    if (tune.gemm_fm == 1 || tune.gemm_fm == 2) fm = tune.gemm_fm;
+    // token tiles of 32, 64 or (groups of hundreds of tokens) 128 tokens; a group starts at any token,
+    // so the tiles are read token by token (no 16-byte token pairs)
+    int fm = p.pg_max <= 32 ? 1 : (p.pg_max >= 256 ? 4 : 2);
+    if (tune.gemm_fm == 1 || tune.gemm_fm == 2 || tune.gemm_fm == 4) fm = tune.gemm_fm;
     const int tiles_m = DivUp(p.pg_max, fm * 32);
     p.xcd_m = 1;  // few token tiles per matrix: the XCDs share the channel tiles
     if (tune.gemm_xcd_m == 1 || tune.gemm_xcd_m == 2 || tune.gemm_xcd_m == 4 || tune.gemm_xcd_m == 8) p.xcd_m = tune.gemm_xcd_m;
     const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), 1, a.weights_batch);
     const bool zp = p.seg[0].zp != nullptr;
-    if (fm == 2)
+    if (fm == 4)
+      LaunchDirect<4, 4, 4, false, false>(a.weight_bits, zp, grid, stream, p);
+    else if (fm == 2)
       LaunchDirect<2, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);
     else
       LaunchDirect<1, 4, 8, false, false>(a.weight_bits, zp, grid, stream, p);

@@ -116,10 +116,10 @@ def test_mixture_prefill_shapes_in_output_groups(oracle, bits, width, per_item, 
         check(rows, rest.astype(np.float64), td, k)
 
 
-@pytest.mark.parametrize("fm", [1, 2])
+@pytest.mark.parametrize("fm", [1, 2, 4])
 def test_groups_of_every_size_on_the_matrix_cores(oracle, fm):
     """Group sizes 0, 1, odd, one token tile exactly, several tiles, beyond max_group_size; offsets that
-    are odd and that leave gaps; both token tiles (32 and 64 tokens).  fp16, against the restatement."""
+    are odd and that leave gaps; every token tile (32, 64 and 128 tokens).  fp16, against the restatement."""
     c = make_packed_groups_case(21, 300, 1, 256, 136, 8, 4, 8, True)
     sizes = np.array([0, 1, 33, 64, 65, 100, 7, 40], np.int32)
     # (runs that do not overlap; the last one is cut at the end of the tensor)
@@ -130,6 +130,23 @@ def test_groups_of_every_size_on_the_matrix_cores(oracle, fm):
     ref = run_packed_groups_oracle(oracle, c, oracle.PREC_F32F16, max_group_size=80, dst_before=before, sizes=sizes, offsets=offsets)
     assert np.array_equal(got == 7.0, ref == 7.0)
     written = ref != 7.0
+    rms = np.sqrt(np.mean(ref[written] ** 2))
+    assert np.abs(got - ref)[written].max() <= FP16_TOL * rms
+
+
+def test_groups_of_hundreds_of_tokens(oracle):
+    """Groups large enough for the 128-token tiles (max_group_size >= 256): sizes around the tile
+    edges, odd offsets, zero points; against the restatement."""
+    c = make_packed_groups_case(31, 900, 1, 128, 264, 3, 4, 4, True)
+    sizes = np.array([257, 128, 385], np.int32)
+    offsets = np.array([1, 260, 391], np.int32)
+    got = run_device(c, np.float16, sizes=sizes, offsets=offsets, max_group_size=400, fill=7.0, group=2)
+    before = oracle.f32_to_f16_bits(np.full(((264 + 3) // 4, 900, 4), 7.0, np.float32))
+    ref = run_packed_groups_oracle(oracle, c, oracle.PREC_F32F16, max_group_size=400, dst_before=before, sizes=sizes,
+                                   offsets=offsets)
+    assert np.array_equal(got == 7.0, ref == 7.0)
+    written = ref != 7.0
+    assert written.sum() >= 0.999 * (257 + 128 + 385) * 264  # (a result may be 7.0 itself)
     rms = np.sqrt(np.mean(ref[written] ** 2))
     assert np.abs(got - ref)[written].max() <= FP16_TOL * rms
 
