@@ -279,12 +279,40 @@ def run_other(args, torch, M, W):
         wall, _, reg = time_graph(torch, stream, step, args.steps, args.warmup)
         _, us, _ = time_graph(torch, stream, lambda s, i: conv.launch(s), args.steps, args.warmup)
         _, q_us, _ = time_graph(torch, stream, lambda s, i: q.launch(s), args.steps, args.warmup)
+        # the same step with the reference's default, asymmetric quantization (the rescale then adds
+        # w_scale * offset * sum_i(w) per token and channel)
+        codes_a, params_a = torch.zeros_like(codes), torch.zeros_like(params)
+        out_a = torch.zeros_like(out_t)
+        qa = M.quantization_create(M.FLOAT16, M.PACKED_INT8C16, k, calculate_sum=False, symmetric=False, max_tokens=m)
+        qa.bind([src], [codes_a, params_a])
+        qa.set_shape(1, 1, m)
+        conv_a = M.conv_int8_create(M.FLOAT16, n, k, wd, max_tokens=m)
+        conv_a.bind([codes_a, wt, params_a, wsum, wscale], [out_a])
+        conv_a.set_shape(1, 1, m)
+
+        def step_a(s, i):
+            qa.launch(s)
+            conv_a.launch(s)
+        wall_a, _, _ = time_graph(torch, stream, step_a, args.steps, args.warmup)
+        # codes that round-to-nearest-even (the wording of the configuration) would change: the library
+        # follows the reference's floor(x * scale + 128.5)
+        codes_e, params_e = torch.zeros_like(codes), torch.zeros_like(params)
+        qe = M.quantization_create(M.FLOAT16, M.PACKED_INT8C16, k, calculate_sum=False, symmetric=True, max_tokens=m,
+                                   round_to_nearest_even=True)
+        qe.bind([src], [codes_e, params_e])
+        qe.set_shape(1, 1, m)
+        q.launch(stream.cuda_stream)
+        qe.launch(stream.cuda_stream)
+        stream.synchronize()
+        differing = int((codes_e[:, :, :] != codes[:, :, :]).sum().item())
         ops = 2.0 * m * k * n
         out = dict(base, metric="int8_dynamic_gemm_throughput", value=round(ops / wall / 1e12, 1),
                    unit="TOP/s", ms_per_step=round(wall * 1e3, 6),
                    dtype="i8 x i8, i32 accumulate (int8 MFMA), f32 rescale",
                    config=dict({"workload": "c4: per-token int8 quantization + int8 x int8 GEMM M=2048 K=2048 N=8192, fp16 out",
-                                "ops_per_step": ops, "quantize_us": round(q_us, 3)}, **reg),
+                                "ops_per_step": ops, "quantize_us": round(q_us, 3),
+                                "asymmetric_quantization_ms_per_step": round(wall_a * 1e3, 6),
+                                "codes_changed_by_round_to_nearest_even": "%d of %d" % (differing, m * k)}, **reg),
                    roofline={"bound": "mfma", "kernel": conv.kernel_name, "achieved": round(ops / us / 1e6, 1),
                              "peak": 5000.0, "unit": "TOP/s", "frac": round(ops / us / 1e6 / 5000.0, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})

@@ -355,6 +355,12 @@ typedef struct {
   int32_t calculate_sum;
   int32_t symmetric;
   int32_t max_tokens;
+  /* 0 (the reference's kernel): codes by floor(x * scale + zero point + 0.5), asymmetric
+   * int((x - min) * scale + 0.5) (quantize_and_dequantize.cc:424-434).  1: round-to-nearest-even of
+   * the scaled value, rint(x * scale) + zero point and rint((x - min) * scale); no counterpart in the
+   * reference.  The two differ by one code where the scaled value lies (within fp32 rounding of the
+   * reference's sum) half way between two codes. */
+  int32_t round_to_nearest_even;
 } mldhip_quant_desc;
 
 int mldhip_quantization_create(const mldhip_quant_desc* desc, mldhip_op** op);

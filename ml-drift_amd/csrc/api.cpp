@@ -493,6 +493,8 @@ int mldhip_quantization_create(const mldhip_quant_desc* d, mldhip_op** out) {
   if (d->packed_type < MLDHIP_PACKED_UINT8C4 || d->packed_type > MLDHIP_PACKED_UINT4C32)
     return Fail(MLDHIP_INVALID_ARGUMENT, "unknown packed type");
   if (d->channels <= 0 || d->max_tokens <= 0) return Fail(MLDHIP_INVALID_ARGUMENT, "bad shape");
+  if (d->round_to_nearest_even != 0 && d->round_to_nearest_even != 1)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "round_to_nearest_even must be 0 or 1");
   mldhip_op* op = new (std::nothrow) mldhip_op();
   if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
   op->kind = mldhip_op::kQuant;
@@ -795,6 +797,7 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     a.packed_type = d.packed_type;
     a.symmetric = d.symmetric != 0;
     a.calculate_sum = d.calculate_sum != 0;
+    a.nearest_even = d.round_to_nearest_even != 0;
     e = LaunchQuantize(a, stream, &op->last_kernel);
   } else {
     const mldhip_conv_int8_desc& d = op->cv;

@@ -64,7 +64,8 @@ struct FcArgs {
   // Batched weights selected by a runtime tensor of ids (the reference's
   // CreateFullyConnectedWeightsBatchIds): dst row y (of `rows`, m tokens each) = FC of src row
   // min(y, src_rows - 1) with weight matrix batch_ids[y] of `weights_batch`.  The packed buffer
-  // holds the matrices one after the other, scales are [groups][weights_batch][Ns][4].
+  // holds the matrices of an output group one after the other (BatchedBlockIndex), scales are
+  // [groups][weights_batch][Ns][4].
   // Plain launches: batch_ids = nullptr, rows = src_rows = weights_batch = 1.
   const int32_t* batch_ids = nullptr;
   int rows = 1, src_rows = 1, weights_batch = 1;
@@ -113,7 +114,7 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
 struct FcBatchRows {
   const int32_t* ids = nullptr;
   int rows = 1, src_rows = 1, weights_batch = 1;
-  int group = 0;  // output group size of the packed weights (plain launches only; 0 = one group)
+  int group = 0;  // output group size of the packed weights (0 = one group)
   // runtime channel bounds, as in FcArgs (the tiled kernel only)
   const int32_t* params = nullptr;
   int src_end_ch_index = -1, dst_end_ch_index = -1;
@@ -157,6 +158,7 @@ struct QuantArgs {
   int packed_type = 2;  // PackedType (common/data_type.h:48-58)
   bool symmetric = false;
   bool calculate_sum = false;
+  bool nearest_even = false;  // round-to-nearest-even codes instead of the reference's floor(v + 0.5)
 };
 hipError_t LaunchQuantize(const QuantArgs& a, hipStream_t stream, const char** kernel_name);
 

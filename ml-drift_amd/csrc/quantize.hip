@@ -34,6 +34,7 @@ struct QuantParams {
   int is_signed, layout, symmetric, calculate_sum;
   int bits;           // 8, or 4 for the C32 types
   int width, height;  // tokens = height * width * batch, token = (y * width + x) * batch + b
+  int nearest_even;   // codes by round-to-nearest-even of the scaled value instead of the reference's floor(v + 0.5)
 };
 // where the codes of a token go
 enum : int { kCodesC4 = 0, kCodesC16 = 1, kCodesC32 = 2, kCodesW4C4 = 3 };
@@ -72,7 +73,7 @@ __device__ __forceinline__ float RangeInSrcType(const float*, float mx, float mn
   return Sub(mx, mn);
 }
 
-template <bool SYM>
+template <bool SYM, bool RNE>
 struct Quantizer {
   float scale, min_value;
   float round_offset;  // symmetric: range / 2 + 0.5
@@ -81,9 +82,14 @@ struct Quantizer {
   // saturates it at 0.  Asymmetric: truncation of a value >= 0.5, i.e. floor; a NaN (constant
   // row: 0 * inf) becomes code 0.
   __device__ __forceinline__ float Value(float x) const {
-    if (SYM) return fminf(floorf(Add(Mul(x, scale), round_offset)), top);
-    const float f = floorf(Add(Mul(Sub(x, min_value), scale), 0.5f));
-    return f != f ? 0.0f : fminf(f, top);
+    // RNE (not the reference's rule): rint(x * scale) + range / 2 and rint((x - min) * scale), ties to even
+    if (SYM) {
+      if (RNE) return fminf(Add(rintf(Mul(x, scale)), round_offset - 0.5f), top);
+      return fminf(floorf(Add(Mul(x, scale), round_offset)), top);
+    }
+    const float scaled = Mul(Sub(x, min_value), scale);
+    if (scaled != scaled) return 0.0f;
+    return fminf(RNE ? rintf(scaled) : floorf(Add(scaled, 0.5f)), top);
   }
 };
 
@@ -93,7 +99,7 @@ struct Quantizer {
 // codes in the C16 layout); the first CACHE groups of a thread stay in registers between the
 // min/max pass and the encoding pass, so a row of up to 16 * CACHE * lanes channels is read
 // from memory once.
-template <typename SrcT, int TT, bool SYM, int CACHE>
+template <typename SrcT, int TT, bool SYM, int CACHE, bool RNE = false>
 __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
   using RawT = typename Raw<SrcT>::type;
   __shared__ float s_a[kMaxWaves][TT];
@@ -189,7 +195,7 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
   }
 
   float inv_scale = 0.0f, offset = 0.0f;
-  Quantizer<SYM> qz;
+  Quantizer<SYM, RNE> qz;
   qz.scale = 0.0f;
   qz.min_value = 0.0f;
   // code range: 256 values, or 16 for the 4-bit types
@@ -313,16 +319,23 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
         make_float4(inv_scale, offset, p.calculate_sum ? (float)(int)sum : 0.0f, 0.0f);
 }
 
+template <int TT, int CACHE, bool RNE>
+void Launch3(bool f16, bool sym, dim3 grid, dim3 block, hipStream_t stream, const QuantParams& p) {
+  if (f16 && sym)
+    hipLaunchKernelGGL((quantize_kernel<__half, TT, true, CACHE, RNE>), grid, block, 0, stream, p);
+  else if (f16)
+    hipLaunchKernelGGL((quantize_kernel<__half, TT, false, CACHE, RNE>), grid, block, 0, stream, p);
+  else if (sym)
+    hipLaunchKernelGGL((quantize_kernel<float, TT, true, CACHE, RNE>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((quantize_kernel<float, TT, false, CACHE, RNE>), grid, block, 0, stream, p);
+}
 template <int TT, int CACHE>
 void Launch2(bool f16, bool sym, dim3 grid, dim3 block, hipStream_t stream, const QuantParams& p) {
-  if (f16 && sym)
-    hipLaunchKernelGGL((quantize_kernel<__half, TT, true, CACHE>), grid, block, 0, stream, p);
-  else if (f16)
-    hipLaunchKernelGGL((quantize_kernel<__half, TT, false, CACHE>), grid, block, 0, stream, p);
-  else if (sym)
-    hipLaunchKernelGGL((quantize_kernel<float, TT, true, CACHE>), grid, block, 0, stream, p);
+  if (p.nearest_even)
+    Launch3<TT, CACHE, true>(f16, sym, grid, block, stream, p);
   else
-    hipLaunchKernelGGL((quantize_kernel<float, TT, false, CACHE>), grid, block, 0, stream, p);
+    Launch3<TT, CACHE, false>(f16, sym, grid, block, stream, p);
 }
 // One register-cached group per thread when that covers the row, four otherwise.
 template <int TT>
@@ -357,6 +370,7 @@ hipError_t LaunchQuantize(const QuantArgs& a, hipStream_t stream, const char** k
   if (p.layout == kCodesW4C4 && (long long)a.width * a.height * a.batch != a.tokens) return hipErrorInvalidValue;
   p.symmetric = a.symmetric;
   p.calculate_sum = a.calculate_sum;
+  p.nearest_even = a.nearest_even ? 1 : 0;
   if (kernel_name) *kernel_name = "quantize_kernel";
   // Few channel groups: wide token tiles (32 tokens x >= 2 lanes); otherwise 8 tokens per
   // work-group and as many reduction lanes as there are groups, up to 128.

@@ -240,7 +240,7 @@ inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType
 
 inline Status CreateQuantization(DataType src_type, PackedType dst_type, const BHWC& shape, bool calculate_sum,
                                  bool symmetric, HipOperation* result) {
-  mldhip_quant_desc d{(int)src_type, (int)dst_type, shape.c, calculate_sum, symmetric, shape.b * shape.h * shape.w};
+  mldhip_quant_desc d{(int)src_type, (int)dst_type, shape.c, calculate_sum, symmetric, shape.b * shape.h * shape.w, 0};
   mldhip_op* op = nullptr;
   const int rc = mldhip_quantization_create(&d, &op);
   if (rc != MLDHIP_OK) return Status::FromCode(rc);

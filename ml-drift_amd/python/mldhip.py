@@ -59,7 +59,8 @@ class FcDesc(C.Structure):
 
 class QuantDesc(C.Structure):
     _fields_ = [("src_type", C.c_int32), ("packed_type", C.c_int32), ("channels", C.c_int32),
-                ("calculate_sum", C.c_int32), ("symmetric", C.c_int32), ("max_tokens", C.c_int32)]
+                ("calculate_sum", C.c_int32), ("symmetric", C.c_int32), ("max_tokens", C.c_int32),
+                ("round_to_nearest_even", C.c_int32)]
 
 
 class ConvInt8Desc(C.Structure):
@@ -429,8 +430,9 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
 
 
 def quantization_create(src_type, packed_type, channels, calculate_sum=False, symmetric=False,
-                        max_tokens=1):
-    d = QuantDesc(src_type, packed_type, channels, int(calculate_sum), int(symmetric), max_tokens)
+                        max_tokens=1, round_to_nearest_even=False):
+    d = QuantDesc(src_type, packed_type, channels, int(calculate_sum), int(symmetric), max_tokens,
+                  int(round_to_nearest_even))
     h = C.c_void_p()
     check(lib().mldhip_quantization_create(C.byref(d), C.byref(h)))
     return Op(h)

@@ -8,7 +8,7 @@ import mldhip as M
 import workloads as W
 
 
-def run_quant(src_slices_np, tokens, channels, packed_type, symmetric, calc_sum, batch=1, height=1):
+def run_quant(src_slices_np, tokens, channels, packed_type, symmetric, calc_sum, batch=1, height=1, nearest_even=False):
     import torch
     f16 = src_slices_np.dtype == np.float16
     src = torch.from_numpy(src_slices_np).cuda()
@@ -27,7 +27,7 @@ def run_quant(src_slices_np, tokens, channels, packed_type, symmetric, calc_sum,
     codes = torch.full(shape, 0x5A, dtype=torch.int8 if signed else torch.uint8, device="cuda")
     params = torch.zeros((tokens, 4), dtype=torch.float32, device="cuda")
     op = M.quantization_create(M.FLOAT16 if f16 else M.FLOAT32, packed_type, channels, calc_sum,
-                               symmetric, max_tokens=tokens)
+                               symmetric, max_tokens=tokens, round_to_nearest_even=nearest_even)
     op.bind([src], [codes, params])
     op.set_shape(batch, height, width)
     print("quant", tokens, channels, packed_type, symmetric, calc_sum, batch, height, flush=True)
@@ -144,3 +144,62 @@ def test_int4_literal_bytes_on_gpu():
     codes, params = run_quant(src, 1, 8, M.PACKED_UINT4C32, True, False)
     assert codes.tobytes() == bytes([0x1F, 0x9C, 0x58, 0x8E] + [0x58, 0x8E] * 6)
     assert params[0].tolist() == [1.0, -8.0, 0.0, 0.0]
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_round_to_nearest_even_switch(oracle, symmetric, dtype):
+    """The switch that is not the reference's rule: codes = rint(x * scale) + 128 (symmetric) or
+    rint((x - min) * scale) (asymmetric), ties to even, with the params of the reference's rule.
+    Against a numpy fp32 restatement of exactly that, bit for bit; and against the reference's rule:
+    the two differ by one code, only where the scaled value lies half way between two codes (within
+    the fp32 rounding of the reference's sum x * scale + 128.5), and the test prints how often."""
+    rng = np.random.default_rng(17)
+    tokens, channels = 64, 512
+    x = edge_tensor(rng, tokens, channels)
+    # a row of exact ties: multiples of half a step at scale 1 (symmetric: absmax 127; asymmetric: range 0 .. 255)
+    x[5] = 0.0
+    if symmetric:
+        x[5, :255] = np.arange(-127, 128) * 0.5
+        x[5, 255] = 127.0
+    else:
+        x[5, :511] = np.arange(511) * 0.5
+        x[5, 511] = 255.0
+    x = x.astype(dtype)
+    src = W.to_slices(x)
+    packed = M.PACKED_INT8C4
+    ref_codes, ref_params = run_quant(src, tokens, channels, packed, symmetric, True)
+    codes, params = run_quant(src, tokens, channels, packed, symmetric, True, nearest_even=True)
+    assert np.array_equal(params[:, :2], ref_params[:, :2])  # inv_scale and offset do not depend on the rounding
+    # numpy restatement of the switch, in fp32 like the kernel (the scale is the kernel's: 1 / inv_scale, or
+    # 255 / range for the asymmetric rule, recomputed here from the oracle's params of the same rows)
+    rc, rp = oracle.quantize(oracle.f32_to_f16_bits(src.astype(np.float32)) if dtype == np.float16 else src,
+                             tokens, channels, oracle.PACKED_INT8C4, symmetric, True)
+    assert np.array_equal(ref_codes, rc) and np.array_equal(ref_params, rp)
+    xf = x.astype(np.float32)
+    inv = rp[:, 0].astype(np.float32)
+    want = np.zeros((tokens, channels), np.int32)
+    for t in range(tokens):
+        if symmetric:
+            scale = np.float32(0.0) if inv[t] == 0 else np.float32(1.0) / inv[t]
+            v = np.rint(xf[t] * scale).astype(np.float32) + np.float32(128.0)
+        else:
+            # (the reference's search starts from element (b, 0, 0, 0): the first channel of the batch
+            # element's first token takes part in every token's range)
+            mn, mx = min(xf[t].min(), xf[0, 0]), max(xf[t].max(), xf[0, 0])
+            with np.errstate(over="ignore"):
+                rng_t = np.float32(dtype(mx) - dtype(mn))  # in the source type: +-65504 in fp16 gives inf
+            with np.errstate(divide="ignore", invalid="ignore"):
+                scale = np.float32(255.0) / rng_t
+                v = np.rint((xf[t] - mn) * scale)
+            v = np.where(np.isnan(v), 0.0, v)
+        want[t] = np.clip(v, 0, 255).astype(np.int32) - 128
+    got = W.from_slices(codes.astype(np.int32), channels)
+    assert np.array_equal(got, want)
+    ref = W.from_slices(ref_codes.astype(np.int32), channels)
+    diff = got != ref
+    assert np.abs(got - ref).max() <= 1
+    assert (got[5][diff[5]] % 2 == 0).all()  # in the row of exact ties the switch took the even code
+    print("codes that differ between the two rules: %d of %d (%d of them in the row of exact ties)" % (
+        diff.sum(), diff.size, diff[5].sum()))
+    assert 0 < diff[5].sum() and diff.sum() - diff[5].sum() <= diff.size // 1000
