@@ -158,7 +158,9 @@ def run_other(args, torch, M, W):
         # decode GEMVs over a ring of weight copies larger than the 256 MB cache
         if args.workload == "c1":
             case = W.make_fc_case(**W.CONFIGS["c1"])
-            dev0 = W.FcDevice(case)
+            # the weights as mldhip_fc_int8_weights_desc_decode asks for them (--layout reference: the
+            # reference's one output group)
+            dev0 = W.FcDevice(case, decode_layout=args.layout not in ("reference", "library"))
             m, k, n = case["m"], case["k"], case["n"]
             ring = max(args.ring, 80)  # 80 x 4.2 MB
             gen = torch.Generator(device="cuda").manual_seed(1)
@@ -171,7 +173,8 @@ def run_other(args, torch, M, W):
                 ops.append(op)
                 keep.append(wt)
             nbytes = n * k + k * 4 + n * 4 + n * 4  # W + act + scale + out (fp32 tensors)
-            label = "c1: FullyConnected decode GEMV M=1 K=2048 N=2048 int8 per-channel, fp32 act/out"
+            label = ("c1: FullyConnected decode GEMV M=1 K=2048 N=2048 int8 per-channel, fp32 act/out, "
+                     "kOSpatialIOGroupI4O4 output_group_size %d" % dev0.desc.output_group_size)
             metric, dtype = "int8_decode_gemv_hbm_bandwidth", "u8 weights x f32 activations, f32 accumulate"
         else:
             m, k, n = 1, 4096, 14336

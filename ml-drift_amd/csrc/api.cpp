@@ -160,6 +160,13 @@ int mldhip_fc_int4_weights_desc(int o, int i, mldhip_weights_desc* desc) {
 int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* desc) {
   return FcDesc(o, i, MLDHIP_UINT4, false, desc);
 }
+int mldhip_fc_int8_weights_desc_decode(int o, int i, mldhip_weights_desc* desc) {
+  if (int rc = FcDesc(o, i, MLDHIP_UINT8, false, desc)) return rc;
+  // fewer than 128 strips of 64 channels: output groups of one slice (what FullyConnectedOI reads), which
+  // the one-token kernel reads with the whole K of 4 channels inside a work-group
+  if (o > 4 && o / 64 < 128 && GetTuning().fc_group <= 0) desc->output_group_size = 1;
+  return MLDHIP_OK;
+}
 int mldhip_fc_int4_weights_desc_decode(int o, int i, mldhip_weights_desc* desc) {
   if (int rc = FcDesc(o, i, MLDHIP_UINT4, true, desc)) return rc;
   // fewer than 128 strips of 64 channels: strips of 8 channels (output groups of 2 slices), which the
@@ -776,6 +783,8 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         e = LaunchFcW4Stream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4MfmaSupported(a)) {
         e = LaunchFcW4Mfma(a, stream, &op->last_kernel);
+      } else if (!force_generic && FcW8RowsSupported(a)) {
+        e = LaunchFcW8Rows(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW8StreamSupported(a)) {
         e = LaunchFcW8Stream(a, stream, &op->last_kernel);
       } else {

@@ -59,6 +59,24 @@ __device__ __forceinline__ void Load4(const __half* p, size_t i, float v[4]) {
   v[2] = __low2float(hi);
   v[3] = __high2float(hi);
 }
+// Four values as they lie in memory, and their conversion: a load and its conversion are kept apart
+// where several loads must be in flight at once.
+__device__ __forceinline__ float4 LoadRaw4(const float* p, size_t i) { return *reinterpret_cast<const float4*>(p + i); }
+__device__ __forceinline__ uint2 LoadRaw4(const __half* p, size_t i) { return *reinterpret_cast<const uint2*>(p + i); }
+__device__ __forceinline__ void Cvt4(const float4& r, float v[4]) {
+  v[0] = r.x;
+  v[1] = r.y;
+  v[2] = r.z;
+  v[3] = r.w;
+}
+__device__ __forceinline__ void Cvt4(const uint2& r, float v[4]) {
+  const __half2 lo = *reinterpret_cast<const __half2*>(&r.x);
+  const __half2 hi = *reinterpret_cast<const __half2*>(&r.y);
+  v[0] = __low2float(lo);
+  v[1] = __high2float(lo);
+  v[2] = __low2float(hi);
+  v[3] = __high2float(hi);
+}
 __device__ __forceinline__ void Store1(float* dst, size_t i, float r, const float* bias, size_t bi) {
   dst[i] = bias ? r + bias[bi] : r;
 }
@@ -214,6 +232,142 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// One token over weights packed in output groups of one slice (the layout FullyConnectedOI reads,
+// fully_connected_oi.cc:122-133): the K rows of a slice are one contiguous run of 16-byte blocks,
+// so a work-group streams the whole K of 4 output channels and layers of a few thousand channels
+// give every CU several work-groups without a split of K.  Lane l reads rows l, l + T, l + 2T, ...
+// (T threads): every load instruction of a wave covers 1 KB of contiguous memory, eight of them in
+// flight per lane.  Same arithmetic as the kernel above (fp32, one conversion and one fused
+// multiply-add per weight, the centre removed per row with group-wise scales, once otherwise);
+// K is reduced inside the wave by butterflies, across waves through LDS in wave order.
+// group_chunks carries log2 of the K-slices per scale group here.
+// ------------------------------------------------------------------------------------------
+template <typename T, int WAVES, bool GROUPED>
+__global__ __launch_bounds__(WAVES * 64) void fc_w8_rows_kernel(W8Params p) {
+  constexpr int TH = WAVES * 64;
+  __shared__ float red[WAVES][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  // Work-groups go round-robin to the 8 XCDs.  The scales of 8 neighbouring slices share a line, so
+  // of every 64 work-groups XCD x takes slices 8x .. 8x + 7 (its L2 then fetches the line once).
+  int slice = blockIdx.x;
+  if (slice < (int)(gridDim.x & ~63u)) slice = (slice & ~63) + ((slice & 7) << 3) + ((slice >> 3) & 7);
+  const int ks = p.ks;
+  const u32x4* wrow = p.weights + (size_t)slice * ks;
+  const T* act = static_cast<const T*>(p.act);
+  const T* scale = static_cast<const T*>(p.scale);
+  const T* zero_point = static_cast<const T*>(p.zero_point);
+  const size_t group_stride = (size_t)p.ns * 4;
+  const int group_shift = p.group_chunks;
+
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f}, asum_all = 0.0f;
+  float s_lin[4] = {1.0f, 1.0f, 1.0f, 1.0f}, z_lin[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (!GROUPED) {
+    Load4(scale, (size_t)slice * 4, s_lin);
+    if (zero_point) Load4(zero_point, (size_t)slice * 4, z_lin);
+  }
+  // zero points come from the scales' address when there are none, and are dropped behind the fence
+  const bool has_zp = zero_point != nullptr;
+  const T* zsrc = has_zp ? zero_point : scale;
+  for (int r0 = tid; r0 < ks; r0 += 8 * TH) {
+    u32x4 w[8];
+    decltype(LoadRaw4(act, 0)) araw[8], sraw[8], zraw[8];
+    // small loads that come from cache first, then the eight weight loads back to back; rows past
+    // K re-read the last one.  Conversions, and the zeroing of activations past K, come behind the
+    // fence: next to their loads they would make the kernel wait for every load in turn.
+#pragma unroll
+    for (int j = 0; j < 8; ++j) araw[j] = LoadRaw4(act, (size_t)min(r0 + TH * j, ks - 1) * 4);
+    if (GROUPED) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const size_t so = (size_t)(min(r0 + TH * j, ks - 1) >> group_shift) * group_stride + (size_t)slice * 4;
+        sraw[j] = LoadRaw4(scale, so);
+        zraw[j] = LoadRaw4(zsrc, so);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wrow + min(r0 + TH * j, ks - 1));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float a[4], t[4] = {0.0f, 0.0f, 0.0f, 0.0f}, asum = 0.0f;
+      Cvt4(araw[j], a);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t word = w[j][i];
+        const float u0 = (float)(word & 0xFFu), u1 = (float)((word >> 8) & 0xFFu);
+        const float u2 = (float)((word >> 16) & 0xFFu), u3 = (float)(word >> 24);
+        const float av = r0 + TH * j < ks ? a[i] : 0.0f;
+        asum += av;
+        t[0] = fmaf(av, u0, t[0]);
+        t[1] = fmaf(av, u1, t[1]);
+        t[2] = fmaf(av, u2, t[2]);
+        t[3] = fmaf(av, u3, t[3]);
+      }
+      if (GROUPED) {
+        float sc[4], zp[4];
+        Cvt4(sraw[j], sc);
+        Cvt4(zraw[j], zp);
+#pragma unroll
+        for (int o = 0; o < 4; ++o) acc[o] = fmaf(sc[o], fmaf(-(128.0f + (has_zp ? zp[o] : 0.0f)), asum, t[o]), acc[o]);
+      } else {
+        asum_all += asum;
+#pragma unroll
+        for (int o = 0; o < 4; ++o) acc[o] += t[o];
+      }
+    }
+  }
+  if (!GROUPED) {
+#pragma unroll
+    for (int o = 0; o < 4; ++o) acc[o] = s_lin[o] * fmaf(-(128.0f + z_lin[o]), asum_all, acc[o]);
+  }
+  // Every lane holds sums of the same 4 channels.  Two exchange steps halve what a lane carries
+  // (lanes 32.. keep channels 2 and 3, then lanes 16.. of each half the odd one), four more add
+  // the 16 lanes that are left with the same channel: lane l ends with channel 2 * (l / 32) + (l / 16) % 2.
+  // (Named scalars and selects between them: an index into `acc` that depends on the lane would
+  // move the array out of registers.)
+  const float c0 = acc[0], c1 = acc[1], c2 = acc[2], c3 = acc[3];
+  const bool up32 = (lane & 32) != 0, up16 = (lane & 16) != 0;
+  const float x0 = (up32 ? c2 : c0) + __shfl_xor(up32 ? c0 : c2, 32, 64);
+  const float x1 = (up32 ? c3 : c1) + __shfl_xor(up32 ? c1 : c3, 32, 64);
+  float v = (up16 ? x1 : x0) + __shfl_xor(up16 ? x0 : x1, 16, 64);
+#pragma unroll
+  for (int off = 8; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  const int ch = 2 * (lane >> 5) + ((lane >> 4) & 1);
+  if (WAVES > 1) {
+    if ((lane & 15) == 0) red[wave][ch] = v;
+    __syncthreads();
+    if (tid >= 64) return;
+    v = 0.0f;
+#pragma unroll
+    for (int q = 0; q < WAVES; ++q) v += red[q][ch];
+  }
+  if ((lane & 15) != 0) return;
+  const size_t n = (size_t)slice * 4 + ch;
+  Store1(static_cast<T*>(p.dst), n, v, static_cast<const T*>(p.bias), n);
+}
+
+template <typename T, int WAVES>
+hipError_t LaunchRowsG(const W8Params& p, dim3 grid, hipStream_t stream) {
+  if (p.grouped)
+    hipLaunchKernelGGL((fc_w8_rows_kernel<T, WAVES, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  else
+    hipLaunchKernelGGL((fc_w8_rows_kernel<T, WAVES, false>), grid, dim3(WAVES * 64), 0, stream, p);
+  return hipGetLastError();
+}
+template <typename T>
+hipError_t LaunchRowsT(const W8Params& p, int waves, hipStream_t stream) {
+  const dim3 grid(p.ns);
+  switch (waves) {
+    case 1: return LaunchRowsG<T, 1>(p, grid, stream);
+    case 2: return LaunchRowsG<T, 2>(p, grid, stream);
+    case 4: return LaunchRowsG<T, 4>(p, grid, stream);
+    default: return LaunchRowsG<T, 8>(p, grid, stream);
+  }
+}
+
 template <typename T, int LPR, int WAVES, bool BATCHED>
 hipError_t LaunchMB(const W8Params& p, dim3 grid, hipStream_t stream) {
   const dim3 block(WAVES * 64);
@@ -252,6 +406,49 @@ bool FcW8StreamSupported(const FcArgs& a) {
     if ((ks / a.groups) % 8 != 0) return false;  // a chunk of 8 K-slices must not straddle groups
   }
   return true;
+}
+
+// The row-interleaved kernel serves: one token, output groups of one slice, scale groups of a
+// power-of-two number of K-slices.
+bool FcW8RowsSupported(const FcArgs& a) {
+  if (a.weight_bits != 8 || a.act_f16 != a.dst_f16 || a.m != 1 || a.batch_ids != nullptr) return false;
+  const int ns = DivUp(a.n, 4), ks = DivUp(a.k, 4);
+  if (ns < 2 || EffectiveGroup(a.group, ns) != 1) return false;
+  if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
+  if (a.scale_kind == kScaleScalar) return false;
+  if (a.scale_kind == kScaleBlock) {
+    if (a.groups <= 0 || ks % a.groups != 0) return false;
+    const int group_slices = ks / a.groups;
+    if (group_slices & (group_slices - 1)) return false;
+  }
+  return true;
+}
+
+hipError_t LaunchFcW8Rows(const FcArgs& a, hipStream_t stream, const char** kernel_name) {
+  W8Params p;
+  p.weights = reinterpret_cast<const u32x4*>(a.weights);
+  p.act = a.act;
+  p.scale = a.scale;
+  p.zero_point = a.has_zero_point ? a.zero_point : nullptr;
+  p.bias = a.bias;
+  p.dst = a.dst;
+  p.m = 1;
+  p.ks = DivUp(a.k, 4);
+  p.ns = DivUp(a.n, 4);
+  p.chunks = DivUp(p.ks, 8);
+  p.grouped = a.scale_kind == kScaleBlock;
+  p.groups = p.grouped ? a.groups : 1;
+  p.group_chunks = 0;  // here: log2 of the K-slices per scale group
+  if (p.grouped)
+    for (int gs = p.ks / a.groups; gs > 1; gs >>= 1) ++p.group_chunks;
+  p.batch_ids = nullptr;
+  p.rows = p.src_rows = p.weights_batch = 1;
+  // eight rows per thread where K allows: all of a thread's loads are in flight at once
+  int waves = 1;
+  while (waves < 8 && waves * 64 * 8 < p.ks) waves *= 2;
+  if (GetTuning().gemv_waves > 0) waves = GetTuning().gemv_waves;
+  if (kernel_name) *kernel_name = "fc_w8_rows_kernel";
+  return a.act_f16 ? LaunchRowsT<__half>(p, waves, stream) : LaunchRowsT<float>(p, waves, stream);
 }
 
 hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name) {

@@ -108,6 +108,9 @@ hipError_t LaunchFcW4MfmaStream(const FcArgs& a, hipStream_t stream, const char*
 // Streaming GEMV over uint8 weights (1..4 tokens, fp32 or fp16 tensors of one type).
 bool FcW8StreamSupported(const FcArgs& a);
 hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+// One token over uint8 weights in output groups of one slice (fp32 or fp16 tensors of one type).
+bool FcW8RowsSupported(const FcArgs& a);
+hipError_t LaunchFcW8Rows(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 
 // Batched weights selected by runtime ids, for the integer-math launches (the same fields as in
 // FcArgs): dst row y of `rows` (m tokens each) = source row min(y, src_rows - 1) x matrix ids[y].

@@ -33,7 +33,7 @@ SYMBOLS = [
     "mldhip_op_kernel_name", "mldhip_op_cost", "mldhip_op_destroy", "mldhip_fc_launch_fused",
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
-    "mldhip_fc_int4_weights_desc_reference", "mldhip_fc_int4_weights_desc_decode", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
+    "mldhip_fc_int4_weights_desc_reference", "mldhip_fc_int4_weights_desc_decode", "mldhip_fc_int8_weights_desc_decode", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
     "mldhip_probe_launch",
 ]
 
@@ -138,9 +138,11 @@ def div_up(a, b):
 
 
 # ---- weight descriptions / packers (host) ----
-def fc_int8_weights_desc(o, i):
+def fc_int8_weights_desc(o, i, decode=False):
+    """The reference's layout (one output group); with `decode` the layout for ops that run one token
+    per launch (output groups of one slice for layers of a few thousand channels)."""
     d = WeightsDesc()
-    check(lib().mldhip_fc_int8_weights_desc(o, i, C.byref(d)))
+    check((lib().mldhip_fc_int8_weights_desc_decode if decode else lib().mldhip_fc_int8_weights_desc)(o, i, C.byref(d)))
     return d
 
 

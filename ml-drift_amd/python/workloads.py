@@ -67,7 +67,7 @@ def pack_fc_weights(case, reference_layout=False, output_group=None, decode_layo
         if output_group is not None:
             desc.output_group_size = output_group
         return desc, M.rearrange_int8_as_uint4(case["w"], desc)
-    desc = M.fc_int8_weights_desc(n, k)
+    desc = M.fc_int8_weights_desc(n, k, decode=decode_layout)
     if output_group is not None:
         desc.output_group_size = output_group
     return desc, M.rearrange_int8_as_uint8(case["w"], desc)
@@ -81,14 +81,14 @@ class FcDevice:
     """An FC op with its device buffers (torch tensors) for one synthetic case."""
 
     def __init__(self, case, device="cuda", max_tokens=None, scalar_scale=None, reference_layout=False,
-                 output_group=None, precision=None):
+                 output_group=None, precision=None, decode_layout=False):
         import torch
         self.torch = torch
         self.case = case
         m, k, n = case["m"], case["k"], case["n"]
         td = case["tensor_dtype"]
         tt = torch.float16 if td == np.float16 else torch.float32
-        self.desc, packed = pack_fc_weights(case, reference_layout, output_group)
+        self.desc, packed = pack_fc_weights(case, reference_layout, output_group, decode_layout)
         self.packed_host = packed
         self.weights = torch.from_numpy(packed).to(device)
         self.act = torch.from_numpy(to_slices(case["act"]).astype(td)).to(device)

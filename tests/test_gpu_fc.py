@@ -592,3 +592,46 @@ def test_rows_kernel(oracle, k, n, groups, zp, bias):
             dev.out.zero_()
             dev.run()
             check_fp(dev.result(), ref, case, "waves %d" % waves)
+
+
+@pytest.mark.parametrize("td", [np.float32, np.float16])
+@pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 1, False, False), (2048, 2048, 64, True, True),
+                                               (171, 536, 1, True, True), (16384, 256, 512, False, False),
+                                               (4096, 1536, 1, False, True), (40, 8, 1, False, False),
+                                               (10000, 64, 1, True, False)])
+def test_w8_rows_kernel(oracle, td, k, n, groups, zp, bias):
+    """One token over uint8 weights packed in output groups of one slice (the layout FullyConnectedOI
+    reads) on the row-interleaved kernel: fp32 and fp16 tensors, per-channel and group-wise scales,
+    zero points, ragged K, K shorter than a work-group's rows and K that needs several passes."""
+    case = W.make_fc_case(seed=k + n + 1, m=1, k=k, n=n, weight_bits=8, tensor_dtype=td, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    print("w8 rows kernel", td.__name__, k, n, groups, zp, bias, flush=True)
+    dev = W.FcDevice(case, decode_layout=True)
+    assert dev.desc.output_group_size == 1
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w8_rows_kernel", dev.op.kernel_name
+    dev.out.zero_()
+    dev.run()
+    assert np.array_equal(got, dev.result())
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    if k * n <= 1 << 24:
+        rest = oracle_fc(oracle, case).astype(np.float64)
+        check_fp(got, rest, case, "kernel restatement")
+    for waves in (1, 2, 8):
+        with M.tuning(gemv_waves=waves):
+            dev.out.zero_()
+            dev.run()
+            check_fp(dev.result(), ref, case, "waves %d" % waves)
+
+
+def test_config1_decode_layout(oracle):
+    """c1 over the layout mldhip_fc_int8_weights_desc_decode asks for, as the bench runs it."""
+    case = W.make_fc_case(**W.CONFIGS["c1"])
+    dev = W.FcDevice(case, decode_layout=True)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w8_rows_kernel", dev.op.kernel_name
+    check_fp(got, textbook(case), case, "textbook")
+    check_fp(got, oracle_fc(oracle, case).astype(np.float64), case, "kernel restatement")
