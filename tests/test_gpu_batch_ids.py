@@ -222,9 +222,7 @@ def test_int8_math_bit_exact(oracle, bits, rows, row_tokens, src_rows, k, n, bat
     ns = W.div_up(n, 4)
     desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
     if group is not None:  # output groups: the matrices of a group one after the other
-        if ns % group != 0:
-            pytest.skip("the group does not divide the slices")
-        desc.output_group_size = group
+        desc.output_group_size = group if ns % group == 0 else 1  # (an odd slice count: groups of one slice)
     packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
     act = torch.from_numpy(W.to_slices(c["src"].reshape(-1, k))).cuda()
     ids = torch.from_numpy(c["ids"]).cuda()
