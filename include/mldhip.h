@@ -134,10 +134,9 @@ int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* des
  * sums.  Ops over this layout run any number of tokens, but more than one token is served by the
  * slower general kernels. */
 int mldhip_fc_int4_weights_desc_decode(int o, int i, mldhip_weights_desc* desc);
-/* The same for uint8 weights: layers of fewer than 8192 output channels take output groups of one
- * slice, the layout FullyConnectedOI reads (linear_i4o4 = dst_s * src_slices + src_s,
- * common/kernels/fully_connected_oi.cc:122-133): the K rows of 4 channels are one contiguous run
- * that one work-group streams.  Wider layers keep mldhip_fc_int8_weights_desc. */
+/* The same for uint8 weights: output groups of one slice, the layout FullyConnectedOI reads
+ * (linear_i4o4 = dst_s * src_slices + src_s, common/kernels/fully_connected_oi.cc:122-133): the K
+ * rows of 4 channels are one contiguous run that one work-group streams. */
 int mldhip_fc_int8_weights_desc_decode(int o, int i, mldhip_weights_desc* desc);
 
 /* The weights layout the int8 x int8 MFMA convolution asks for, the counterpart of the

@@ -162,9 +162,9 @@ int mldhip_fc_int4_weights_desc_reference(int o, int i, mldhip_weights_desc* des
 }
 int mldhip_fc_int8_weights_desc_decode(int o, int i, mldhip_weights_desc* desc) {
   if (int rc = FcDesc(o, i, MLDHIP_UINT8, false, desc)) return rc;
-  // fewer than 128 strips of 64 channels: output groups of one slice (what FullyConnectedOI reads), which
-  // the one-token kernel reads with the whole K of 4 channels inside a work-group
-  if (o > 4 && o / 64 < 128 && GetTuning().fc_group <= 0) desc->output_group_size = 1;
+  // output groups of one slice (what FullyConnectedOI reads), which the one-token kernel reads with
+  // the whole K of 4 channels inside a work-group
+  if (o > 4 && GetTuning().fc_group <= 0) desc->output_group_size = 1;
   return MLDHIP_OK;
 }
 int mldhip_fc_int4_weights_desc_decode(int o, int i, mldhip_weights_desc* desc) {

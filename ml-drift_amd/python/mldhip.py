@@ -140,7 +140,7 @@ def div_up(a, b):
 # ---- weight descriptions / packers (host) ----
 def fc_int8_weights_desc(o, i, decode=False):
     """The reference's layout (one output group); with `decode` the layout for ops that run one token
-    per launch (output groups of one slice for layers of a few thousand channels)."""
+    per launch (output groups of one slice)."""
     d = WeightsDesc()
     check((lib().mldhip_fc_int8_weights_desc_decode if decode else lib().mldhip_fc_int8_weights_desc)(o, i, C.byref(d)))
     return d
