@@ -35,7 +35,7 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=None, help="default 4000 (c2, c1, f2), 2000 (moe), 200 (c3, c4), 20 (c5-*)")
     p.add_argument("--warmup", type=int, default=None, help="default steps / 10")
-    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe", "floors"],
+    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe"],
                    help="c2 (default) is the headline line; the others time the remaining configurations "
                         "the same way (one JSON line each, no CPU baseline)")
     p.add_argument("--tokens", type=int, default=128,
@@ -57,7 +57,7 @@ def parse():
                         "reference dispatch) followed by 64 launches over the weight ring, then exit")
     a = p.parse_args()
     if a.steps is None:
-        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "floors": 4000, "moe": 2000, "c3": 200, "c4": 200}.get(a.workload, 20)
+        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "moe": 2000, "c3": 200, "c4": 200}.get(a.workload, 20)
     if a.warmup is None:
         a.warmup = max(1, a.steps // 10)
     return a
@@ -137,24 +137,7 @@ def run_other(args, torch, M, W):
     stream = torch.cuda.Stream()
     base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "data": "synthetic"}
-    if args.workload == "floors":
-        # the two floors of a memory-bound launch on this box, timed like the ops: an empty launch and
-        # a plain streaming read of c2's 29.4 MB (packed weights) over a ring of 16 buffers
-        nbytes = 29360128
-        sink = torch.zeros(4096, dtype=torch.uint8, device="cuda")
-        bufs = [torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(args.ring)]
-        steps = args.steps or 4000
-        _, empty_us, _ = time_graph(torch, stream, lambda s, i: M.probe_launch(0, None, sink, s), steps, args.warmup)
-        wall, read_us, reg = time_graph(torch, stream, lambda s, i: M.probe_launch(1, bufs[i % len(bufs)], sink, s), steps,
-                                        args.warmup, ring=len(bufs))
-        out = dict(base, metric="streaming_read_floor", value=round(nbytes / wall / 1e9, 1), unit="GB/s",
-                   ms_per_step=round(wall * 1e3, 6), dtype="u8",
-                   config=dict({"workload": "floors: empty launch and plain streaming read of 29,360,128 B per launch",
-                                "empty_launch_us": round(empty_us, 3), "stream_read_us": round(read_us, 3)}, **reg),
-                   roofline={"bound": "hbm", "kernel": "probe_stream_read_kernel", "achieved": round(nbytes / read_us / 1e3, 1),
-                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / read_us / 1e3 / HBM_PEAK_GBS, 4),
-                             "traffic": None, "avg_launch_us": round(read_us, 3)})
-    elif args.workload in ("c1", "f2"):
+    if args.workload in ("c1", "f2"):
         # decode GEMVs over a ring of weight copies larger than the 256 MB cache
         if args.workload == "c1":
             case = W.make_fc_case(**W.CONFIGS["c1"])
@@ -467,14 +450,17 @@ def main():
     value = algo_bytes / wall / 1e9
     achieved = algo_bytes / (launch_us * 1e-6) / 1e9
 
-    # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
-    # scaled by a known-size copy); null when no summary is there
+    # HBM bytes per launch are not measured by this run (hardware counters need rocprofv3 around the
+    # process): `traffic` stays null, and the figure of the committed rocprofv3 --pmc summary (FETCH_SIZE
+    # + WRITE_SIZE, scaled by a known-size copy) is passed on under a name that says where it is from
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "fc_w4_stream_c2.md" if args.layout == "reference" else "fc_w4_strip_c2.md")
+    traffic_from_profile = None
+    tname = "fc_w4_stream_c2.md" if args.layout == "reference" else "fc_w4_strip_c2.md"
+    tpath = os.path.join(ROOT, "profiles", tname)
     if os.path.exists(tpath):
         import re
         mt = re.search(r"^hbm_bytes_per_launch = (\d+)", open(tpath).read(), re.M)
-        traffic = int(mt.group(1)) if mt else None
+        traffic_from_profile = {"bytes": int(mt.group(1)), "source": "profiles/" + tname} if mt else None
 
     out = {
         "metric": "int4_decode_gemv_hbm_bandwidth",
@@ -498,7 +484,7 @@ def main():
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "avg_launch_us": round(launch_us, 3)},
+                     "traffic_from_profile": traffic_from_profile, "avg_launch_us": round(launch_us, 3)},
     }
     if not args.no_cpu_baseline:
         runs, cores, path = cpu_baseline(case, args.cpu_seconds)

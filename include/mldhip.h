@@ -264,7 +264,7 @@ int mldhip_fc_is_recommended(int precision, int tokens);
  *   2 "weights_scale"         present iff scale_o*scale_i > 1
  *   3 "weights_zero_point"    present iff has_zero_point_tensor
  *   4 "biases"                present iff has_bias, ceil(o/4)*4 values of dst_type
- *   5 "params"                present iff a runtime channel bound is set (int32, see below)
+ *   5 "params"                present iff a runtime channel bound or a ring offset is set (int32, see below)
  * (absent objects do not take an index).  dst 0 "dst_tensor": [ceil(o/4)][tokens][4].
  *
  * Zero points (fully_connected_util.cc:91-99: w = u*s - s*(shift + zp)) are taken by every
@@ -298,8 +298,24 @@ typedef struct {
    *     over all groups, :784-794);
    *   dst slices from min(round_up(params[dst_end_ch_index], 32) / 4, ceil(o/4)) on are not
    *     written (fully_connected_util.cc:231-243, fully_connected.cc:644-652).
-   * Ringed weights are refused as the reference refuses them for these weights: uint4 by type,
-   * uint8 I4O4 by layout (fully_connected.cc:1087-1097). */
+   * Ringed weights (ring_o_offset_index / ring_i_offset_index >= 0, ring_size > 0; uint8 weights in
+   * one output group): the weights buffer is a ring along one axis (a key / value cache bound as
+   * weights) whose start is read at launch, offset = params[index] taken modulo ring_size
+   * (fully_connected.cc:676-706).
+   *   ring_i_offset_index, kOSpatialIOGroupI4O4 (GetRingedIAddresses, fully_connected.cc:424-441):
+   *     `i` is the ring's length in input channels, the src tensor has `src_channels` channels, and
+   *     src channel c meets weights row (c + offset) % ring_size; composes with src_end_ch_index.
+   *   ring_o_offset_index, kOSpatialIOGroupO4I4 (GetRingedOAddresses, fully_connected.cc:411-422):
+   *     `o` is the ring's length in output channels (= ring_size, a multiple of 4), the dst tensor has
+   *     `dst_channels` channels, and dst channel c is weights row (c + offset) % ring_size; scales,
+   *     zero points and biases belong to the dst channel.
+   *   With batched weights every matrix is a ring of its own (ring_batch_offset, ring_i_base,
+   *   fully_connected.cc:690-706).
+   * As in the reference (fully_connected.cc:1087-1097), INVALID_ARGUMENT for weights of fewer than 8
+   * bits ("Unsupported WeightsDescription type for ringed weights.") and for the 2D texture layouts
+   * ("Unsupported WeightsDescription layout for ringed weights.").  The integer-math variant does not
+   * apply a ring in the reference (fully_connected.cc:543-621 reads linear_i4o4) and returns
+   * UNIMPLEMENTED here. */
   int32_t has_runtime_check;
   int32_t src_end_ch_index, dst_end_ch_index;
   int32_t ring_o_offset_index, ring_i_offset_index, ring_size;
@@ -314,6 +330,9 @@ typedef struct {
    * packed_max_group_size of them; dst tokens that belong to no group are not written.  "params" is
    * the last src object; mldhip_op_set_shape(op, 1, 1, tokens). */
   int32_t packed_params_offset, packed_num_groups, packed_max_group_size;
+  /* Channels of the src / dst tensors where they differ from the weights' i / o: ringed weights
+   * only (ring_i: src_channels, ring_o: dst_channels); 0 = the weights' own. */
+  int32_t src_channels, dst_channels;
 } mldhip_fc_desc;
 
 int mldhip_fc_create(const mldhip_fc_desc* desc, mldhip_op** op);
@@ -454,7 +473,10 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
  * without an op object: the buffers are passed directly and the split-K sums, which an op keeps in
  * the workspace that its create call allocates, go to an array of 2 MiB that the library holds
  * statically on every GPU it runs on (until the process ends).  Calls no hipMalloc / hipFree.
- * Same kernels and same results as mldhip_op_launch on an op of the same description.
+ * Runs the streaming GEMV kernels (fc_w4_strip_kernel / fc_w4_rows_kernel / fc_w4_stream_kernel), with
+ * the results mldhip_op_launch gives wherever it takes the same kernel (one token always; at 2..4
+ * tokens mldhip_op_launch prefers the matrix-core GEMV for per-channel layers of 8192 channels and
+ * more, whose sums are added in another order).  The current device must be the stream's device.
  * Limits: o <= 65536 (MLDHIP_OUT_OF_RANGE beyond), an even number of 4-channel slices,
  * output_group_size = any even number of slices that divides ceil(o/4) (the reference's one group,
  * 16, the decode layout's 2, ...).  All calls on one GPU share
@@ -465,13 +487,6 @@ int mldhip_fc_launch_gated(mldhip_op* gate, mldhip_op* up, int activation, void*
 int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const void* weights_scale,
                                   const void* biases, void* dst, int o, int i, int scale_groups,
                                   int output_group_size, int tokens, void* stream);
-
-/* Measurement aid, no counterpart in the reference: the two floors that a memory-bound launch is
- * read against on a given box.  kind 0: an empty launch (224 work-groups of 1024 threads);
- * kind 1: a plain streaming read of `bytes` of `src` (whole multiples of 128 KB; 16-byte loads,
- * one contiguous 128 KB run per work-group, nothing kept).  `sink`: at least 4 KB of device memory
- * (never written in practice).  bench.py --workload floors times both the way it times the ops. */
-int mldhip_probe_launch(int kind, const void* src, size_t bytes, void* sink, void* stream);
 
 /* Name of the kernel the last launch used, and the algorithmic bytes / flops of one launch
  * at the current shape (GPUOperation::flops_/read_size_/write_size_,

@@ -101,6 +101,7 @@ struct mldhip_op {
   int idx_weights = 1, idx_ids = -1;
   int idx_params = -1;  // runtime channel bounds
   int weights_batch = 1;  // ExternalWeights::shape.h
+  int src_c = 0, dst_c = 0;  // channels of the src / dst tensors (the weights' i / o unless the weights are ringed)
   int shared_src = 0;     // the source tensor has one row that every dst row reads
   float* partial = nullptr;
   size_t partial_floats = 0;
@@ -382,11 +383,43 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
       return Fail(MLDHIP_UNIMPLEMENTED, "float weights are outside the quantized path");
     return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type.");
   }
-  if (wd.layout != MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4) {
+  // Ringed weights: refused where the reference refuses them (fully_connected.cc:1087-1097: types under
+  // 8 bits, layouts that are not linear = the 2D texture layouts, weights_layout.cc:167-171)
+  const bool ring_i = d->has_runtime_check && d->ring_i_offset_index >= 0;
+  const bool ring_o = d->has_runtime_check && d->ring_o_offset_index >= 0;
+  if (ring_i || ring_o) {
+    if (wd.type == MLDHIP_UINT4) return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type for ringed weights.");
+    if (wd.layout == MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4)
+      return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout for ringed weights.");
+    if (ring_i && ring_o) return Fail(MLDHIP_INVALID_ARGUMENT, "ring_o_offset_index and ring_i_offset_index exclude each other");
+    if (d->ring_size < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "ringed weights need a positive ring_size");
+    // the reference's address arithmetic is written for these two (fully_connected.cc:411-441: "kOSpatialIOGroupO4I4 ->
+    // kBIOI4", "kOSpatialIOGroupI4O4 -> kBIOI4O4")
+    if (wd.layout != (ring_i ? MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4 : MLDHIP_LAYOUT_OSPATIAL_IOGROUP_O4I4))
+      return Fail(MLDHIP_UNIMPLEMENTED, "ring_i_offset_index reads kOSpatialIOGroupI4O4 weights, ring_o_offset_index kOSpatialIOGroupO4I4");
+    if (wd.output_group_size != DivUp(d->o, 4))
+      return Fail(MLDHIP_UNIMPLEMENTED, "ringed weights are read in one output group (output_group_size = ceil(o / 4))");
+    if (d->src_type == MLDHIP_INT8)
+      return Fail(MLDHIP_UNIMPLEMENTED, "the integer-math FullyConnected does not apply a ring (nor does the reference's)");
+    if (d->packed_num_groups > 0) return Fail(MLDHIP_UNIMPLEMENTED, "ringed weights with packed groups are not supported");
+    if (ring_i && (d->ring_size > DivUp(d->i, 4) * 4 || ((batch_ids && weights_batch > 1) && d->ring_size != d->i)))
+      return Fail(MLDHIP_INVALID_ARGUMENT, "ring_size exceeds the weights' input channels (batched weights: must equal them)");
+    if (ring_o && (d->ring_size != d->o || d->o % 4 != 0))
+      return Fail(MLDHIP_INVALID_ARGUMENT, "ring_o_offset_index: ring_size must equal the weights' output channels, a multiple of 4");
+  } else if (wd.layout != MLDHIP_LAYOUT_OSPATIAL_IOGROUP_I4O4) {
     if (wd.layout == MLDHIP_LAYOUT_2D_YSPATIALIO_XOGROUP_I4O4)
       return Fail(MLDHIP_UNIMPLEMENTED, "texture weight layouts are not supported; use the buffer layout");
+    if (wd.layout == MLDHIP_LAYOUT_OSPATIAL_IOGROUP_O4I4)
+      return Fail(MLDHIP_UNIMPLEMENTED, "kOSpatialIOGroupO4I4 weights are served as ringed weights only; use kOSpatialIOGroupI4O4");
     return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout");
   }
+  if (!ring_i && d->src_channels > 0 && d->src_channels != d->i)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "src_channels differs from the weights' input channels without ring_i_offset_index");
+  if (!ring_o && d->dst_channels > 0 && d->dst_channels != d->o)
+    return Fail(MLDHIP_INVALID_ARGUMENT, "dst_channels differs from the weights' output channels without ring_o_offset_index");
+  // channels of the tensors: the weights' own, except along a ringed axis
+  const int src_c = ring_i && d->src_channels > 0 ? d->src_channels : d->i;
+  const int dst_c = ring_o && d->dst_channels > 0 ? d->dst_channels : d->o;
   {
     const int ns = DivUp(d->o, 4);
     // One output group is the layout of FullyConnected (fully_connected.cc:1073-1086); groups of one
@@ -410,29 +443,20 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
     if (d->src_type != tensor_type || d->dst_type != tensor_type)
       return Fail(MLDHIP_INVALID_ARGUMENT, "tensor types do not match the calculations precision");
     if (d->scale_o < 1 || d->scale_i < 1) return Fail(MLDHIP_INVALID_ARGUMENT, "bad scale_zp_shape");
-    if (d->scale_o != 1 && d->scale_o != d->o)
+    if (d->scale_o != 1 && d->scale_o != dst_c)
       return Fail(MLDHIP_INVALID_ARGUMENT, "scale_zp_shape.o must be 1 or the output channel count");
     if (d->scale_o == 1 && d->scale_i != 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "group-wise scales need one row per output channel");
-    if (d->scale_i > 1 && (d->scale_i > d->i / 4 || (d->i % (4 * d->scale_i)) != 0))
+    if (d->scale_i > 1 && (d->scale_i > src_c / 4 || (src_c % (4 * d->scale_i)) != 0))
       return Fail(MLDHIP_INVALID_ARGUMENT, "input channels must split into scale groups of whole 4-channel slices");
     if (d->has_zero_point_tensor && d->scale_o * d->scale_i == 1)
       return Fail(MLDHIP_INVALID_ARGUMENT, "a zero-point tensor needs a scale tensor of the same shape");
   }
   bool runtime_bounds = false, packed_groups = false;
   if (d->has_runtime_check) {
-    // ringed weights: refused as the reference refuses them for these weights (fully_connected.cc:1087-1097)
-    if (d->ring_o_offset_index >= 0 || d->ring_i_offset_index >= 0) {
-      if (wd.type == MLDHIP_UINT4)
-        return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription type for ringed weights.");
-      return Fail(MLDHIP_INVALID_ARGUMENT, "Unsupported WeightsDescription layout for ringed weights.");
-    }
-    runtime_bounds = d->src_end_ch_index >= 0 || d->dst_end_ch_index >= 0;
-    if (runtime_bounds && batch_ids)
-      return Fail(MLDHIP_UNIMPLEMENTED, "runtime channel bounds with batched weights are not supported");
+    runtime_bounds = d->src_end_ch_index >= 0 || d->dst_end_ch_index >= 0 || ring_i || ring_o;
     if (d->packed_num_groups > 0) {
       if (batch_ids) return Fail(MLDHIP_INVALID_ARGUMENT, "packed groups and batch ids exclude each other");
-      if (int8_math) return Fail(MLDHIP_UNIMPLEMENTED, "packed groups: floating-point FullyConnected only");
       if (d->packed_params_offset < 0 || d->packed_max_group_size < 1)
         return Fail(MLDHIP_INVALID_ARGUMENT, "packed groups need a params offset >= 0 and a positive max_group_size");
       packed_groups = true;
@@ -443,7 +467,10 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   if (!op) return Fail(MLDHIP_INTERNAL, "out of memory");
   op->kind = mldhip_op::kFc;
   op->fc = *d;
-  if (!d->has_runtime_check) op->fc.src_end_ch_index = op->fc.dst_end_ch_index = -1;
+  if (!d->has_runtime_check)
+    op->fc.src_end_ch_index = op->fc.dst_end_ch_index = op->fc.ring_i_offset_index = op->fc.ring_o_offset_index = -1;
+  op->src_c = src_c;
+  op->dst_c = dst_c;
   if (!packed_groups) op->fc.packed_num_groups = 0;
   if (packed_groups) op->weights_batch = weights_batch;
   op->max_tokens = d->max_tokens;
@@ -612,18 +639,20 @@ static void RequiredSizes(const mldhip_op* op, std::vector<size_t>* src, std::ve
   dst->assign(op->dst_ptr.size(), 0);
   if (op->kind == mldhip_op::kFc) {
     const mldhip_fc_desc& d = op->fc;
-    const size_t ks = DivUp(d.i, 4), ns = DivUp(d.o, 4);
+    // tensor slices, and the slices of the weights' own shape (they differ along a ringed axis)
+    const size_t ks = DivUp(op->src_c, 4), ns = DivUp(op->dst_c, 4);
+    const size_t wks = DivUp(d.i, 4), wns = DivUp(d.o, 4);
     const size_t wbatch = (size_t)op->weights_batch;
     // batched weights: h rows of w tokens; a shared source has one row
     (*src)[0] = ks * (op->shared_src ? (size_t)op->w : m) * 4 * TypeBytes(d.src_type);
     if (op->idx_ids >= 0) (*src)[op->idx_ids] = (size_t)op->h * sizeof(int32_t);
-    (*src)[op->idx_weights] = wbatch * ks * ns * 16 * WeightBits(d.weights.type) / 8;
+    (*src)[op->idx_weights] = wbatch * wks * wns * 16 * WeightBits(d.weights.type) / 8;
     const size_t tb = TypeBytes(d.src_type);
     if (op->idx_scale >= 0) (*src)[op->idx_scale] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_zp >= 0) (*src)[op->idx_zp] = (size_t)d.scale_i * wbatch * ns * 4 * tb;
     if (op->idx_bias >= 0) (*src)[op->idx_bias] = ns * 4 * TypeBytes(d.dst_type);
     if (op->idx_params >= 0) {
-      int values = std::max(d.src_end_ch_index, d.dst_end_ch_index) + 1;
+      int values = std::max(std::max(d.src_end_ch_index, d.dst_end_ch_index), std::max(d.ring_i_offset_index, d.ring_o_offset_index)) + 1;
       if (d.packed_num_groups > 0) values = std::max(values, d.packed_params_offset + 2 * d.packed_num_groups);
       (*src)[op->idx_params] = (size_t)values * sizeof(int32_t);
     }
@@ -696,8 +725,9 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
     a.weights_batch = op->weights_batch;
     a.m = op->w;  // tokens per row
   }
-  a.k = d.i;
-  a.n = d.o;
+  a.k = op->src_c;
+  a.n = op->dst_c;
+  a.weights_k = d.i;
   a.act_f16 = d.src_type == MLDHIP_FLOAT16;
   a.dst_f16 = d.dst_type == MLDHIP_FLOAT16;
   a.weight_bits = WeightBits(d.weights.type);
@@ -713,6 +743,9 @@ static int BuildFcArgs(mldhip_op* op, FcArgs* out) {
     a.params = static_cast<const int32_t*>(op->src_ptr[op->idx_params]);
     a.src_end_ch_index = d.src_end_ch_index;
     a.dst_end_ch_index = d.dst_end_ch_index;
+    a.ring_i_index = d.ring_i_offset_index;
+    a.ring_o_index = d.ring_o_offset_index;
+    a.ring_size = d.ring_size;
     if (d.packed_num_groups > 0) {
       a.packed_params_offset = d.packed_params_offset;
       a.packed_max_group_size = d.packed_max_group_size;
@@ -746,6 +779,11 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
         batch.params = static_cast<const int32_t*>(op->src_ptr[op->idx_params]);
         batch.src_end_ch_index = d.src_end_ch_index;
         batch.dst_end_ch_index = d.dst_end_ch_index;
+        if (d.packed_num_groups > 0) {  // one launch plane per matrix over the one row of tokens
+          batch.packed_params_offset = d.packed_params_offset;
+          batch.packed_max_group_size = d.packed_max_group_size;
+          batch.weights_batch = op->weights_batch;
+        }
       }
       const int8_t* act = static_cast<const int8_t*>(op->src_ptr[0]);
       const uint8_t* weights = static_cast<const uint8_t*>(op->src_ptr[op->idx_weights]);
@@ -930,13 +968,6 @@ int mldhip_fc_int4_decode_noalloc(const void* src, const void* weights, const vo
   return MLDHIP_OK;
 }
 
-int mldhip_probe_launch(int kind, const void* src, size_t bytes, void* sink, void* stream_ptr) {
-  if (!sink || (kind == 1 && !src)) return Fail(MLDHIP_INVALID_ARGUMENT, "null device pointer");
-  hipError_t e = LaunchProbe(kind, src, bytes, sink, static_cast<hipStream_t>(stream_ptr));
-  if (e != hipSuccess) return HipFail(e, "probe launch");
-  return MLDHIP_OK;
-}
-
 const char* mldhip_op_kernel_name(const mldhip_op* op) { return op ? op->last_kernel : ""; }
 
 int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {
@@ -957,7 +988,7 @@ int mldhip_op_cost(const mldhip_op* op, uint64_t* bytes, uint64_t* flops) {
   if (flops) {
     const uint64_t m = (uint64_t)op->Tokens();
     if (op->kind == mldhip_op::kFc)
-      *flops = 2 * m * (uint64_t)op->fc.i * (uint64_t)op->fc.o;
+      *flops = 2 * m * (uint64_t)op->src_c * (uint64_t)op->dst_c;
     else if (op->kind == mldhip_op::kConvInt8)
       *flops = 2 * m * (uint64_t)op->cv.i * (uint64_t)op->cv.o;
     else

@@ -61,6 +61,10 @@ struct GenericParams {
   // packed groups (fully_connected_util.cc:263-277; fully_connected.cc:706-710, 810-816): blockIdx.z =
   // weight matrix g; its tokens are params[off + g] many from token params[off + weights_batch + g]
   int packed_params_offset, packed_max_group_size;
+  // ringed weights (fully_connected.cc:411-441, 676-706; uint8 only): 1 = ring over the input channels
+  // of an I4O4 buffer of w_ks K-slices, 2 = ring over the output channels of an O4I4 buffer; the
+  // offset is params[ring_index] modulo ring_size
+  int ring_kind, ring_index, ring_size, w_ks;
 };
 
 // K-slices the loop covers and dst slices that are written, with runtime channel bounds
@@ -116,6 +120,9 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
 
   const int ks_end = RuntimeSrcEndSlices(p.params, p.src_end_ch_index, p.k_channels, p.ks, p.scale_kind == kScaleBlock);
   const int ns_end = RuntimeDstEndSlice(p.params, p.dst_end_ch_index, p.ns);
+  // ring start: ((offset % ring_size) + ring_size) % ring_size (fully_connected.cc:678-679, 699-700)
+  int ring_off = 0;
+  if (WBITS == 8 && p.ring_kind != 0) ring_off = ((p.params[p.ring_index] % p.ring_size) + p.ring_size) % p.ring_size;
   if (ds < ns_end) {
     float s[4], z[4];
 #pragma unroll
@@ -144,7 +151,40 @@ __global__ __launch_bounds__(256) void fc_generic_kernel(GenericParams p) {
       }
       const size_t blk = BatchedBlockIndex(ks, ds, wb, p.weights_batch, p.ks, p.ns, p.wgroup);
       float wf[4][4];
-      if (WBITS == 8) {
+      if (WBITS == 8 && p.ring_kind != 0) {
+        // four 4-byte reads with addresses of their own (ReadRingedWeightsAsFloat, fully_connected.cc:443-471)
+        const uint32_t* w32 = reinterpret_cast<const uint32_t*>(weights);
+        uint32_t w[4];
+        if (p.ring_kind == 1) {
+          // rows of 4 output channels: a = (i >> 2) * dst_stride + (i & 3) + ring_i_base, dst_stride =
+          // 4 * Ns, ring_i_base = dst_s * 4 + w_batch_id * ring_size * Ns (fully_connected.cc:424-441, 701-706)
+          const size_t base = (size_t)wb * p.ring_size * p.ns + (size_t)ds * 4;
+          int ij = (ks * 4 + ring_off) % p.ring_size;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            w[i] = w32[base + (size_t)(ij >> 2) * p.ns * 4 + (ij & 3)];
+            ij = ij + 1 >= p.ring_size ? ij + 1 - p.ring_size : ij + 1;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) wf[i][c] = ((float)((w[i] >> (8 * c)) & 0xFFu) - (shift + z[c])) * s[c];
+        } else {
+          // rows of 4 input channels: a = src_s * ring_size + o + w_batch_id * ring_size * Ks
+          // (fully_connected.cc:411-422, 680-697); scale and zero point belong to the dst channel
+          const size_t base = ((size_t)wb * p.ks + ks) * p.ring_size;
+          int oc = (ds * 4 + ring_off) % p.ring_size;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            w[c] = w32[base + oc];
+            oc = oc + 1 >= p.ring_size ? oc + 1 - p.ring_size : oc + 1;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) wf[i][c] = ((float)((w[c] >> (8 * i)) & 0xFFu) - (shift + z[c])) * s[c];
+        }
+      } else if (WBITS == 8) {
         const u32x4 w = *reinterpret_cast<const u32x4*>(weights + blk * 16);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -222,8 +262,20 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
   const int row = blockIdx.z;
   int wb = batch.ids ? batch.ids[row] : 0;
   wb = min(max(wb, 0), batch.weights_batch - 1);
-  const size_t act_stride = (size_t)batch.src_rows * m, dst_stride = (size_t)batch.rows * m;
-  const size_t act_tok0 = (size_t)min(row, batch.src_rows - 1) * m, dst_tok0 = (size_t)row * m;
+  size_t act_stride = (size_t)batch.src_rows * m, dst_stride = (size_t)batch.rows * m;
+  size_t act_tok0 = (size_t)min(row, batch.src_rows - 1) * m, dst_tok0 = (size_t)row * m;
+  int tok_count = m;  // tokens of this row: tok0 + t < tok_count
+  if (batch.packed_params_offset >= 0) {
+    // packed groups (fully_connected_util.cc:263-277; fully_connected.cc:706-710, 810-816): one row of m
+    // tokens; this plane's matrix owns tok_count of them from token dst_tok0 on
+    wb = row;
+    const int size = batch.params[batch.packed_params_offset + row];
+    const int offset = batch.params[batch.packed_params_offset + batch.weights_batch + row];
+    tok_count = min(min(size, batch.packed_max_group_size), m - offset);
+    act_stride = dst_stride = (size_t)m;
+    act_tok0 = dst_tok0 = (size_t)max(offset, 0);
+    if (offset < 0 || tok0 >= tok_count) return;  // (the whole work-group: no barrier is left waiting)
+  }
   int acc[TB][4];
 #pragma unroll
   for (int t = 0; t < TB; ++t)
@@ -272,7 +324,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
 #pragma unroll
       for (int t = 0; t < TB; ++t) {
         const int tok = tok0 + t;
-        if (tok >= m) continue;
+        if (tok >= tok_count) continue;
         const int v = *reinterpret_cast<const int*>(act + ((size_t)ks * act_stride + act_tok0 + tok) * 4);
         acc[t][0] = __builtin_amdgcn_sdot4(v, (int)w0, acc[t][0], false);
         acc[t][1] = __builtin_amdgcn_sdot4(v, (int)w1, acc[t][1], false);
@@ -298,7 +350,7 @@ __global__ __launch_bounds__(256) void fc_int8_math_kernel(const int8_t* __restr
 #pragma unroll
     for (int t = 0; t < TB; ++t) {
       const int tok = tok0 + t;
-      if (tok >= m) continue;
+      if (tok >= tok_count) continue;
 #pragma unroll
       for (int c = 0; c < 4; ++c)
       {
@@ -341,6 +393,16 @@ hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** ker
   p.k_channels = a.k;
   p.packed_params_offset = a.params ? a.packed_params_offset : -1;
   p.packed_max_group_size = a.packed_max_group_size;
+  p.ring_kind = a.params && a.ring_i_index >= 0 ? 1 : (a.params && a.ring_o_index >= 0 ? 2 : 0);
+  p.ring_index = p.ring_kind == 1 ? a.ring_i_index : a.ring_o_index;
+  p.ring_size = a.ring_size;
+  p.w_ks = DivUp(a.weights_k > 0 ? a.weights_k : a.k, 4);
+  if (p.ring_kind != 0 && (a.weight_bits != 8 || a.ring_size < 1 || a.packed_params_offset >= 0 ||
+                           EffectiveGroup(a.group, p.ns) != p.ns))
+    return hipErrorInvalidValue;
+  if (p.ring_kind == 1 && (a.ring_size > 4 * p.w_ks || (a.weights_batch > 1 && a.ring_size != 4 * p.w_ks)))
+    return hipErrorInvalidValue;
+  if (p.ring_kind == 2 && a.ring_size % 4 != 0) return hipErrorInvalidValue;
   if (p.packed_params_offset >= 0 && (a.batch_ids != nullptr || a.packed_max_group_size < 1 || a.weights_batch < 1))
     return hipErrorInvalidValue;
   if (kernel_name) *kernel_name = "fc_generic_kernel";
@@ -360,6 +422,11 @@ hipError_t LaunchFcInt8Math(const int8_t* act, const uint8_t* weights, int32_t* 
   constexpr int TB = 4;
   const int ks = DivUp(k, 4), ns = DivUp(n, 4);
   dim3 grid(DivUp(ns, kSl), DivUp(m, TB), batch.ids ? batch.rows : 1);
+  if (batch.packed_params_offset >= 0) {
+    if (batch.ids != nullptr || batch.params == nullptr || batch.packed_max_group_size < 1 || batch.weights_batch < 1)
+      return hipErrorInvalidValue;
+    grid = dim3(DivUp(ns, kSl), DivUp(std::min(m, batch.packed_max_group_size), TB), batch.weights_batch);
+  }
   dim3 block(kSl, kKl);
   if (kernel_name) *kernel_name = "fc_int8_math_kernel";
   if (weight_bits == 8)

@@ -77,6 +77,12 @@ struct FcArgs {
   // tokens of the one source row are sorted by weight matrix; params[offset + g] tokens starting at
   // token params[offset + weights_batch + g] are multiplied with matrix g.  offset < 0 = not set.
   int packed_params_offset = -1, packed_max_group_size = 0;
+  // Ringed weights (fully_connected.cc:411-441, 676-706; uint8, one output group, the unspecialised
+  // kernel): the offset is params[ring_*_index] modulo ring_size.  ring_i: k = src channels, the
+  // I4O4 buffer holds weights_k input channels; ring_o: n = dst channels, the O4I4 buffer holds
+  // ring_size output channels.
+  int ring_o_index = -1, ring_i_index = -1, ring_size = 0;
+  int weights_k = 0;  // input channels of the weights buffer (ring_i); 0 = k
 };
 
 // Split-K workspace sizing for the streaming GEMV.
@@ -121,6 +127,8 @@ struct FcBatchRows {
   // runtime channel bounds, as in FcArgs (the tiled kernel only)
   const int32_t* params = nullptr;
   int src_end_ch_index = -1, dst_end_ch_index = -1;
+  // packed groups, as in FcArgs (the tiled kernel only): one launch plane per matrix
+  int packed_params_offset = -1, packed_max_group_size = 0;
 };
 
 // int8 activations x uint8/uint4 weights -> int32 (no scales).
@@ -146,10 +154,6 @@ struct Tuning {
   int gemm_i8_fm = -1;
 };
 Tuning& GetTuning();
-
-// Measurement aids (mldhip_probe_launch): kind 0 = an empty launch of 224 x 1024 threads, kind 1 = a
-// plain streaming read of `bytes` (whole multiples of 128 KB are read).
-hipError_t LaunchProbe(int kind, const void* src, size_t bytes, void* sink, hipStream_t stream);
 
 struct QuantArgs {
   const void* src = nullptr;

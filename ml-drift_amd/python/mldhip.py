@@ -34,7 +34,6 @@ SYMBOLS = [
     "mldhip_checkpoint_fc_probe", "mldhip_checkpoint_fc_read", "mldhip_fc_launch_gated",
     "mldhip_scale_to_tensor_batched", "mldhip_fc_batch_ids_create",
     "mldhip_fc_int4_weights_desc_reference", "mldhip_fc_int4_weights_desc_decode", "mldhip_fc_int8_weights_desc_decode", "mldhip_set_tuning", "mldhip_fc_int4_decode_noalloc",
-    "mldhip_probe_launch",
 ]
 
 
@@ -54,7 +53,7 @@ class FcDesc(C.Structure):
                 ("src_end_ch_index", C.c_int32), ("dst_end_ch_index", C.c_int32),
                 ("ring_o_offset_index", C.c_int32), ("ring_i_offset_index", C.c_int32), ("ring_size", C.c_int32),
                 ("packed_params_offset", C.c_int32), ("packed_num_groups", C.c_int32),
-                ("packed_max_group_size", C.c_int32)]
+                ("packed_max_group_size", C.c_int32), ("src_channels", C.c_int32), ("dst_channels", C.c_int32)]
 
 
 class QuantDesc(C.Structure):
@@ -120,7 +119,6 @@ def lib():
         _lib.mldhip_op_destroy.restype = None
         _lib.mldhip_set_tuning.argtypes = [C.c_char_p, C.c_int]
         _lib.mldhip_fc_int4_decode_noalloc.argtypes = [C.c_void_p] * 5 + [C.c_int] * 5 + [C.c_void_p]
-        _lib.mldhip_probe_launch.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     return _lib
 
 
@@ -402,9 +400,11 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
               scalar_scale=1.0, has_zero_point_tensor=False, scalar_zero_point=None,
               has_bias=False, max_tokens=1, weights_batch=None, shared_src=False, src_end_ch_index=None,
               dst_end_ch_index=None, ring_o_offset_index=None, ring_i_offset_index=None, ring_size=0,
-              packed_groups=None):
+              packed_groups=None, src_channels=0, dst_channels=0):
     """weights_batch: number of weight matrices of a batch-ids op (mldhip_fc_batch_ids_create).
     src_end_ch_index / dst_end_ch_index: ConvRuntimeCheckDesc indices into the "params" object.
+    ring_o_offset_index / ring_i_offset_index, ring_size: ringed weights (src_channels / dst_channels:
+    channels of the tensors where they differ from the weights' i / o).
     packed_groups: (params_offset, num_groups, max_group_size) of ConvRuntimeCheckDesc::PackedGroups."""
     d = FcDesc()
     d.precision, d.src_type, d.dst_type, d.o, d.i = precision, src_type, dst_type, o, i
@@ -423,6 +423,7 @@ def fc_create(precision, src_type, dst_type, o, i, weights_desc, scale_shape=(1,
     d.src_end_ch_index, d.dst_end_ch_index, d.ring_o_offset_index, d.ring_i_offset_index = [
         -1 if v is None else v for v in checks]
     d.ring_size = ring_size
+    d.src_channels, d.dst_channels = src_channels, dst_channels
     h = C.c_void_p()
     if weights_batch is not None:
         check(lib().mldhip_fc_batch_ids_create(C.byref(d), weights_batch, int(shared_src), C.byref(h)))
@@ -456,10 +457,3 @@ def fc_int4_decode_noalloc(src, weights, scale, bias, dst, o, i, scale_groups, o
     ptr = lambda t: None if t is None else C.c_void_p(t.data_ptr())
     check(lib().mldhip_fc_int4_decode_noalloc(ptr(src), ptr(weights), ptr(scale), ptr(bias), ptr(dst), o, i,
                                               scale_groups, output_group_size, tokens, C.c_void_p(stream)))
-
-
-def probe_launch(kind, src, sink, stream=0):
-    """mldhip_probe_launch over torch tensors: kind 0 = empty launch, 1 = streaming read of `src`."""
-    nbytes = 0 if src is None else src.numel() * src.element_size()
-    check(lib().mldhip_probe_launch(kind, None if src is None else C.c_void_p(src.data_ptr()), nbytes,
-                                    C.c_void_p(sink.data_ptr()), C.c_void_p(stream)))

@@ -2,6 +2,23 @@
 
 Only tests, the smoke check and the benchmark's cpu_baseline leg import this module; the
 product package never does.  Functions take and return numpy arrays.
+
+The restatements written here in numpy on top of the C kernel restatement, and what pins each
+(the C functions' pins are listed in mld_oracle.c):
+  fc_kernel_runtime_check   literal end-slice values and the reference's four runtime-channel cases
+                            (K = 171, N = 533) against the float product over the aligned bounds
+  fc_batch_ids_kernel       the reference's own test shapes against FullyConnectedWeightsBatchIdsReference
+                            restated per row, and the id-permutation property
+  fc_packed_groups_kernel   the reference test's flow (sort by matrix, run, unsort) against per-token
+                            float64 products
+  ringed_gather / fc_ringed_kernel
+                            what the mathematics fixes: a ring offset r equals the plain FullyConnected
+                            over the weights rolled by r along I (ring_i) or O (ring_o), computed in
+                            float64 from the unpacked values, on the sizes and offsets of the
+                            reference's FullyConnectedRingedITest / RingedOTest (72 / 20 / 56 channels,
+                            offsets 0, 17, 20, 33, 49, one and three matrices), plus negative and
+                            beyond-the-ring offsets and the composition with src_end_ch
+  gated_activation          closed forms (0 at 0, g * u for large g, the clamps)
 """
 import ctypes as C
 import os
@@ -281,6 +298,70 @@ def fc_kernel_runtime_check(act_slices, weights, m, k, n, precision, weight_bits
                          weight_bits, scale_kind, scale, zero_point, bias, groups)
     out[:ns_end] = full[:ns_end]
     return out
+
+
+def ringed_gather(weights, ring_axis, ring_size, ring_offset, src_slices, dst_slices, batch_id=0):
+    """The 16-byte I4O4 blocks (word i = input channel i of the K-slice, byte c = output channel c of the
+    dst slice) that the generated kernel assembles from ringed uint8 weights, for every (src_s, dst_s),
+    by the reference's own address arithmetic on 4-byte words (ReadRingedWeightsAsFloat,
+    common/kernels/fully_connected.cc:443-471):
+      ring_axis "i" (kOSpatialIOGroupI4O4 buffer, GetRingedIAddresses :424-441 with :699-706):
+        ring_i_offset = ((offset % ring_size) + ring_size) % ring_size; i0 = (src_s * 4 + ring_i_offset) %
+        ring_size, i1..i3 = i0 + 1..3 wrapped once; word j at (ij >> 2) * dst_stride + (ij & 3) + ring_i_base,
+        dst_stride = 4 * dst slices, ring_i_base = dst_s * 4 + w_batch_id * ring_size * dst slices;
+      ring_axis "o" (kOSpatialIOGroupO4I4 buffer, GetRingedOAddresses :411-422 with :676-697):
+        o0 = (dst_s * 4 + ring_o_offset) % ring_size, o1..o3 wrapped once; word c at src_s * ring_size + oc
+        + w_batch_id * ring_size * src slices holds the 4 input channels of output oc, so the I4O4 block is
+        its byte transpose.
+    Returns uint8 [src_slices][dst_slices][16]: the packed buffer (one output group) of an unringed
+    FullyConnected with the same results."""
+    w32 = _c(weights, np.uint8).view(np.uint32)
+    off = ((int(ring_offset) % ring_size) + ring_size) % ring_size
+    if ring_axis == "i":
+        src_s = np.arange(src_slices)[:, None, None]
+        dst_s = np.arange(dst_slices)[None, :, None]
+        j = np.arange(4)[None, None, :]
+        i0 = (src_s * 4 + off) % ring_size
+        ij = i0 + j
+        ij = np.where(ij >= ring_size, ij - ring_size, ij)
+        addr = (ij >> 2) * (dst_slices * 4) + (ij & 3) + dst_s * 4 + batch_id * ring_size * dst_slices
+        words = w32[addr]  # [src_s][dst_s][word j]
+        return np.ascontiguousarray(words).view(np.uint8).reshape(src_slices, dst_slices, 16)
+    assert ring_axis == "o"
+    src_s = np.arange(src_slices)[:, None, None]
+    dst_s = np.arange(dst_slices)[None, :, None]
+    c = np.arange(4)[None, None, :]
+    o0 = (dst_s * 4 + off) % ring_size
+    oc = o0 + c
+    oc = np.where(oc >= ring_size, oc - ring_size, oc)
+    addr = src_s * ring_size + oc + batch_id * ring_size * src_slices
+    words = np.ascontiguousarray(w32[addr]).view(np.uint8).reshape(src_slices, dst_slices, 4, 4)  # [c][i]
+    return np.ascontiguousarray(words.transpose(0, 1, 3, 2)).reshape(src_slices, dst_slices, 16)  # [i][c]
+
+
+def fc_ringed_kernel(act_slices, weights, m, src_channels, dst_channels, ring_axis, ring_size, ring_offset, precision,
+                     scale_kind=SCALE_LINEAR, scale=None, zero_point=None, bias=None, groups=1, src_end_ch=None,
+                     dst_end_ch=None, batch_id=0, dst_before=None, scalar_scale=1.0, scalar_zero_point=0.0):
+    """The generated kernel over ringed uint8 weights (ConvRuntimeCheckDesc::ring_i_offset_index /
+    ring_o_offset_index, common/kernels/fully_connected.cc:676-706, 411-471): it differs from the plain
+    kernel only in where the four weight words of a (src_s, dst_s) step come from, so this restatement
+    gathers them (`ringed_gather`) and runs `fc_kernel_runtime_check` on the result.  Scales, zero points
+    and biases are read at the dst slice (fully_connected.cc:762-776), i.e. they belong to the dst channel,
+    not to the ring position.  For ring_axis "o" the reference accumulates `r.c += dot(v, w_c)` per output
+    (fully_connected_util.cc:186-199), whose summation order inside dot() is the compiler's; the I4O4
+    order used here is one valid choice (results agree within the FullyConnected tolerance, not bit for
+    bit).  `weights`: the packed ring buffer (all matrices); `batch_id`: the matrix of this dst row."""
+    ks, ns = div_up(src_channels, 4), div_up(dst_channels, 4)
+    blocks = ringed_gather(weights, ring_axis, ring_size, ring_offset, ks, ns, batch_id)
+    if scale_kind == SCALE_SCALAR:
+        tdt = np.float32 if precision == PREC_F32 else np.uint16
+        out = fc_kernel(act_slices, blocks, m, src_channels, dst_channels, precision, 8, scale_kind, None, None, bias, 1,
+                        scalar_scale=scalar_scale, scalar_zero_point=scalar_zero_point)
+        assert src_end_ch is None and dst_end_ch is None
+        return out.astype(tdt)
+    return fc_kernel_runtime_check(act_slices, blocks, m, src_channels, dst_channels, precision, 8, scale_kind, scale,
+                                   zero_point, bias, groups, src_end_ch=src_end_ch, dst_end_ch=dst_end_ch,
+                                   dst_before=dst_before)
 
 
 def fc_batch_ids_kernel(act_slices, ids, weights, rows, row_tokens, src_rows, weights_batch, k, n, precision,

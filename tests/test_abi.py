@@ -90,8 +90,9 @@ def test_fc_create_rejects_what_the_reference_rejects():
     msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_group)
     assert "output_group_size" in msg  # fully_connected.cc:1107-1110
     bad_layout = M.make_desc(M.UINT4, M.LAYOUT_O4I4, 16)
-    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_layout)
-    assert "layout" in msg  # fully_connected.cc:1111-1115
+    # the reference reads kOSpatialIOGroupO4I4 as a linear layout; this library serves it for ringed weights only
+    msg = expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_layout)
+    assert "kOSpatialIOGroupO4I4" in msg
     bad_type = M.make_desc(M.INT32, M.LAYOUT_I4O4, 16)
     expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F16, M.FLOAT16, M.FLOAT16, 64, 64, bad_type)
     # precision / tensor type mismatch (fully_connected.cc:1098-1102 for the weights; same rule for tensors)
@@ -194,8 +195,10 @@ def test_scale_to_tensor_batched_matches_oracle(oracle):
 
 
 def test_runtime_check_objects_and_ringed_weights():
-    """Runtime channel bounds add a last src object "params"; ringed weights are refused with the
-    reference's messages (common/kernels/fully_connected.cc:1087-1097)."""
+    """Runtime channel bounds and ring offsets add a last src object "params".  Ringed weights are refused
+    where the reference refuses them, with its messages (common/kernels/fully_connected.cc:1087-1097:
+    types under 8 bits; layouts that are not linear, i.e. the 2D texture layouts,
+    common/task/weights_layout.cc:167-171); uint8 weights in the two buffer layouts are served."""
     d4 = M.fc_int4_weights_desc(64, 64)
     op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4, scale_shape=(64, 1), has_bias=True,
                      src_end_ch_index=1, dst_end_ch_index=3)
@@ -203,6 +206,28 @@ def test_runtime_check_objects_and_ringed_weights():
     msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4,
                        scale_shape=(64, 1), ring_o_offset_index=0, ring_size=64)
     assert "type for ringed weights" in msg
-    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64,
-                       M.fc_int8_weights_desc(64, 64), scale_shape=(64, 1), ring_i_offset_index=0, ring_size=64)
+    d2d = M.make_desc(M.UINT8, M.LAYOUT_2D_I4O4, 16)
+    msg = expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d2d,
+                       scale_shape=(64, 1), ring_i_offset_index=0, ring_size=64)
     assert "layout for ringed weights" in msg
+    # uint8, kOSpatialIOGroupI4O4: a ring over the input channels (20 src channels against 56 ring rows)
+    d8 = M.fc_int8_weights_desc(72, 56)
+    op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 72, 56, d8, scale_shape=(72, 1), has_bias=True,
+                     ring_i_offset_index=0, src_end_ch_index=1, ring_size=56, src_channels=20)
+    assert op.src_names == ["src_tensor", "weights", "weights_scale", "biases", "params"]
+    # uint8, kOSpatialIOGroupO4I4: a ring over the output channels (20 dst channels out of 56 ring rows)
+    do = M.make_desc(M.UINT8, M.LAYOUT_O4I4, 14)
+    op = M.fc_create(M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 56, 72, do, scale_shape=(20, 1),
+                     ring_o_offset_index=0, ring_size=56, dst_channels=20)
+    assert op.src_names == ["src_tensor", "weights", "weights_scale", "params"]
+    # what this library adds to the reference's refusals carries messages of its own
+    expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 56, 72, do, scale_shape=(56, 1))
+    expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 56, 72, d8, scale_shape=(56, 1),
+                 ring_o_offset_index=0, ring_size=56)
+    expect_error(M.UNIMPLEMENTED, M.fc_create, M.PRECISION_F32, M.INT8, M.INT32, 72, 56, d8, ring_i_offset_index=0, ring_size=56)
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 72, 56, d8, scale_shape=(72, 1),
+                 ring_i_offset_index=0, ring_size=0)
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 72, 56, d8, scale_shape=(72, 1),
+                 ring_i_offset_index=0, ring_size=64)
+    expect_error(M.INVALID_ARGUMENT, M.fc_create, M.PRECISION_F32, M.FLOAT32, M.FLOAT32, 72, 56, d8, scale_shape=(72, 1),
+                 src_channels=20)

@@ -167,6 +167,41 @@ def test_packed_groups_arguments():
     with pytest.raises(M.MldhipError) as e:
         M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d, scale_shape=(64, 1), packed_groups=(0, 4, 0))
     assert e.value.code == M.INVALID_ARGUMENT
-    with pytest.raises(M.MldhipError) as e:
-        M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 64, 64, d, packed_groups=(0, 4, 8))
-    assert e.value.code == M.UNIMPLEMENTED
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, 64, 64, d, packed_groups=(0, 4, 8))
+    assert op.src_names == ["src_tensor", "weights", "params"]
+
+
+@pytest.mark.parametrize("bits,width,per_item,k,n,batch,group", [
+    (8, 64, 4, 64, 32, 16, None), (4, 40, 3, 112, 152, 5, None), (4, 96, 2, 768, 512, 8, 16), (8, 7, 1, 64, 20, 4, 1)])
+def test_integer_math_variant(bits, width, per_item, k, n, batch, group):
+    """Packed groups on the integer-math FullyConnected (int8 sources -> int32; the reference's kernel has
+    the group parameters in both variants, common/kernels/fully_connected.cc:706-710, 810-816): every token
+    of a group against its matrix, bit for bit against the integer product; tokens outside every group
+    keep what the tensor held."""
+    import torch
+    c = make_packed_groups_case(width + n, width, per_item, k, n, batch, bits)
+    rng = np.random.default_rng(width)
+    tokens = c["packed_src"].shape[0]
+    src = rng.integers(-128, 128, size=(tokens, k), dtype=np.int8)
+    desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    if group is not None:
+        desc.output_group_size = group
+    packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(c["w"], desc)
+    sizes, offsets = c["sizes"].copy(), c["offsets"].copy()
+    sizes[0] = max(0, sizes[0] - 1)  # the last token of the first group belongs to no group
+    params = np.concatenate([[77], sizes, offsets]).astype(np.int32)
+    ns = W.div_up(n, 4)
+    out = torch.full((ns, tokens, 4), -5, dtype=torch.int32, device="cuda")
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=tokens, packed_groups=(1, batch, tokens))
+    op.bind([torch.from_numpy(W.to_slices(src)).cuda(), torch.from_numpy(packed).cuda(), torch.from_numpy(params).cuda()], [out])
+    op.set_shape(1, 1, tokens)
+    print("packed groups int8 math", bits, tokens, k, n, batch, group, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert op.kernel_name == "fc_int8_math_kernel", op.kernel_name
+    got = W.from_slices(out.cpu().numpy(), n)
+    ref = np.full((tokens, n), -5, np.int64)
+    for g in range(batch):
+        for t in range(int(offsets[g]), int(offsets[g]) + int(sizes[g])):
+            ref[t] = c["w"][:, g, 0, :].astype(np.int64) @ src[t].astype(np.int64)
+    assert np.array_equal(got, ref)

@@ -100,12 +100,70 @@ def test_bounds_are_read_at_launch(oracle):
     assert np.array_equal(a[:16], b[:16]) and np.all(a[16:] == 7.0) and not np.any(b == 7.0)
 
 
-def test_ringed_weights_are_refused_like_the_reference():
-    d4 = M.fc_int4_weights_desc(64, 64)
-    with pytest.raises(M.MldhipError) as e:
-        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d4, scale_shape=(64, 1), ring_o_offset_index=0, ring_size=64)
-    assert e.value.code == M.INVALID_ARGUMENT and "type for ringed weights" in e.value.message
-    d8 = M.fc_int8_weights_desc(64, 64)
-    with pytest.raises(M.MldhipError) as e:
-        M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, 64, 64, d8, scale_shape=(64, 1), ring_i_offset_index=0, ring_size=64)
-    assert e.value.code == M.INVALID_ARGUMENT and "layout for ringed weights" in e.value.message
+@pytest.mark.parametrize("bits,td", [(8, np.float32), (4, np.float16), (8, np.int8), (4, np.int8)])
+def test_runtime_bounds_with_batched_weights(oracle, bits, td):
+    """ConvRuntimeCheckDesc is independent of batched weights in the reference (common/kernels/
+    fully_connected.cc:1123-1128: conv_params.runtime_check beside batched_weights): every dst row runs the
+    bounded kernel with the matrix its id selects.  Floating-point variant against the oracle's bounded
+    restatement per row; integer-math variant (np.int8) bit for bit against the integer product over the
+    bounded K range."""
+    import torch
+    o = oracle
+    rows, k, n, batch, src_end, dst_end = 5, 172, 536, 4, 61, 200
+    rng = np.random.default_rng(bits)
+    lim = 127 if bits == 8 else 7
+    w = rng.integers(-lim, lim + 1, size=(n, batch, 1, k), dtype=np.int8)
+    ids = np.array([2, 0, 3, 3, 1], np.int32)
+    int8_math = td == np.int8
+    desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
+    packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(w, desc)
+    ks, ns = (k + 3) // 4, (n + 3) // 4
+    ks_end, ns_end = o.runtime_end_slices(src_end, dst_end, k, n, False)
+    params = torch.tensor([-1, src_end, -1, dst_end], dtype=torch.int32, device="cuda")
+    if int8_math:
+        src = rng.integers(-128, 128, size=(rows, k), dtype=np.int8)
+        out = torch.full((ns, rows, 4), -5, dtype=torch.int32, device="cuda")
+        op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=rows, weights_batch=batch,
+                         src_end_ch_index=1, dst_end_ch_index=3)
+        assert op.src_names == ["src_tensor", "batch_ids", "weights", "params"]
+        op.bind([torch.from_numpy(W.to_slices(src)).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(packed).cuda(), params], [out])
+    else:
+        f16 = td == np.float16
+        mt = M.FLOAT16 if f16 else M.FLOAT32
+        src = rng.uniform(-1, 1, size=(rows, k)).astype(td).astype(np.float32)
+        scale = (np.abs(rng.normal(0.0, 1.0, size=(n, batch, 1))) / 128.0 + 1e-3).astype(td).astype(np.float32)
+        st = M.scale_to_tensor_batched(scale, mt)
+        out = torch.full((ns, rows, 4), 7.0, dtype=torch.float16 if f16 else torch.float32, device="cuda")
+        op = M.fc_create(M.PRECISION_F32_F16 if f16 else M.PRECISION_F32, mt, mt, n, k, desc, scale_shape=(n, 1),
+                         max_tokens=rows, weights_batch=batch, src_end_ch_index=1, dst_end_ch_index=3)
+        assert op.src_names == ["src_tensor", "batch_ids", "weights", "weights_scale", "params"]
+        op.bind([torch.from_numpy(W.to_slices(src).astype(td)).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(packed).cuda(),
+                 torch.from_numpy(st.view(td) if f16 else st).cuda(), params], [out])
+    op.set_shape(1, rows, 1)
+    print("runtime bounds x batched weights", bits, td.__name__, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert op.kernel_name == ("fc_int8_math_kernel" if int8_math else "fc_generic_kernel"), op.kernel_name
+    got = out.cpu().numpy()
+    if int8_math:
+        assert np.all(got[ns_end:] == -5)
+        a = src.astype(np.int64).copy()
+        a[:, ks_end * 4:] = 0
+        for y in range(rows):
+            ref = (w[:, ids[y], 0, :].astype(np.int64) @ a[y])[:ns_end * 4]
+            assert np.array_equal(W.from_slices(got[:ns_end, y:y + 1], min(n, ns_end * 4))[0], ref[:min(n, ns_end * 4)])
+        return
+    got = got.astype(np.float32)
+    assert np.all(got[ns_end:] == 7.0)
+    conv = (lambda a: o.f32_to_f16_bits(np.asarray(a, np.float32))) if f16 else (lambda a: np.asarray(a, np.float32))
+    prec = o.PREC_F32F16 if f16 else o.PREC_F32
+    pack_o = o.int8_as_uint8 if bits == 8 else o.int8_as_uint4
+    for y in range(rows):
+        e = int(ids[y])
+        sc = np.zeros(ns * 4, np.float32); sc[:n] = scale[:, e, 0]
+        ref = o.fc_kernel_runtime_check(conv(o.to_slices(src[y:y + 1])), pack_o(w[:, e, 0, :], o.LAYOUT_I4O4, ns), 1, k, n, prec, bits,
+                                        o.SCALE_LINEAR, conv(sc), None, None, 1, src_end_ch=src_end, dst_end_ch=dst_end)
+        ref = o.f16_bits_to_f32(ref) if f16 else ref
+        sub = dict(tensor_dtype=np.float16 if f16 else np.float32, k=k)
+        check_fp(W.from_slices(got[:ns_end, y:y + 1], ns_end * 4), W.from_slices(ref[:ns_end], ns_end * 4).astype(np.float64), sub,
+                 "bounded kernel restatement, row %d" % y)

@@ -153,13 +153,16 @@ def test_graph_replays_match_eager(decode_layout):
 
 
 @pytest.mark.timeout(900)
-def test_stack_chain_18_layers_decode():
+@pytest.mark.parametrize("decode_layout", [False, True])
+def test_stack_chain_18_layers_decode(decode_layout):
     """The whole 18-layer stack at one token with the values flowing through it: every FC has its
     own weights (seed layer * 7 + index) and reads the re-normalised output of the FC before it in
     the layer's graph (q, k, v read the layer input; o reads q's output; gate and up read o's; down
     reads gate's; the next layer reads down's), N(0,1) after re-normalisation as the synthetic
-    inputs are.  Each FC goes through the C-ABI on the kernel the bench uses and is held to the
-    FullyConnected bar against float64 arithmetic over its dequantised weights."""
+    inputs are.  Each FC goes through the C-ABI on the kernel the bench uses (`decode_layout`: the weights
+    as a decode graph's ops ask for them, the bench's default for the decode step; else the one layout
+    that serves both graphs) and is held to the FullyConnected bar against float64 arithmetic over its
+    dequantised weights."""
     import torch
     rng = np.random.default_rng(1234)
     x = rng.standard_normal(2048).astype(np.float16).astype(np.float32)
@@ -183,10 +186,11 @@ def test_stack_chain_18_layers_decode():
             case = W.make_fc_case(seed=layer * 7 + idx, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16,
                                   groups=k // 32)
             case["act"] = src[None, :].astype(np.float32)
-            dev = W.FcDevice(case)
+            dev = W.FcDevice(case, decode_layout=decode_layout)
             dev.run()
             got = dev.result()
-            assert dev.op.kernel_name == "fc_w4_strip_kernel", dev.op.kernel_name
+            want = "fc_w4_rows_kernel" if decode_layout and n < 8192 else "fc_w4_strip_kernel"
+            assert dev.op.kernel_name == want, dev.op.kernel_name
             worst = max(worst, check_fp(got, reference(case), case, "layer %d %s" % (layer, name)))
             outs[name] = renorm(got[0])
             del dev

@@ -52,6 +52,27 @@ def test_no_alloc_decode_layout():
     run_pair(three, False, output_group=8)
 
 
+def test_no_alloc_where_op_launch_takes_another_kernel(oracle):
+    """2 and 4 tokens on a per-channel layer of 8192 channels: mldhip_op_launch runs the matrix-core
+    GEMV there, this entry point the streaming one, so the result is held to the oracle, not to the op."""
+    import torch
+    from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, textbook
+    for m in (2, 4):
+        case = W.make_fc_case(seed=76 + m, m=m, k=1024, n=8192, weight_bits=4, tensor_dtype=np.float16, groups=1, with_bias=True)
+        dev = W.FcDevice(case)
+        dev.run()
+        assert dev.op.kernel_name == "fc_w4_mfma_stream_kernel", dev.op.kernel_name
+        out = torch.zeros_like(dev.out)
+        print("no-alloc", m, "tokens, 8192 channels", flush=True)
+        M.fc_int4_decode_noalloc(dev.act, dev.weights, dev.scale, dev.bias, out, case["n"], case["k"], 1,
+                                 dev.desc.output_group_size, m, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        got = W.from_slices(out.cpu().numpy().astype(np.float32), case["n"])
+        exact = textbook(case)
+        check_fp(got, exact, case, "no-alloc")
+        check_as_accurate_as(got, oracle_fc(oracle, case), exact, case, "no-alloc")
+
+
 def test_no_alloc_rejects():
     import torch
     t = torch.zeros(4096, dtype=torch.float16, device="cuda")
