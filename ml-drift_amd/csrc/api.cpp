@@ -797,8 +797,13 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
     } else {
       FcArgs a;
       if (int rc = BuildFcArgs(op, &a)) return rc;
-      // runtime channel bounds are served by the unspecialised kernel
-      const bool force_generic = GetTuning().force_generic > 0 || a.params != nullptr;
+      // Runtime channel bounds at 1..4 tokens run on the streaming GEMVs (which stop their K loop at the
+      // bound and skip the dst strips beyond it); ringed weights, packed groups off the matrix cores and
+      // bounds at more tokens on the unspecialised kernel.
+      const bool bounded = a.params != nullptr;
+      const bool bounded_stream = bounded && a.packed_params_offset < 0 && a.ring_i_index < 0 && a.ring_o_index < 0 &&
+                                  (FcW4StreamSupported(a) || FcW8StreamSupported(a));
+      const bool force_generic = GetTuning().force_generic > 0 || (bounded && !bounded_stream);
       // packed groups: the matrix-core GEMM with one launch plane per matrix where it serves the shape
       if (GetTuning().force_generic <= 0 && FcW4MfmaPackedSupported(a)) {
         e = LaunchFcW4Mfma(a, stream, &op->last_kernel);

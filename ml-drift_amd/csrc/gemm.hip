@@ -763,73 +763,187 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     load_step(t_begin + u, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
     __builtin_amdgcn_sched_barrier(0);
   }
-  for (int tt = 0; tt < per_wave; tt += U) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int t = t_begin + tt + u;
-      // consume stage u
-      const wblk_t wr[2] = {rw[u][0], rw[u][1]};
-      const u32x2 scr = rsc[u & ~1];
-      u32x4 blk = {0u, 0u, 0u, 0u}, blk8 = blk;
-      if constexpr (WB == 4) {
-        blk = u32x4{wr[0][0], wr[0][1], wr[1][0], wr[1][1]};
-        blk8 = u32x4{blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
-      }
-      const half2_t sc01 = AsHalf2(scr[0]), sc23 = AsHalf2(scr[1]);
-      half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
-      if (ZP) {
-        zp01 = AsHalf2(rzp[u & ~1][0]);
-        zp23 = AsHalf2(rzp[u & ~1][1]);
-      }
-      if (PAIR) {
-        // The two 16-byte loads of a token pair hold {token 2j, token 2j+1} of K-slice rows 2q
-        // and 2q+1; exchanging the inner halves makes each of them one token's operand.
-#pragma unroll
-        for (int i = 0; i < NX; ++i) {
-          SwapRegisters(rxp[u][i][0], rxp[u][i][1]);
+  if constexpr (FM == 1) {
+  // 32-token tiles: four weight words per MFMA keep the vector ALU busier than the matrix pipe
+  // whatever the order (two waves per SIMD fill each other's gaps), and the plain loop is the
+  // faster one there.
+    for (int tt = 0; tt < per_wave; tt += U) {
+  #pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = t_begin + tt + u;
+        // consume stage u
+        const wblk_t wr[2] = {rw[u][0], rw[u][1]};
+        const u32x2 scr = rsc[u & ~1];
+        u32x4 blk = {0u, 0u, 0u, 0u}, blk8 = blk;
+        if constexpr (WB == 4) {
+          blk = u32x4{wr[0][0], wr[0][1], wr[1][0], wr[1][1]};
+          blk8 = u32x4{blk[0] >> 8, blk[1] >> 8, blk[2] >> 8, blk[3] >> 8};
         }
-      }
-#pragma unroll
-      for (int t4 = 0; t4 < 4; ++t4) {
-        const half2_t sp = (t4 & 2) ? sc23 : sc01;
-        const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
-        const half2_t off = WB == 8 ? off_w8 : ((t4 & 1) ? off_hi : off_lo);
-        // zero point: (u - shift) * s - zp * s in one fused step, so that a fractional zero point
-        // costs one extra rounding of zp * s and not a rounding of shift + zp to an integer
-        half2_t mzs = {(_Float16)0.0f, (_Float16)0.0f};
+        const half2_t sc01 = AsHalf2(scr[0]), sc23 = AsHalf2(scr[1]);
+        half2_t zp01 = {(_Float16)0.0f, (_Float16)0.0f}, zp23 = zp01;
         if (ZP) {
-          const half2_t zq = (t4 & 2) ? zp23 : zp01;
-          mzs = -(((t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0)) * s2);
+          zp01 = AsHalf2(rzp[u & ~1][0]);
+          zp23 = AsHalf2(rzp[u & ~1][1]);
         }
-        u32x4 aop;
-#pragma unroll
-        for (int wd = 0; wd < 4; ++wd) {
-          uint32_t bits;
-          if constexpr (WB == 8) {
-            // bytes t4 of the words of input channels 2*wd, 2*wd + 1 -> the low bytes of two halfs
-            const uint32_t sel = 0x0c000c00u | (uint32_t)t4 | ((uint32_t)(4 + t4) << 16);
-            bits = __builtin_amdgcn_perm(wr[wd >> 1][2 * (wd & 1) + 1], wr[wd >> 1][2 * (wd & 1)], sel) | magic_lo;
-          } else {
-            const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
-            bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
+        if (PAIR) {
+          // The two 16-byte loads of a token pair hold {token 2j, token 2j+1} of K-slice rows 2q
+          // and 2q+1; exchanging the inner halves makes each of them one token's operand.
+  #pragma unroll
+          for (int i = 0; i < NX; ++i) {
+            SwapRegisters(rxp[u][i][0], rxp[u][i][1]);
           }
-          const half2_t centred = AsHalf2(bits) + off;  // exact: u - shift
-          aop[wd] = AsU32(ZP ? __builtin_elementwise_fma(centred, s2, mzs) : centred * s2);
         }
-#pragma unroll
-        for (int fm = 0; fm < FM; ++fm) {
-          const u32x4 bop = PAIR ? rxp[u][fm / 2][fm & 1]
-                                 : u32x4{rx[u][PAIR ? 0 : fm][0][0], rx[u][PAIR ? 0 : fm][0][1], rx[u][PAIR ? 0 : fm][1][0],
-                                         rx[u][PAIR ? 0 : fm][1][1]};
-          acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
-                                                               __builtin_bit_cast(half8_t, bop), acc[t4][fm], 0, 0, 0);
+  #pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) {
+          const half2_t sp = (t4 & 2) ? sc23 : sc01;
+          const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
+          const half2_t off = WB == 8 ? off_w8 : ((t4 & 1) ? off_hi : off_lo);
+          // zero point: (u - shift) * s - zp * s in one fused step, so that a fractional zero point
+          // costs one extra rounding of zp * s and not a rounding of shift + zp to an integer
+          half2_t mzs = {(_Float16)0.0f, (_Float16)0.0f};
+          if (ZP) {
+            const half2_t zq = (t4 & 2) ? zp23 : zp01;
+            mzs = -(((t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0)) * s2);
+          }
+          u32x4 aop;
+  #pragma unroll
+          for (int wd = 0; wd < 4; ++wd) {
+            uint32_t bits;
+            if constexpr (WB == 8) {
+              // bytes t4 of the words of input channels 2*wd, 2*wd + 1 -> the low bytes of two halfs
+              const uint32_t sel = 0x0c000c00u | (uint32_t)t4 | ((uint32_t)(4 + t4) << 16);
+              bits = __builtin_amdgcn_perm(wr[wd >> 1][2 * (wd & 1) + 1], wr[wd >> 1][2 * (wd & 1)], sel) | magic_lo;
+            } else {
+              const uint32_t x = (t4 & 2) ? blk8[wd] : blk[wd];
+              bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
+            }
+            const half2_t centred = AsHalf2(bits) + off;  // exact: u - shift
+            aop[wd] = AsU32(ZP ? __builtin_elementwise_fma(centred, s2, mzs) : centred * s2);
+          }
+  #pragma unroll
+          for (int fm = 0; fm < FM; ++fm) {
+            const u32x4 bop = PAIR ? rxp[u][fm / 2][fm & 1]
+                                   : u32x4{rx[u][PAIR ? 0 : fm][0][0], rx[u][PAIR ? 0 : fm][0][1], rx[u][PAIR ? 0 : fm][1][0],
+                                           rx[u][PAIR ? 0 : fm][1][1]};
+            acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
+                                                                 __builtin_bit_cast(half8_t, bop), acc[t4][fm], 0, 0, 0);
+          }
         }
+        // refill stage u with step t + U; the fences keep the loads of a stage together and in
+        // program order, so that waiting for one stage leaves the younger ones in flight
+        __builtin_amdgcn_sched_barrier(0);
+        load_step(t + U, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      // refill stage u with step t + U; the fences keep the loads of a stage together and in
-      // program order, so that waiting for one stage leaves the younger ones in flight
-      __builtin_amdgcn_sched_barrier(0);
-      load_step(t + U, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
-      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    // The loop is software-pipelined by one weight operand: while the FM MFMAs of output-channel phase
+    // t4 run, the vector ALU dequantizes the operand of phase t4 + 1 (at t4 = 3: phase 0 of the next
+    // stage), 4 / FM words behind every MFMA.  A wave issues in order, and an MFMA that waits for the
+    // matrix pipe holds back whatever follows it, so a run of MFMAs followed by a run of vector
+    // instructions serialises the two; placed between the MFMAs, the vector instructions issue in the
+    // 32 cycles each MFMA occupies the pipe.  The scheduling groups at the end of a step ask for that order.
+    struct Stage {
+      u32x4 blk, blk8;   // WB == 4: the stage's 32 weights, and the same shifted by 8 bits
+      wblk_t w0, w1;     // WB == 8: the two blocks
+      half2_t sc01, sc23, zp01, zp23;
+    };
+    auto open_stage = [&](int u) {
+      Stage st;
+      st.w0 = rw[u][0];
+      st.w1 = rw[u][1];
+      st.blk = st.blk8 = u32x4{0u, 0u, 0u, 0u};
+      if constexpr (WB == 4) {
+        st.blk = u32x4{rw[u][0][0], rw[u][0][1], rw[u][1][0], rw[u][1][1]};
+        st.blk8 = u32x4{st.blk[0] >> 8, st.blk[1] >> 8, st.blk[2] >> 8, st.blk[3] >> 8};
+      }
+      const u32x2 scr = rsc[u & ~1];
+      st.sc01 = AsHalf2(scr[0]);
+      st.sc23 = AsHalf2(scr[1]);
+      st.zp01 = st.zp23 = half2_t{(_Float16)0.0f, (_Float16)0.0f};
+      if (ZP) {
+        st.zp01 = AsHalf2(rzp[u & ~1][0]);
+        st.zp23 = AsHalf2(rzp[u & ~1][1]);
+      }
+      return st;
+    };
+    // word wd (input channels 2 wd, 2 wd + 1 of the step's 8) of the operand of phase t4
+    auto dequant_word = [&](const Stage& st, int t4, int wd) -> uint32_t {
+      const half2_t sp = (t4 & 2) ? st.sc23 : st.sc01;
+      const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sp, sp, 1, 1) : __builtin_shufflevector(sp, sp, 0, 0);
+      const half2_t off = WB == 8 ? off_w8 : ((t4 & 1) ? off_hi : off_lo);
+      // zero point: (u - shift) * s - zp * s in one fused step, so that a fractional zero point
+      // costs one extra rounding of zp * s and not a rounding of shift + zp to an integer
+      half2_t mzs = {(_Float16)0.0f, (_Float16)0.0f};
+      if (ZP) {
+        const half2_t zq = (t4 & 2) ? st.zp23 : st.zp01;
+        mzs = -(((t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0)) * s2);
+      }
+      uint32_t bits;
+      if constexpr (WB == 8) {
+        // bytes t4 of the words of input channels 2*wd, 2*wd + 1 -> the low bytes of two halfs
+        const uint32_t sel = 0x0c000c00u | (uint32_t)t4 | ((uint32_t)(4 + t4) << 16);
+        const wblk_t& wr = (wd >> 1) ? st.w1 : st.w0;
+        bits = __builtin_amdgcn_perm(wr[2 * (wd & 1) + 1], wr[2 * (wd & 1)], sel) | magic_lo;
+      } else {
+        const uint32_t x = (t4 & 2) ? st.blk8[wd] : st.blk[wd];
+        bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
+      }
+      const half2_t centred = AsHalf2(bits) + off;  // exact: u - shift
+      return AsU32(ZP ? __builtin_elementwise_fma(centred, s2, mzs) : centred * s2);
+    };
+    // vector instructions per MFMA of a step: 13-14 per phase (3 per word, the scale broadcast, the shifts of a new stage)
+    constexpr int kValuPerMfma = FM >= 4 ? 4 : (FM == 2 ? 8 : 16);
+    Stage cur = open_stage(0);
+    u32x4 aop;
+  #pragma unroll
+    for (int wd = 0; wd < 4; ++wd) aop[wd] = dequant_word(cur, 0, wd);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int tt = 0; tt < per_wave; tt += U) {
+  #pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int t = t_begin + tt + u;
+        if (PAIR) {
+          // The two 16-byte loads of a token pair hold {token 2j, token 2j+1} of K-slice rows 2q
+          // and 2q+1; exchanging the inner halves makes each of them one token's operand.
+  #pragma unroll
+          for (int i = 0; i < NX; ++i) {
+            SwapRegisters(rxp[u][i][0], rxp[u][i][1]);
+          }
+        }
+        Stage nxt = cur;
+  #pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) {
+          // the operand that follows this one: the next phase of this stage, or phase 0 of the next
+          // stage (after the last step: of a stage that was fetched beyond the range and holds zeros)
+          if (t4 == 3) nxt = open_stage((u + 1) % U);
+          const int t4n = (t4 + 1) & 3;
+          u32x4 anext;
+  #pragma unroll
+          for (int fm = 0; fm < FM; ++fm) {
+            const u32x4 bop = PAIR ? rxp[u][fm / 2][fm & 1]
+                                   : u32x4{rx[u][PAIR ? 0 : fm][0][0], rx[u][PAIR ? 0 : fm][0][1], rx[u][PAIR ? 0 : fm][1][0],
+                                           rx[u][PAIR ? 0 : fm][1][1]};
+            acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, aop),
+                                                                 __builtin_bit_cast(half8_t, bop), acc[t4][fm], 0, 0, 0);
+          }
+  #pragma unroll
+          for (int wd = 0; wd < 4; ++wd) anext[wd] = dequant_word(nxt, t4n, wd);
+          aop = anext;
+        }
+        cur = nxt;
+        // the order of the step's instructions: one MFMA, then its share of the vector instructions
+  #pragma unroll
+        for (int i = 0; i < 4 * FM; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+        }
+        // refill stage u with step t + U; the fences keep the loads of a stage together and in
+        // program order, so that waiting for one stage leaves the younger ones in flight
+        __builtin_amdgcn_sched_barrier(0);
+        load_step(t + U, u % 2 == 1, rw[u], rsc[u & ~1], rzp[u & ~1], rx[u], rxp[u]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 

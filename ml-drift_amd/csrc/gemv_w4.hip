@@ -86,6 +86,12 @@ struct StreamParams {
   // holds weights_batch matrices one after the other, scales are [group][weights_batch][Ns][4].
   const int32_t* batch_ids;
   int rows, src_rows, weights_batch;
+  // Runtime channel bounds (the streaming kernel only): int32 values in device memory, read at the top
+  // of the kernel; an index < 0 = not set; null = no bounds.  The K loop stops after the bounded
+  // K-slices (not with group-wise scales, whose loop runs over all groups in the reference too), dst
+  // slices beyond the bound are not written.
+  const int32_t* rt_params;
+  int src_end_idx, dst_end_idx, k_channels;
 };
 
 __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const __half* bias, size_t bi) {
@@ -100,9 +106,10 @@ __device__ __forceinline__ void StoreHalf(__half* dst, size_t i, float r, const 
 // act_stride / act_tok0: tokens per K-slice row of the activation tensor and the first token of
 // this launch row in it (M and 0 unless the launch has batched weights).
 // wcol: the lane's column of the packed weights (K-slice row 0), rstride: uint4 per K-slice row.
+// ks_live: K-slices that count (p.ks, or fewer under a runtime bound): activations from there on read as zero.
 template <int M>
 __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* wcol, int rstride, int c,
-                                          u32x4 w[8], u32x2 a[8][M], int act_stride = M, int act_tok0 = 0) {
+                                          u32x4 w[8], u32x2 a[8][M], int ks_live, int act_stride = M, int act_tok0 = 0) {
   const int ks0 = c * 8;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -112,7 +119,7 @@ __device__ __forceinline__ void LoadChunk(const StreamParams& p, const u32x4* wc
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       const u32x2 v = *reinterpret_cast<const u32x2*>(p.act + ((size_t)ksc * act_stride + act_tok0 + m) * 4);
-      a[j][m] = u32x2{ks < p.ks ? v[0] : 0u, ks < p.ks ? v[1] : 0u};
+      a[j][m] = u32x2{ks < ks_live ? v[0] : 0u, ks < ks_live ? v[1] : 0u};
     }
   }
 }
@@ -204,7 +211,14 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   const int rstride = sg.gu4;
   const int ky = blockIdx.y;
   const int c_begin = ky * p.chunks_per_split;
-  const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
+  // runtime channel bounds: K-slices that count, dst slices that are written
+  int ks_live = p.ks, ns_live = sg.ns;
+  if (p.rt_params != nullptr) {
+    if (!GROUPED && p.src_end_idx >= 0) ks_live = SrcEndSlices(p.rt_params[p.src_end_idx], p.k_channels, p.ks);
+    if (p.dst_end_idx >= 0) ns_live = DstEndSlice(p.rt_params[p.dst_end_idx], sg.ns);
+    if (strip * (STRIP / 4) >= ns_live) return;  // (the whole work-group: no barrier is left waiting)
+  }
+  const int c_end = min(c_begin + p.chunks_per_split, p.rt_params != nullptr ? (ks_live + 7) / 8 : p.chunks);
 
   float acc[M][8];
 #pragma unroll
@@ -228,13 +242,13 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   if (c < c_end) {
     u32x4 w[8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, wcol, rstride, c, w, a, act_stride, act_tok0);
+    LoadChunk<M>(p, wcol, rstride, c, w, a, ks_live, act_stride, act_tok0);
     while (true) {
       const int cn = c + ROWS;
       const bool more = cn < c_end;
       u32x4 wn[8];
       u32x2 an[8][M];
-      if (more) LoadChunk<M>(p, wcol, rstride, cn, wn, an, act_stride, act_tok0);
+      if (more) LoadChunk<M>(p, wcol, rstride, cn, wn, an, ks_live, act_stride, act_tok0);
       u32x4 sv;
       if (GROUPED) {
         int g = c / p.group_chunks;
@@ -303,7 +317,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_stream_kernel(StreamParams p
   for (int idx = tid; idx < M * STRIP; idx += THREADS) {
     const int m = idx / STRIP, ol = idx % STRIP;
     const int n = n0 + ol;
-    if (n >= sg.n_pad) continue;
+    if (n >= ns_live * 4) continue;
     float v = 0.0f;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
@@ -329,6 +343,7 @@ __global__ __launch_bounds__(256) void fc_w4_reduce_kernel(StreamParams p, int n
   if (p.segments > 1 && nt >= p.seg[1].n_off) si = (p.segments > 2 && nt >= p.seg[2].n_off) ? 2 : 1;
   const StreamSegment& sg = p.seg[si];
   const int n = nt - sg.n_off;
+  if (p.rt_params != nullptr && p.dst_end_idx >= 0 && (n >> 2) >= DstEndSlice(p.rt_params[p.dst_end_idx], sg.ns)) return;
   // The parts are fetched eight at a time before any is added (a part past the last re-reads the
   // last one and is dropped by a select), so that their latencies overlap; added in split order.
   const float scale = GROUPED ? 1.0f : __half2float(sg.scale[n]);
@@ -398,7 +413,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_gated_stream_kernel(StreamPa
   for (int c = row; c < p.chunks; c += ROWS) {
     u32x4 w[2][8];
     u32x2 a[8][M];
-    LoadChunk<M>(p, p.seg[0].weights + wcol_off, rstride, c, w[0], a);
+    LoadChunk<M>(p, p.seg[0].weights + wcol_off, rstride, c, w[0], a, p.ks);
     {
       const int ks0 = c * 8;
 #pragma unroll
@@ -845,6 +860,7 @@ hipError_t LaunchStripL(const StripParams& p, int waves, bool grouped, dim3 grid
 // groups of the same size (16, 8 or 4 slices), K a multiple of 32 channels (whole chunks).
 bool StripKernelServes(const FcArgs* args, int count) {
   if (GetTuning().gemv_fast == 0) return false;
+  if (args[0].params != nullptr) return false;  // runtime channel bounds: the streaming kernel
   if (args[0].m != 1) return false;
   if (DivUp(args[0].k, 4) % 8 != 0 || args[0].k % 4 != 0) return false;
   const int group = EffectiveGroup(args[0].group, DivUp(args[0].n, 4));
@@ -1082,6 +1098,7 @@ hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_
 // of 2 slices, scale groups of a power-of-two number of K-slices.
 bool RowsKernelServes(const FcArgs* args, int count) {
   if (GetTuning().gemv_fast == 0) return false;
+  if (args[0].params != nullptr) return false;  // runtime channel bounds: the streaming kernel
   if (args[0].m != 1 || args[0].batch_ids != nullptr || args[0].k % 4 != 0) return false;
   for (int i = 0; i < count; ++i) {
     const int ns = DivUp(args[i].n, 4);
@@ -1137,6 +1154,7 @@ hipError_t LaunchRows(const StreamParams& p, const FcArgs* args, int count, bool
 
 bool FcW4StreamSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
+  if (a.params != nullptr && (a.packed_params_offset >= 0 || a.ring_i_index >= 0 || a.ring_o_index >= 0)) return false;
   if (a.m < 1 || a.m > kGemvMaxTokens) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   const int ks = DivUp(a.k, 4), ns = DivUp(a.n, 4);
@@ -1194,6 +1212,11 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   p.rows = a.rows;
   p.src_rows = a.src_rows;
   p.weights_batch = a.weights_batch;
+  p.rt_params = a.params;
+  p.src_end_idx = a.src_end_ch_index;
+  p.dst_end_idx = a.dst_end_ch_index;
+  p.k_channels = a.k;
+  if (a.params != nullptr && count != 1) return hipErrorInvalidValue;  // bounded launches are single launches
   if (a.batch_ids) {
     // One dst row per blockIdx.z, K inside the work-group.  128-byte row segments when the rows
     // together still give most CUs a work-group, else 64-byte ones.
@@ -1334,6 +1357,11 @@ hipError_t LaunchFcW4Gated(const FcArgs& gate, const FcArgs& up, int activation,
     sg.strip_end = 0;
   }
   p.seg[2] = p.seg[0];
+  p.batch_ids = nullptr;
+  p.rows = p.src_rows = p.weights_batch = 1;
+  p.rt_params = nullptr;
+  p.src_end_idx = p.dst_end_idx = -1;
+  p.k_channels = gate.k;
   if (kernel_name) *kernel_name = "fc_w4_gated_stream_kernel";
   // 128-byte row segments, 8 waves: 64 rows of chunks per pass (one pass covers K = 2048); the
   // 16-wave shape would spill with the two sets of accumulators

@@ -192,6 +192,7 @@ __global__ __launch_bounds__(kMsWaves * 64) void fc_w4_mfma_stream_kernel(MsPara
 
 bool FcW4MfmaStreamSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
+  if (a.params != nullptr || a.batch_ids != nullptr) return false;  // runtime channel bounds, batched weights: the other kernels
   if (a.scale_kind != kScaleLinear) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
   if (a.m < 1 || a.m > 16) return false;

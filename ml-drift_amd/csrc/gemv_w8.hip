@@ -41,6 +41,10 @@ struct W8Params {
   // after the other, scales are [group][weights_batch][Ns][4].
   const int32_t* batch_ids;
   int rows, src_rows, weights_batch;
+  // Runtime channel bounds (the streaming kernel only): int32 values in device memory, read at the top
+  // of the kernel; an index < 0 = not set; null = no bounds.
+  const int32_t* rt_params;
+  int src_end_idx, dst_end_idx, k_channels;
 };
 
 __device__ __forceinline__ void Load4(const float* p, size_t i, float v[4]) {
@@ -116,6 +120,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
   const int row = wave * RPW + lane / LPR;
   const int slice_raw = blockIdx.x * LPR + col;
   const int slice = slice_raw < p.ns ? slice_raw : p.ns - 1;  // clamp: loads stay in range, result unused
+  // runtime channel bounds: K-slices that count (the loop over scale groups runs over all of them in
+  // the reference), dst slices that are written
+  int ks_live = p.ks, ns_live = p.ns, chunks_live = p.chunks;
+  if (p.rt_params != nullptr) {
+    if (!p.grouped && p.src_end_idx >= 0) ks_live = SrcEndSlices(p.rt_params[p.src_end_idx], p.k_channels, p.ks);
+    if (p.dst_end_idx >= 0) ns_live = DstEndSlice(p.rt_params[p.dst_end_idx], p.ns);
+    if ((int)blockIdx.x * LPR >= ns_live) return;  // (the whole work-group: no barrier is left waiting)
+    chunks_live = (ks_live + 7) / 8;
+  }
 
   float acc[M][4];
 #pragma unroll
@@ -148,12 +161,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
         float v[4];
         Load4(act, ((size_t)min(ks, p.ks - 1) * act_stride + act_tok0 + m) * 4, v);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[j][m][i] = ks < p.ks ? v[i] : 0.0f;
+        for (int i = 0; i < 4; ++i) a[j][m][i] = ks < ks_live ? v[i] : 0.0f;
       }
     }
   };
 
-  for (int c = row; c < p.chunks; c += ROWS) {
+  for (int c = row; c < chunks_live; c += ROWS) {
     u32x4 w[8];
     float a[8][M][4];
     load_weights(c, w);
@@ -224,7 +237,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_stream_kernel(W8Params p) {
   for (int idx = tid; idx < M * STRIP; idx += THREADS) {
     const int m = idx / STRIP, ol = idx % STRIP;
     const int n = n0 + ol;
-    if (n >= p.ns * 4) continue;
+    if (n >= ns_live * 4) continue;
     float v = 0.0f;
 #pragma unroll
     for (int q = 0; q < PARTS; ++q) v += red2[q][m][ol];
@@ -396,6 +409,7 @@ hipError_t LaunchT(const W8Params& p, int lpr, int waves, hipStream_t stream) {
 
 bool FcW8StreamSupported(const FcArgs& a) {
   if (a.weight_bits != 8 || a.act_f16 != a.dst_f16) return false;
+  if (a.params != nullptr && (a.packed_params_offset >= 0 || a.ring_i_index >= 0 || a.ring_o_index >= 0)) return false;
   if (EffectiveGroup(a.group, DivUp(a.n, 4)) != DivUp(a.n, 4)) return false;  // one output group only
   if (a.m < 1 || a.m > kGemvMaxTokens) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
@@ -412,6 +426,7 @@ bool FcW8StreamSupported(const FcArgs& a) {
 // power-of-two number of K-slices.
 bool FcW8RowsSupported(const FcArgs& a) {
   if (a.weight_bits != 8 || a.act_f16 != a.dst_f16 || a.m != 1 || a.batch_ids != nullptr) return false;
+  if (a.params != nullptr) return false;  // runtime channel bounds: the streaming kernel
   const int ns = DivUp(a.n, 4), ks = DivUp(a.k, 4);
   if (ns < 2 || EffectiveGroup(a.group, ns) != 1) return false;
   if (a.has_zero_point && a.zero_point == nullptr) return false;  // a scalar zero point: generic kernel
@@ -443,6 +458,9 @@ hipError_t LaunchFcW8Rows(const FcArgs& a, hipStream_t stream, const char** kern
     for (int gs = p.ks / a.groups; gs > 1; gs >>= 1) ++p.group_chunks;
   p.batch_ids = nullptr;
   p.rows = p.src_rows = p.weights_batch = 1;
+  p.rt_params = nullptr;
+  p.src_end_idx = p.dst_end_idx = -1;
+  p.k_channels = a.k;
   // eight rows per thread where K allows: all of a thread's loads are in flight at once
   int waves = 1;
   while (waves < 8 && waves * 64 * 8 < p.ks) waves *= 2;
@@ -470,6 +488,10 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
   p.rows = a.rows;
   p.src_rows = a.src_rows;
   p.weights_batch = a.weights_batch;
+  p.rt_params = a.params;
+  p.src_end_idx = a.src_end_ch_index;
+  p.dst_end_idx = a.dst_end_ch_index;
+  p.k_channels = a.k;
   // 128-byte row segments (8 slices) when that still gives a work-group to half the CUs, else
   // 64-byte ones; small work-groups when K is covered by 64 / 128 rows of chunks
   const int lpr = (long)DivUp(p.ns, 8) * (a.batch_ids ? a.rows : 1) >= 128 ? 8 : 4;

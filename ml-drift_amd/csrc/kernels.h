@@ -40,6 +40,20 @@ inline int NativeGroupFor(int o) {
 
 enum ScaleKind { kScaleScalar = 0, kScaleLinear = 1, kScaleBlock = 2 };
 
+// Runtime channel bounds (ConvRuntimeCheckDesc, common/task/gpu_operation.h:384-412) from the values a
+// kernel has read out of "params": K-slices the loop covers, src_end_slices = (min(end_ch, channels) +
+// 3) / 4 (fully_connected.cc:750-755), and dst slices that are written, min(round_up(end_ch, 32) / 4,
+// slices) (GetRuntimeEndSlice, common/task/gpu_operation.cc:1832-1836; fully_connected_util.cc:231-243).
+__host__ __device__ inline int SrcEndSlices(int end_ch, int k_channels, int ks) {
+  const int c = end_ch < k_channels ? end_ch : k_channels;
+  const int s = (c + 3) / 4;
+  return s < 0 ? 0 : (s > ks ? ks : s);
+}
+__host__ __device__ inline int DstEndSlice(int end_ch, int ns) {
+  const int s = ((end_ch + 31) / 32) * 32 / 4;
+  return s < 0 ? 0 : (s > ns ? ns : s);
+}
+
 // One FullyConnected launch.  Tensors are slice-major: act [Ks][m][4], dst [Ns][m][4].
 struct FcArgs {
   const void* act = nullptr;

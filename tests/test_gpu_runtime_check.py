@@ -1,7 +1,9 @@
 """GPU parity of the FullyConnected with runtime channel bounds (ConvRuntimeCheckDesc: src_end_ch /
 dst_end_ch read at launch from the int32 "params" object), through the C-ABI, against the oracle's
 restatement of the bounded kernel; the reference's own test shape and runtime channels
-(common/kernels/tests/fully_connected_test_util.cc:1260-1300) and larger layers."""
+(common/kernels/tests/fully_connected_test_util.cc:1260-1300) and larger layers.  Up to 4 tokens the
+bounded op runs on the streaming GEMVs (fc_w4_stream_kernel / fc_w8_stream_kernel), beyond on the
+unspecialised kernel; every case also runs with the unspecialised kernel forced."""
 import numpy as np
 import pytest
 
@@ -12,7 +14,30 @@ import workloads as W
 from test_gpu_fc import check_fp
 
 
+def streaming_kernel_for(case):
+    """The kernel a bounded op of this case takes (None: the unspecialised one)."""
+    ks, ns, groups = (case["k"] + 3) // 4, (case["n"] + 3) // 4, case["groups"]
+    if case["m"] > 4 or (groups > 1 and (ks % groups != 0 or (ks // groups) % 8 != 0)):
+        return None
+    if case["weight_bits"] == 8:
+        return "fc_w8_stream_kernel"
+    return "fc_w4_stream_kernel" if case["tensor_dtype"] == np.float16 and ns % 2 == 0 else None
+
+
 def run_bounded(oracle, case, src_end_ch, dst_end_ch, params_values=None):
+    got = run_bounded_once(oracle, case, src_end_ch, dst_end_ch, streaming_kernel_for(case) or "fc_generic_kernel")
+    if streaming_kernel_for(case):
+        with M.tuning(force_generic=1):
+            run_bounded_once(oracle, case, src_end_ch, dst_end_ch, "fc_generic_kernel")
+        if case["weight_bits"] == 4:
+            # the same op over the layouts the library asks for (output groups of 16 slices; of 2 for a decode op)
+            for layout in ("library", "decode"):
+                other = run_bounded_once(oracle, case, src_end_ch, dst_end_ch, None, layout=layout)
+                assert np.array_equal(other, got), layout
+    return got
+
+
+def run_bounded_once(oracle, case, src_end_ch, dst_end_ch, expect_kernel, layout="reference"):
     import torch
     o = oracle
     m, k, n, bits, groups = case["m"], case["k"], case["n"], case["weight_bits"], case["groups"]
@@ -21,7 +46,8 @@ def run_bounded(oracle, case, src_end_ch, dst_end_ch, params_values=None):
     tt = torch.float16 if f16 else torch.float32
     mt = M.FLOAT16 if f16 else M.FLOAT32
     ns = (n + 3) // 4
-    desc, packed = W.pack_fc_weights(case, reference_layout=True)
+    desc, packed_dev = W.pack_fc_weights(case, reference_layout=layout == "reference", decode_layout=layout == "decode")
+    packed = (o.int8_as_uint4 if bits == 4 else o.int8_as_uint8)(case["w"], o.LAYOUT_I4O4, ns)  # what the restatement reads
     # params: 4 int32 values as the reference's tests lay them out (src start, src end, dst start, dst end)
     params = np.full(4, -1, np.int32)
     kwargs = {}
@@ -32,7 +58,7 @@ def run_bounded(oracle, case, src_end_ch, dst_end_ch, params_values=None):
         params[3] = dst_end_ch
         kwargs["dst_end_ch_index"] = 3
     scale_dev = torch.from_numpy(M.scale_to_tensor(case["scale"], mt).view(td) if f16 else M.scale_to_tensor(case["scale"], mt)).cuda()
-    srcs = [torch.from_numpy(W.to_slices(case["act"]).astype(td)).cuda(), torch.from_numpy(packed).cuda(), scale_dev]
+    srcs = [torch.from_numpy(W.to_slices(case["act"]).astype(td)).cuda(), torch.from_numpy(packed_dev).cuda(), scale_dev]
     bias = None
     if case["bias"] is not None:
         bias = np.zeros(ns * 4, td)
@@ -45,10 +71,13 @@ def run_bounded(oracle, case, src_end_ch, dst_end_ch, params_values=None):
     assert op.src_names[-1] == "params"
     op.bind(srcs, [out])
     op.set_shape(1, 1, m)
-    print("runtime check", m, k, n, bits, groups, src_end_ch, dst_end_ch, flush=True)
+    print("runtime check", m, k, n, bits, groups, src_end_ch, dst_end_ch, layout, expect_kernel, flush=True)
     op.launch(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert op.kernel_name == "fc_generic_kernel", op.kernel_name
+    if expect_kernel is None:  # another layout of the same weights: the streaming kernel where it reads that layout
+        assert op.kernel_name in ("fc_w4_stream_kernel", "fc_generic_kernel"), op.kernel_name
+    else:
+        assert op.kernel_name == expect_kernel, op.kernel_name
     got = out.cpu().numpy().astype(np.float32)
     # oracle: the bounded kernel restatement over the reference's layout
     prec = o.PREC_F32F16 if f16 else o.PREC_F32
@@ -83,7 +112,9 @@ def test_reference_runtime_channel_cases(oracle, dtype, rc):
 
 @pytest.mark.parametrize("bits,m,k,n,groups,src_end,dst_end", [
     (4, 1, 4096, 2048, 1, 1000, 300), (4, 3, 2048, 1024, 64, 77, 1000), (8, 5, 1024, 516, 1, 0, 33),
-    (4, 1, 512, 256, 1, 512, 0), (4, 2, 256, 8192, 1, 129, 4097), (8, 1, 96, 64, 3, 5, 64)])
+    (4, 1, 512, 256, 1, 512, 0), (4, 2, 256, 8192, 1, 129, 4097), (8, 1, 96, 64, 3, 5, 64),
+    (4, 1, 16384, 2048, 1, 5000, 2048), (4, 4, 4096, 14336, 1, 4096, 14000), (8, 2, 4096, 4096, 1, 37, 4096),
+    (4, 1, 2048, 2048, 1, 0, 40), (8, 3, 2048, 1024, 64, 100, 500)])
 def test_runtime_bounds_sweep(oracle, bits, m, k, n, groups, src_end, dst_end):
     """Bounds inside the tensors, at and beyond their ends, zero, unaligned to 4 and to 32; group-wise
     scales ignore the source bound (the reference's group loop runs over all groups)."""
@@ -115,6 +146,7 @@ def test_runtime_bounds_with_batched_weights(oracle, bits, td):
     w = rng.integers(-lim, lim + 1, size=(n, batch, 1, k), dtype=np.int8)
     ids = np.array([2, 0, 3, 3, 1], np.int32)
     int8_math = td == np.int8
+    f16 = td == np.float16
     desc = M.fc_int8_weights_desc(n, k) if bits == 8 else M.fc_int4_weights_desc(n, k, reference=True)
     packed = (M.rearrange_int8_as_uint8 if bits == 8 else M.rearrange_int8_as_uint4)(w, desc)
     ks, ns = (k + 3) // 4, (n + 3) // 4
@@ -128,7 +160,6 @@ def test_runtime_bounds_with_batched_weights(oracle, bits, td):
         assert op.src_names == ["src_tensor", "batch_ids", "weights", "params"]
         op.bind([torch.from_numpy(W.to_slices(src)).cuda(), torch.from_numpy(ids).cuda(), torch.from_numpy(packed).cuda(), params], [out])
     else:
-        f16 = td == np.float16
         mt = M.FLOAT16 if f16 else M.FLOAT32
         src = rng.uniform(-1, 1, size=(rows, k)).astype(td).astype(np.float32)
         scale = (np.abs(rng.normal(0.0, 1.0, size=(n, batch, 1))) / 128.0 + 1e-3).astype(td).astype(np.float32)
@@ -143,7 +174,8 @@ def test_runtime_bounds_with_batched_weights(oracle, bits, td):
     print("runtime bounds x batched weights", bits, td.__name__, flush=True)
     op.launch(torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert op.kernel_name == ("fc_int8_math_kernel" if int8_math else "fc_generic_kernel"), op.kernel_name
+    want = "fc_int8_math_kernel" if int8_math else ("fc_w8_stream_kernel" if bits == 8 else ("fc_w4_stream_kernel" if f16 else "fc_generic_kernel"))
+    assert op.kernel_name == want, op.kernel_name
     got = out.cpu().numpy()
     if int8_math:
         assert np.all(got[ns_end:] == -5)
