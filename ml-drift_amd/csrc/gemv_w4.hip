@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "../../include/mldhip.h"
 #include "gated.h"
@@ -1384,6 +1385,7 @@ namespace {
 static __device__ __align__(256) float scratch[kNoAllocScratchFloats];
 constexpr int kMaxDevices = 64;
 float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;  // guards the first call on a device from several host threads
 }  // namespace
 
 hipError_t LaunchFcW4StreamNoAlloc(FcArgs a, hipStream_t stream, const char** kernel_name) {
@@ -1391,14 +1393,27 @@ hipError_t LaunchFcW4StreamNoAlloc(FcArgs a, hipStream_t stream, const char** ke
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return e;
   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
-  if (g_scratch_ptr[device] == nullptr) {  // first call on this device, which is current
-    float* ptr = nullptr;
-    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+  // the array that is used is the current device's: a stream of another device would launch there
+  // with this device's address
+  if (stream != nullptr) {
+    int stream_device = device;
+    e = hipStreamGetDevice(stream, &stream_device);
     if (e != hipSuccess) return e;
-    g_scratch_ptr[device] = ptr;
+    if (stream_device != device) return hipErrorInvalidDevice;
+  }
+  float* scratch_ptr = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {  // first call on this device, which is current
+      float* ptr = nullptr;
+      e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return e;
+      g_scratch_ptr[device] = ptr;
+    }
+    scratch_ptr = g_scratch_ptr[device];
   }
   // Nothing has to start at zero: a split launch writes every sum that its second kernel reads.
-  a.partial = g_scratch_ptr[device];
+  a.partial = scratch_ptr;
   a.partial_floats = kNoAllocScratchFloats;
   if (!FcW4StreamSupported(a)) return hipErrorInvalidValue;
   return LaunchFcW4StreamFused(&a, 1, stream, kernel_name);

@@ -112,7 +112,9 @@ struct ConvRuntimeCheckDesc {
   int ring_o_offset_index = -1;
   int ring_i_offset_index = -1;
   int ring_size = 0;
-  bool HasValues() const { return src_end_ch_index >= 0 || dst_end_ch_index >= 0; }
+  bool HasValues() const {
+    return src_end_ch_index >= 0 || dst_end_ch_index >= 0 || ring_o_offset_index >= 0 || ring_i_offset_index >= 0;
+  }
   // for batched weights: the tokens of the source row are sorted by weight matrix, sizes and offsets
   // of the groups are read from the params object (gpu_operation.h:396-406); num_groups == 0 = not set
   struct PackedGroups {
@@ -163,7 +165,7 @@ class HipOperation {
 namespace detail {
 inline mldhip_fc_desc FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
                                const ExternalWeights& weights, bool has_bias, int max_tokens,
-                               const ConvRuntimeCheckDesc& runtime_check = {});
+                               const ConvRuntimeCheckDesc& runtime_check = {}, int src_channels = 0, int dst_channels = 0);
 }  // namespace detail
 
 // CreateFullyConnectedWeightsBatchIds (common/kernels/fully_connected.h, .cc:1174-1216): the
@@ -173,8 +175,9 @@ inline mldhip_fc_desc FcDescOf(CalculationsPrecision precision, DataType src_typ
 // has one row that every id reads (its H is 1), else one row per id.
 inline Status CreateFullyConnectedWeightsBatchIds(CalculationsPrecision precision, DataType src_type,
                                                   DataType dst_type, const ExternalWeights& weights, bool has_bias,
-                                                  bool shared_src, int max_tokens, HipOperation* result) {
-  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens);
+                                                  bool shared_src, int max_tokens, HipOperation* result,
+                                                  const ConvRuntimeCheckDesc& runtime_check = {}) {
+  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens, runtime_check);
   mldhip_op* op = nullptr;
   const int rc = mldhip_fc_batch_ids_create(&d, weights.shape.h, shared_src ? 1 : 0, &op);
   if (rc != MLDHIP_OK) return Status::FromCode(rc);
@@ -182,12 +185,18 @@ inline Status CreateFullyConnectedWeightsBatchIds(CalculationsPrecision precisio
   return {};
 }
 
-// With runtime channel bounds the op takes a last src object "params" (int32 values on the device).
+// With runtime channel bounds or a ring offset the op takes a last src object "params" (int32 values on
+// the device).  Ringed weights (fully_connected.cc:411-471, 676-706): the tensor along the ringed axis
+// has channels of its own, which the reference reads from the `src` / `dst` descriptors it is handed:
+// `src_channels` with ring_i_offset_index (weights.shape.i = the ring), `dst_channels` with
+// ring_o_offset_index (weights.shape.o = the ring); 0 = the weights' own.
 inline Status CreateFullyConnectedExternalWeights(CalculationsPrecision precision, DataType src_type,
                                                   DataType dst_type, const ExternalWeights& weights, bool has_bias,
                                                   int max_tokens, HipOperation* result,
-                                                  const ConvRuntimeCheckDesc& runtime_check = {}) {
-  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens, runtime_check);
+                                                  const ConvRuntimeCheckDesc& runtime_check = {}, int src_channels = 0,
+                                                  int dst_channels = 0) {
+  const mldhip_fc_desc d = detail::FcDescOf(precision, src_type, dst_type, weights, has_bias, max_tokens, runtime_check,
+                                            src_channels, dst_channels);
   mldhip_op* op = nullptr;
   const int rc = mldhip_fc_create(&d, &op);
   if (rc != MLDHIP_OK) return Status::FromCode(rc);
@@ -210,8 +219,10 @@ inline Status CreateFullyConnectedOI(CalculationsPrecision precision, DataType s
 
 inline mldhip_fc_desc detail::FcDescOf(CalculationsPrecision precision, DataType src_type, DataType dst_type,
                                        const ExternalWeights& weights, bool has_bias, int max_tokens,
-                                       const ConvRuntimeCheckDesc& runtime_check) {
+                                       const ConvRuntimeCheckDesc& runtime_check, int src_channels, int dst_channels) {
   mldhip_fc_desc d{};
+  d.src_channels = src_channels;
+  d.dst_channels = dst_channels;
   d.has_runtime_check = 1;
   d.src_end_ch_index = runtime_check.src_end_ch_index;
   d.dst_end_ch_index = runtime_check.dst_end_ch_index;

@@ -7,13 +7,22 @@ Writer side, samples/llm/extract_weights_hf.py (read as text, not imported):
   quantize_int4_sym   :167-229, the `optimize_scale=False` branches, channel-wise and block-wise
                       (scale = absmax / 7, clip to [-8, 7])
   pack_int4           :232-241 (low nibble = even element)
-  The `optimize_scale=True` branches go through `_optimize_scale_search` (:78-134), whose
-  alpha-grid search is not restated: parity unpinned for it, and nothing here depends on it
-  (any scales are valid input for the loader).
+  optimize_scale_search :78-134, the grid search of the `optimize_scale=True` branches (the extractor's
+                      default): per block / channel, of the candidate scales absmax * alpha / qmax
+                      (alpha = linspace(1.0, 0.5, 7) for int4, linspace(1.0, 0.7, 7) for int8, float32),
+                      the first one that minimises the mean squared reconstruction error
+  quantize_int8_sym / quantize_int4_sym take `optimize_scale=True` for those branches (:148-159, :188-201,
+                      :211-219)
 Pinned by: the closed forms themselves are checked in tests/test_checkpoint.py through what the
 mathematics fixes (|w - q*s| <= s/2 away from the clip, q = +-7 / +-127 at the extreme of every
 row, scale 1 for zero rows, round-half-even on exact ties, nibble order against a hand-written
-byte string).
+byte string).  The grid search: the chosen scale is one of the seven candidates and no candidate
+reconstructs the block with a smaller mean squared error (checked in float64, block by block, by
+plain loops), ties go to the larger alpha, a block whose extreme is an outlier takes a smaller scale
+than absmax / qmax and clips the outlier, a block of evenly spread values keeps alpha = 1 where the
+closed form is optimal, zero blocks get scale 1 and codes 0.  Not checked against the extractor's
+output bit for bit (it is not run here): the last-place rounding of the float32 error sums could
+break a near-tie differently; parity for such near-ties is unpinned.
 
 Loader side, samples/llm/llm_file_tensor_loader.cc:
   group_size          :399-452 GetQuantizationIGroupSize
@@ -32,9 +41,30 @@ from . import oracle as O
 
 
 # ---- writer side -------------------------------------------------------------------------
-def quantize_int8_sym(w):
+def optimize_scale_search(blocks, bound, scale_bound, min_q, max_q, alphas):
+    """_optimize_scale_search (samples/llm/extract_weights_hf.py:78-134) without its chunking (which
+    only bounds memory): blocks (N, D), bound (N, 1) = max |block| -> (int8 codes (N, D), float32 scales
+    (N, 1)).  Candidate scales bound * alpha / scale_bound (zero -> 1), codes clip(round(x / scale)),
+    error = mean over the block of (x - code * scale)^2, argmin over the candidates (first on ties), all
+    in the arrays' own float type as numpy evaluates the reference's expressions."""
+    blocks = np.asarray(blocks)
+    cand = (bound[:, None, :] * alphas[None, :, None]) / scale_bound
+    cand = np.where(cand == 0.0, 1.0, cand)
+    cq = np.clip(np.round(blocks[:, None, :] / cand), min_q, max_q)
+    err = np.mean((blocks[:, None, :] - cq * cand) ** 2, axis=-1)
+    best = np.argmin(err, axis=1)
+    scales = np.take_along_axis(cand[:, :, 0], best[:, None], axis=1).astype(np.float32)
+    q = np.take_along_axis(cq, best[:, None, None], axis=1)[:, 0, :].astype(np.int8)
+    return q, scales
+
+
+def quantize_int8_sym(w, optimize_scale=False):
     """w: (o, i) float -> (int8 (o, i), float32 scale (o,))."""
     w = np.asarray(w)
+    if optimize_scale:
+        bound = np.max(np.abs(w), axis=-1, keepdims=True)
+        q, scale = optimize_scale_search(w, bound, 127.0, -128, 127, np.linspace(1.0, 0.7, num=7, dtype=np.float32))
+        return q, scale.reshape(-1).astype(np.float32)
     bound = np.max(np.abs(w), axis=1, keepdims=True)
     scale = bound / 127.0
     scale = np.where(scale == 0.0, 1.0, scale)
@@ -42,9 +72,17 @@ def quantize_int8_sym(w):
     return q, np.squeeze(scale, axis=1).astype(np.float32)
 
 
-def quantize_int4_sym(w, block_size=0):
+def quantize_int4_sym(w, block_size=0, optimize_scale=False):
     """w: (o, i) float -> (int8-held int4 (o, i), float32 scale (o,) or (o, i / block_size))."""
     w = np.asarray(w)
+    if optimize_scale:
+        o, i = w.shape
+        if block_size > 0 and i % block_size:
+            raise ValueError("not divisible by block_size")
+        blocks = w.reshape(-1, block_size) if block_size > 0 else w
+        bound = np.max(np.abs(blocks), axis=-1, keepdims=True)
+        q, scale = optimize_scale_search(blocks, bound, 7.0, -8, 7, np.linspace(1.0, 0.5, num=7, dtype=np.float32))
+        return q.reshape(o, i), (scale.reshape(o, i // block_size) if block_size > 0 else scale.reshape(o)).astype(np.float32)
     if block_size > 0:
         o, i = w.shape
         if i % block_size:

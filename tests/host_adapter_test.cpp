@@ -59,7 +59,8 @@ int main() {
                                            false, 1, &bad);
   EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !bad.valid());
 
-  // runtime channel bounds: one more src object, "params", registered last; ringed weights are refused
+  // runtime channel bounds: one more src object, "params", registered last; ringed uint4 weights are refused
+  // as the reference refuses them (types under 8 bits, fully_connected.cc:1087-1092)
   w.desc = GetFullyConnectedInt4WeightsDesc(w.shape);
   ConvRuntimeCheckDesc rc_desc;
   rc_desc.src_end_ch_index = 1;
@@ -76,6 +77,24 @@ int main() {
   st = CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32F16, DataType::kFloat16, DataType::kFloat16, w,
                                            false, 1, &ringed, rc_desc);
   EXPECT(st.code == MLDHIP_INVALID_ARGUMENT && !ringed.valid());
+  // ringed uint8 weights: a ring of 56 input rows under 20 src channels (fully_connected_test_util.cc:742-900)
+  {
+    ExternalWeights w8;
+    w8.shape = OHWI{72, 1, 1, 56};
+    w8.desc = GetFullyConnectedInt8WeightsDesc(w8.shape);
+    w8.scale_zp_shape = OHWI{72, 1, 1, 1};
+    w8.has_scale_tensor = true;
+    ConvRuntimeCheckDesc ring;
+    ring.ring_i_offset_index = 0;
+    ring.src_end_ch_index = 1;
+    ring.ring_size = 56;
+    HipOperation ring_op;
+    EXPECT(CreateFullyConnectedExternalWeights(CalculationsPrecision::kF32, DataType::kFloat32, DataType::kFloat32, w8,
+                                               /*has_bias=*/true, 1, &ring_op, ring, /*src_channels=*/20)
+               .ok());
+    names = ring_op.GetSrcTensorsNames();
+    EXPECT(names.size() == 5 && names[4] == "params");
+  }
 
   // FullyConnectedOI: the same op over output groups of one slice (fully_connected_oi_test_util.cc:109-111)
   ExternalWeights woi = w;

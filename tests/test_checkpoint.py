@@ -155,3 +155,77 @@ def test_loader_errors(tmp_path):
     info = M.checkpoint_fc_probe(d, "z.weight", "z", 4, 8, 4)
     got = M.checkpoint_fc_read(d, "z.weight", "z", info, M.FLOAT32)
     assert got["zero_point"].tolist() == [0.0, 3.0, 1.5, 6.0]
+
+
+# ---- the extractor's scale search (samples/llm/extract_weights_hf.py:78-134) -------------------------
+def _mse(block, scale, lo, hi):
+    """float64, plain loop: mean squared error of the block quantized with `scale`."""
+    total = 0.0
+    for x in block:
+        q = min(max(float(np.round(np.float64(x) / scale)), lo), hi)
+        total += (float(x) - q * scale) ** 2
+    return total / len(block)
+
+
+@pytest.mark.parametrize("bits,block", [(4, 32), (4, 0), (8, 0)])
+def test_scale_search_picks_the_best_candidate(bits, block):
+    """The chosen scale is one of the seven candidates absmax * alpha / qmax and no candidate gives a
+    smaller mean squared error (float64, block by block); the codes are the rounding with that scale."""
+    rng = np.random.default_rng(bits + block)
+    o, i = 12, 64
+    w = rng.standard_normal((o, i)).astype(np.float32)
+    w[3, 5] = 9.0      # an outlier: a smaller scale that clips it wins
+    w[7] = 0.0         # a zero row
+    qmax, lo, hi = (7.0, -8, 7) if bits == 4 else (127.0, -128, 127)
+    alphas = np.linspace(1.0, 0.5 if bits == 4 else 0.7, num=7, dtype=np.float32)
+    if bits == 4:
+        q, scale = CK.quantize_int4_sym(w, block, optimize_scale=True)
+    else:
+        q, scale = CK.quantize_int8_sym(w, optimize_scale=True)
+    blocks = w.reshape(-1, block) if block else w
+    qb = q.reshape(blocks.shape)
+    sb = scale.reshape(-1)
+    assert q.dtype == np.int8 and scale.dtype == np.float32 and q.shape == w.shape
+    assert scale.shape == ((o, i // block) if block else (o,))
+    for b in range(blocks.shape[0]):
+        bound = float(np.max(np.abs(blocks[b])))
+        if bound == 0.0:
+            assert sb[b] == 1.0 and not qb[b].any()
+            continue
+        cands = [float(np.float32(np.float32(bound) * a) / np.float32(qmax)) for a in alphas]
+        assert any(abs(float(sb[b]) - c) <= 1e-7 * c for c in cands), (b, sb[b], cands)
+        errs = [_mse(blocks[b], c, lo, hi) for c in cands]
+        mine = _mse(blocks[b], float(sb[b]), lo, hi)
+        assert mine <= min(errs) * (1 + 1e-5) + 1e-12, (b, mine, errs)
+        want = np.clip(np.round(blocks[b] / sb[b]), lo, hi).astype(np.int8)
+        assert np.array_equal(qb[b], want)
+    if bits == 4 and block:
+        # the outlier's block clips it: a scale below absmax / 7, the outlier at the top code
+        k = 3 * (i // block) + 5 // block
+        assert sb[k] < 9.0 / 7.0 * (1 - 1e-6) and q[3, 5] == 7
+
+
+def test_scale_search_ties_and_spread_blocks():
+    """A block that the largest scale reconstructs exactly keeps alpha = 1 (the first candidate wins a
+    tie at zero error, and nothing beats zero); an evenly spread block of codes -7..7 times a scale s
+    is reproduced with scale s."""
+    s = np.float32(0.25)
+    block = (np.arange(-7, 8, dtype=np.float32) * s)[None, :]
+    q, scale = CK.quantize_int4_sym(np.concatenate([block, block[:, ::-1]], axis=1), 15, optimize_scale=True)
+    assert np.allclose(scale, s) and np.array_equal(q[0, :15], np.arange(-7, 8))
+    # the closed form is the alpha = 1 candidate
+    q1, s1 = CK.quantize_int4_sym(block, 0, optimize_scale=False)
+    q2, s2 = CK.quantize_int4_sym(block, 0, optimize_scale=True)
+    assert np.array_equal(q1, q2) and np.allclose(s1, s2)
+
+
+def test_scale_search_files_load_like_any_other(tmp_path):
+    """Scales from the grid search are ordinary loader input: write, load, compare."""
+    rng = np.random.default_rng(9)
+    o, i, block = 16, 64, 32
+    w = rng.standard_normal((o, i)).astype(np.float32)
+    q, scale = CK.quantize_int4_sym(w, block, optimize_scale=True)
+    d = str(tmp_path) + "/"
+    CK.write_fc_files(d, "layer", q, scale, 4)
+    got = CK.load_fc(d, "layer", o, i, 4, np.float32)
+    assert got["group_size"] == block
