@@ -182,6 +182,7 @@ int mldhip_set_tuning(const char* name, int value) {
   const struct { const char* name; int* field; } knobs[] = {
       {"force_generic", &t.force_generic}, {"gemv_mfma", &t.gemv_mfma}, {"gemv_fast", &t.gemv_fast},
       {"fc_group", &t.fc_group}, {"gemv_rows_rpt", &t.gemv_rows_rpt},
+      {"gemv_one_chunk", &t.gemv_one_chunk},
       {"gemv_lpr", &t.gemv_lpr}, {"gemv_waves", &t.gemv_waves}, {"gemv_ksplit", &t.gemv_ksplit},
       {"gemv_narrow_max_mb", &t.gemv_narrow_max_mb}, {"gemm_fm", &t.gemm_fm}, {"gemm_ksplit", &t.gemm_ksplit},
       {"gemm_no_pair", &t.gemm_no_pair}, {"gemm_dual", &t.gemm_dual}, {"gemm_xcd_m", &t.gemm_xcd_m},

@@ -646,12 +646,43 @@ struct StripParams {
   int rows, src_rows, weights_batch;
 };
 
+// The matrix a work-group belongs to and its strip number inside it.  Every field of every list
+// entry sits at a fixed offset of the kernel arguments, so all of them are fetched by the scalar
+// loads at the top of the kernel and chosen with scalar selects; indexing the list with a run-time
+// number would make the entry's loads wait for a first round trip (the strip ends).
+template <bool MULTI>
+__device__ __forceinline__ StripSegment SelectSegment(const StripParams& p, int& strip) {
+  StripSegment sg = p.seg[0];
+  if (MULTI) {
+    const int e0 = p.seg[0].strip_end, e1 = p.seg[1].strip_end;
+    const bool second = p.segments > 1 && strip >= e0;
+    const bool third = p.segments > 2 && strip >= e1;
+    const StripSegment s1 = p.seg[1], s2 = p.seg[2];
+    // (an input-only operand keeps the pointers' address space; it makes the compiler fetch the
+    // entries with the first batch of scalar loads instead of behind the first wait)
+    asm volatile("" : : "s"(s1.weights), "s"(s2.weights), "s"(s1.scale), "s"(s2.scale), "s"(sg.weights), "s"(sg.scale));
+#define MLD_PICK(f) sg.f = third ? s2.f : (second ? s1.f : sg.f)
+    MLD_PICK(weights); MLD_PICK(scale); MLD_PICK(zero_point); MLD_PICK(bias); MLD_PICK(dst);
+    MLD_PICK(n_pad); MLD_PICK(n_off);
+#undef MLD_PICK
+    strip -= third ? e1 : (second ? e0 : 0);
+  }
+  return sg;
+}
+
 // BATCHED: batched weights selected by runtime ids, one dst row of one token per blockIdx.z (no K
 // split, one matrix list entry): the strip of matrix b is the b-th of its output group's runs,
 // scales are [group][matrix][channel], the token of source row r is every src_rows-th 8 bytes.
-template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false>
+// ONE: every thread owns exactly one chunk and K is not split across work-groups (the launch shape
+// of the wide layers: c.f. the launcher).  The kernel then has no chunk loop, no test for a first
+// chunk and no split-K branch, the lane's byte offsets are 32-bit values over scalar bases, and
+// the compiler is left to order loads and arithmetic (it defers the last weight loads behind the
+// first rows' arithmetic).  At a launch of a few microseconds every instruction in front of the
+// first load and behind the last one counts: 4 waves per SIMD issue them one after the other.
+template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false, bool ONE = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) {
   static_assert(!BATCHED || !MULTI, "a batched launch has one matrix list entry");
+  static_assert(!ONE || (!BATCHED && !ZP), "the one-chunk form serves plain launches");
   constexpr int ROWS = WAVES * 64 / LPR;  // chunks of 8 K-slices the work-group covers per pass
   constexpr int STRIP = LPR * 8;          // channels of a strip (one output group of the layout)
   __shared__ float red[WAVES][STRIP];
@@ -660,12 +691,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   const int wave = tid >> 6;
   const int col = lane % LPR;
   const int row = tid / LPR;
-  int si = 0, strip = blockIdx.x;
-  if (MULTI && p.segments > 1 && strip >= p.seg[0].strip_end) {
-    si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
-    strip -= p.seg[si - 1].strip_end;
-  }
-  const StripSegment& sg = p.seg[MULTI ? si : 0];
+  int strip = blockIdx.x;
+  const StripSegment sg = SelectSegment<MULTI>(p, strip);
   // Everything the loop reads from the arguments, fetched here in one go: a scalar load first
   // issued inside the loop would be a second round trip in front of the weight loads.
   struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
@@ -689,9 +716,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   const size_t group_stride = (size_t)n_pad * nb;  // elements per scale group
   // (the pointers are left to the compiler: through an asm operand they would lose their address
   // space and turn every load into a flat one)
-  const int ky = blockIdx.y;
-  const int c_begin = ky * p.chunks_per_split;
-  const int c_end = min(c_begin + p.chunks_per_split, p.chunks);
+  const int ky = ONE ? 0 : (int)blockIdx.y;
+  const int c_begin = ONE ? 0 : ky * p.chunks_per_split;
+  const int c_end = ONE ? ROWS : min(c_begin + p.chunks_per_split, p.chunks);
   // the output this thread finishes: channel `ch` of the strip (the channel the wave sum leaves in
   // this lane when the work-group is one wave, else thread order)
   const int ch_wave = col * 8 + ((lane >> 3) & 7);  // the channel whose wave sum this lane holds
@@ -704,7 +731,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
   u32x4 zv = {0u, 0u, 0u, 0u};
   // row r of the strip: LPR uint4; chunk c: 8 rows
-  const u32x4* wstrip = weights + ((size_t)strip * nb + wb) * ks * LPR + col;
+  const u32x4* wstrip = weights + ((size_t)strip * nb + wb) * ks * LPR + (ONE ? 0 : col);
   // Loads of one chunk, in the order the memory pipeline returns them (loads return in order): the
   // small ones that come from cache first (activations, group scales), then the eight weight loads
   // back to back.
@@ -712,7 +739,13 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   u32x2 ab[8];
   auto issue = [&](int c) {
     const u32x4* wp = wstrip + (size_t)c * (8 * LPR);
-    if (BATCHED) {
+    if (ONE) {  // c = row: byte offsets of the lane in 32 bits, the strip's base is scalar
+      const uint32_t voff = ((uint32_t)row * (8 * LPR) + (uint32_t)col) * 16u;
+      wp = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wstrip) + voff);
+      const u32x4* ap = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.act) + (uint32_t)row * 64u);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) a4[j] = ap[j];
+    } else if (BATCHED) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) ab[j] = arows[(size_t)(c * 8 + j) * src_rows];
     } else {
@@ -743,9 +776,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
       const float centered = fmaf(centre, asum[0], t[0][o]);
       if (GROUPED) {
         const half2_t sp = AsHalf2(sv[o >> 1]);
-        acc[o] = fmaf((float)sp[o & 1], centered, acc[o]);
+        acc[o] = ONE ? (float)sp[o & 1] * centered : fmaf((float)sp[o & 1], centered, acc[o]);
       } else {
-        acc[o] += centered;
+        acc[o] = ONE ? centered : acc[o] + centered;
       }
     }
   };
@@ -753,20 +786,22 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   // and bias of the output this thread finishes are fetched behind its weight loads: in front of
   // them, their trip to memory would hold back the use of every weight that arrives before they do.
   int c = c_begin + row;
-  const bool first = c < c_end;
+  const bool first = ONE ? true : c < c_end;
   if (ZP && !GROUPED) zv = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * STRIP + col * 8);
   if (first) issue(c);
   const unsigned short out_scale_raw = reinterpret_cast<const unsigned short*>(scale)[n_out];
   const unsigned short out_bias_raw = bias_src[n_out];
   // the fence keeps the arithmetic behind all the loads, so that the waits count the weight loads
   // down one by one instead of some of them being issued after the first wait
-  __builtin_amdgcn_sched_barrier(0);
+  if (!ONE) __builtin_amdgcn_sched_barrier(0);
   if (first) {
     consume();
-    for (c += ROWS; c < c_end; c += ROWS) {
-      issue(c);
-      __builtin_amdgcn_sched_barrier(0);
-      consume();
+    if (!ONE) {
+      for (c += ROWS; c < c_end; c += ROWS) {
+        issue(c);
+        __builtin_amdgcn_sched_barrier(0);
+        consume();
+      }
     }
   }
   float v = WaveStripSum<LPR>(acc, lane);
@@ -778,7 +813,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
 #pragma unroll
     for (int q = 0; q < WAVES; ++q) v += red[q][tid];
   }
-  if (p.ksplit == 1) {
+  if (ONE || p.ksplit == 1) {
     if (!GROUPED) v *= __half2float(__ushort_as_half(out_scale_raw));
     __half h = __float2half_rn(v);
     if (sg.bias) h = __hadd(h, __ushort_as_half(out_bias_raw));
@@ -833,6 +868,16 @@ hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream
       return hipGetLastError();
     }
     return hipErrorInvalidValue;
+  }
+  // every thread exactly one chunk, K inside the work-group: the one-chunk form (strips of 64 channels)
+  if constexpr (LPR == 8) {
+    if (!zp && p.ksplit == 1 && p.chunks == WAVES * 64 / LPR && GetTuning().gemv_one_chunk != 0) {
+#define MLD_STRIP_1(G, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, false, MU, false, true>), grid, block, 0, stream, p)
+      if (grouped) { if (multi) MLD_STRIP_1(true, true); else MLD_STRIP_1(true, false); }
+      else         { if (multi) MLD_STRIP_1(false, true); else MLD_STRIP_1(false, false); }
+#undef MLD_STRIP_1
+      return hipGetLastError();
+    }
   }
 #define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
@@ -966,7 +1011,9 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
 // K reduction: the 8 channel sums of the 64 lanes by the register exchanges of the strip kernel
 // (all lanes hold rows of the same 8 channels), across waves through LDS in wave order.
 // ------------------------------------------------------------------------------------------
-template <int WAVES, bool GROUPED, bool ZP, bool MULTI>
+// ONE: K is exactly 8 rows per thread (the shape the launcher sizes the work-group for): one pass
+// without bounds, the lane's byte offsets are 32-bit values over scalar bases.
+template <int WAVES, bool GROUPED, bool ZP, bool MULTI, bool ONE = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   constexpr int T = WAVES * 64;
   __shared__ float red[WAVES][8];
@@ -976,13 +1023,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   // Work-groups go round-robin to the 8 XCDs.  The scales of 8 neighbouring strips share a 128-byte
   // line per scale group, so neighbouring strips are given to work-groups of one XCD (whose L2 then
   // fetches the line once): of every 64 work-groups, XCD x takes strips 8x .. 8x + 7.
-  int si = 0, strip = blockIdx.x;
+  int strip = blockIdx.x;
   if (strip < (int)(gridDim.x & ~63u)) strip = (strip & ~63) + ((strip & 7) << 3) + ((strip >> 3) & 7);
-  if (MULTI && p.segments > 1 && strip >= p.seg[0].strip_end) {
-    si = (p.segments > 2 && strip >= p.seg[1].strip_end) ? 2 : 1;
-    strip -= p.seg[si - 1].strip_end;
-  }
-  const StripSegment& sg = p.seg[MULTI ? si : 0];
+  const StripSegment sg = SelectSegment<MULTI>(p, strip);
   struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
   const u32x4* wstrip = sg.weights + (size_t)strip * p.ks;  // row r of the strip: K-slice r, 2 slices x 8 bytes
   const u32x2* act2 = reinterpret_cast<const u32x2*>(p.act);
@@ -998,26 +1041,46 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   u32x4 zv_lin = {0u, 0u, 0u, 0u};
   if (ZP && !GROUPED) zv_lin = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * 8);
 
-  for (int r0 = tid; r0 < ks; r0 += 8 * T) {
+  for (int r0 = tid; ONE ? r0 == tid : r0 < ks; r0 += 8 * T) {
     u32x4 w[8], sv[8], zv[8];
     u32x2 a[8];
     // small loads that come from cache first, then the eight weight loads back to back
+    if (ONE) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int r = r0 + T * j;
-      const u32x2 v = act2[min(r, ks - 1)];
-      a[j] = u32x2{r < ks ? v[0] : 0u, r < ks ? v[1] : 0u};
-    }
-    if (GROUPED) {
+      for (int j = 0; j < 8; ++j)
+        a[j] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const char*>(p.act) + (uint32_t)(tid + T * j) * 8u);
+      if (GROUPED) {
+        // a scale group has at most T K-slices (the launcher checks), so row tid + T * j lies
+        // (T * j) >> group_shift groups behind row tid: one lane offset over 8 scalar bases
+        const uint32_t so = (__umul24((uint32_t)tid >> group_shift, (uint32_t)n_pad) + (uint32_t)strip * 8u) * 2u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const size_t sj = (size_t)((uint32_t)((T * j) >> group_shift) * (uint32_t)n_pad) * 2u;
+          sv[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(scale) + sj + so);
+          if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(zero_point) + sj + so);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wstrip) + (uint32_t)(tid + T * j) * 16u));
+    } else {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const size_t so = (size_t)(min(r0 + T * j, ks - 1) >> group_shift) * n_pad + (size_t)strip * 8;
-        sv[j] = *reinterpret_cast<const u32x4*>(scale + so);
-        if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(zero_point + so);
+        const int r = r0 + T * j;
+        const u32x2 v = act2[min(r, ks - 1)];
+        a[j] = u32x2{r < ks ? v[0] : 0u, r < ks ? v[1] : 0u};
       }
-    }
+      if (GROUPED) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wstrip + min(r0 + T * j, ks - 1));
+        for (int j = 0; j < 8; ++j) {
+          const size_t so = (size_t)(min(r0 + T * j, ks - 1) >> group_shift) * n_pad + (size_t)strip * 8;
+          sv[j] = *reinterpret_cast<const u32x4*>(scale + so);
+          if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(zero_point + so);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wstrip + min(r0 + T * j, ks - 1));
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -1083,6 +1146,20 @@ template <int WAVES>
 hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
   const dim3 block(WAVES * 64);
+  // exactly 8 rows per thread, scale tensors within 32-bit byte offsets: the one-pass form
+  if (!zp && p.ks == 8 * WAVES * 64 && GetTuning().gemv_one_chunk != 0) {
+    bool fits = true;
+    for (int i = 0; i < p.segments; ++i)
+      fits = fits && (!grouped || ((size_t)(p.ks >> p.group_chunks) * p.seg[i].n_pad < ((size_t)1 << 24) &&
+                                   p.seg[i].n_pad < (1 << 24) && (1 << p.group_chunks) <= WAVES * 64));
+    if (fits) {
+#define MLD_ROWS_1(G, MU) hipLaunchKernelGGL((fc_w4_rows_kernel<WAVES, G, false, MU, true>), grid, block, 0, stream, p)
+      if (grouped) { if (multi) MLD_ROWS_1(true, true); else MLD_ROWS_1(true, false); }
+      else         { if (multi) MLD_ROWS_1(false, true); else MLD_ROWS_1(false, false); }
+#undef MLD_ROWS_1
+      return hipGetLastError();
+    }
+  }
 #define MLD_ROWS(G, Z, MU) hipLaunchKernelGGL((fc_w4_rows_kernel<WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
     if (zp) { if (multi) MLD_ROWS(true, true, true); else MLD_ROWS(true, true, false); }

@@ -164,6 +164,7 @@ struct Tuning {
   int fc_group = -1;            // output group size that mldhip_fc_int4_weights_desc returns where it divides the slices
   int gemv_lpr = -1, gemv_waves = -1, gemv_ksplit = -1, gemv_narrow_max_mb = -1;
   int gemv_rows_rpt = -1;       // rows per thread the row-interleaved GEMV sizes its work-groups for
+  int gemv_one_chunk = -1;      // 0: never take the one-chunk form of the contiguous-strip GEMV
   int gemm_fm = -1, gemm_ksplit = -1, gemm_no_pair = -1, gemm_dual = -1, gemm_xcd_m = -1;
   int gemm_i8_fm = -1;
 };
