@@ -164,7 +164,7 @@ def run_other(args, torch, M, W):
             rng = np.random.default_rng(0)
             w = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
             src = rng.integers(-128, 128, size=(m, k), dtype=np.int8)
-            desc = M.fc_int4_weights_desc(n, k)
+            desc = M.fc_int4_weights_desc(n, k, reference=args.layout == "reference")
             packed = torch.from_numpy(M.rearrange_int8_as_uint4(w, desc))
             act = torch.from_numpy(W.to_slices(src)).cuda()
             out_t = torch.zeros(((n + 3) // 4, m, 4), dtype=torch.int32, device="cuda")
@@ -178,7 +178,8 @@ def run_other(args, torch, M, W):
                 ops.append(op)
                 keep.append(wt)
             nbytes = n * k // 2 + k + n * 4  # W + int8 act + int32 out
-            label = "f2: int8-math FullyConnected decode GEMV M=1 K=4096 N=14336, int8 act x uint4 weights -> int32"
+            label = ("f2: int8-math FullyConnected decode GEMV M=1 K=4096 N=14336, int8 act x uint4 weights -> int32, "
+                     "kOSpatialIOGroupI4O4 output_group_size %d" % desc.output_group_size)
             metric, dtype = "int8_math_decode_gemv_hbm_bandwidth", "i8 x u4, i32 accumulate (v_dot4)"
         wall, us, reg = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup,
                                    ring=len(ops))

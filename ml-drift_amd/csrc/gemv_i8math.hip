@@ -169,6 +169,88 @@ __global__ __launch_bounds__(WAVES * 64) void fc_i8math_stream_kernel(I8MathPara
   }
 }
 
+// uint4 weights, one token, strips of 64 channels that lie inside one output group of the packed
+// weights (grid x = strip of the group, y = group): 8 lanes cover a 128-byte row segment, a thread
+// owns chunks of 8 consecutive K-slices (ONE: exactly one, no loop), the 8 channel sums of a lane
+// are added across the 8 rows of a wave by register exchanges that halve the live values per
+// step and across waves through 4 KB of LDS.  CONTIG: output groups of 16 slices, a strip's rows
+// lie one after the other (128 bytes apart: immediate offsets).  Integer sums: any order is exact.
+typedef unsigned u32x2s __attribute__((ext_vector_type(2)));
+template <int WAVES, bool ONE, bool CONTIG>
+__global__ __launch_bounds__(WAVES * 64) void fc_i8math_strip_kernel(I8MathParams p) {
+  constexpr int ROWS = WAVES * 8;
+  __shared__ int red[WAVES][64];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63, wave = tid >> 6;
+  const uint32_t col = tid & 7, row = tid >> 3;
+  const uint32_t row_bytes = CONTIG ? 128u : (uint32_t)p.gu4 * 16u;
+  const char* gbase = reinterpret_cast<const char*>(p.weights + (size_t)blockIdx.y * p.ks * p.gu4 + (size_t)blockIdx.x * 8);
+  const int4* act4 = reinterpret_cast<const int4*>(p.act);
+  int acc[8], asum = 0;
+#pragma unroll
+  for (int o = 0; o < 8; ++o) acc[o] = 0;
+  for (uint32_t c = row; ONE ? c == row : c < (uint32_t)p.chunks; c += ROWS) {
+    u32x4 w[8];
+    const uint32_t voff = __umul24(c * 8u, row_bytes) + col * 16u;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(gbase + voff + (CONTIG ? (uint32_t)j * 128u : __umul24((uint32_t)j, row_bytes))));
+    const int4 a0 = act4[c * 2], a1 = act4[c * 2 + 1];
+    const int a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+    if (!ONE) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const uint32_t p01 = Perm(w[j][2 * b + 1], w[j][2 * b], 0x06040200u);  // (o0|o1) of i0..i3
+        const uint32_t p23 = Perm(w[j][2 * b + 1], w[j][2 * b], 0x07050301u);  // (o2|o3) of i0..i3
+        acc[4 * b + 0] = __builtin_amdgcn_sdot4(a[j], (int)(p01 & 0x0F0F0F0Fu), acc[4 * b + 0], false);
+        acc[4 * b + 1] = __builtin_amdgcn_sdot4(a[j], (int)((p01 >> 4) & 0x0F0F0F0Fu), acc[4 * b + 1], false);
+        acc[4 * b + 2] = __builtin_amdgcn_sdot4(a[j], (int)(p23 & 0x0F0F0F0Fu), acc[4 * b + 2], false);
+        acc[4 * b + 3] = __builtin_amdgcn_sdot4(a[j], (int)((p23 >> 4) & 0x0F0F0F0Fu), acc[4 * b + 3], false);
+      }
+      asum = __builtin_amdgcn_sdot4(a[j], 0x01010101, asum, false);
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < 8; ++o) acc[o] -= 8 * asum;
+  int s4[4], s2[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const u32x2s r = __builtin_amdgcn_permlane32_swap((uint32_t)acc[i], (uint32_t)acc[i + 4], false, false);
+    s4[i] = (int)(r[0] + r[1]);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const u32x2s r = __builtin_amdgcn_permlane16_swap((uint32_t)s4[i], (uint32_t)s4[i + 2], false, false);
+    s2[i] = (int)(r[0] + r[1]);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    s2[i] += (int)__builtin_amdgcn_update_dpp(0u, (uint32_t)s2[i], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+  const int mine = (lane & 8) ? s2[1] : s2[0];
+  red[wave][col * 8 + ((lane >> 3) & 7)] = mine;  // (lanes that hold the same channel write the same value)
+  __syncthreads();
+  if (tid < 64) {
+    int v = 0;
+#pragma unroll
+    for (int q = 0; q < WAVES; ++q) v += red[q][tid];
+    const uint32_t strip = blockIdx.y * ((uint32_t)p.gu4 >> 3) + blockIdx.x;
+    p.dst[strip * 64u + tid] = v;
+  }
+}
+
+template <int WAVES>
+hipError_t LaunchStripI8(const I8MathParams& p, dim3 grid, hipStream_t stream) {
+  const dim3 block(WAVES * 64);
+  const bool one = p.chunks == WAVES * 8, contig = p.gu4 == 8;
+#define MLD_I8STRIP(O, C) hipLaunchKernelGGL((fc_i8math_strip_kernel<WAVES, O, C>), grid, block, 0, stream, p)
+  if (one) { if (contig) MLD_I8STRIP(true, true); else MLD_I8STRIP(true, false); }
+  else     { if (contig) MLD_I8STRIP(false, true); else MLD_I8STRIP(false, false); }
+#undef MLD_I8STRIP
+  return hipGetLastError();
+}
+
 template <int WBITS, int LPR, int WAVES, bool BATCHED>
 hipError_t LaunchMB(const I8MathParams& p, dim3 grid, hipStream_t stream) {
   const dim3 block(WAVES * 64);
@@ -223,6 +305,17 @@ hipError_t LaunchFcInt8MathStream(const int8_t* act, const uint8_t* weights, int
   const int lpr = (long)DivUp(p.row_u4, 8) * (batch.ids ? batch.rows : 1) >= 128 ? 8 : 4;
   const int waves = (m > 1 || p.chunks <= 4 * 64 / lpr) ? 4 : 16;
   if (kernel_name) *kernel_name = "fc_i8math_stream_kernel";
+  // one token over uint4 strips of 64 channels inside one output group, whole chunks of K, enough
+  // strips for the chip, offsets within 24-bit factors: the strip form
+  if (weight_bits == 4 && m == 1 && batch.ids == nullptr && p.gu4 % 8 == 0 && p.row_u4 % 8 == 0 && p.ks % 8 == 0 &&
+      p.row_u4 / 8 >= 128 && p.ks < (1 << 20) && p.gu4 < (1 << 20) && (size_t)p.ks * p.gu4 * 16 < ((size_t)1 << 32) &&
+      GetTuning().gemv_one_chunk != 0) {
+    const dim3 grid(p.gu4 / 8, p.row_u4 / p.gu4);
+    if (kernel_name) *kernel_name = "fc_i8math_strip_kernel";
+    if (p.chunks <= 32) return LaunchStripI8<4>(p, grid, stream);
+    if (p.chunks <= 64) return LaunchStripI8<8>(p, grid, stream);
+    return LaunchStripI8<16>(p, grid, stream);
+  }
   return weight_bits == 4 ? LaunchW<4>(p, lpr, waves, stream) : LaunchW<8>(p, lpr, waves, stream);
 }
 

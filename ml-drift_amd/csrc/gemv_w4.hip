@@ -632,7 +632,7 @@ struct StripSegment {
   int n_pad;      // channels of the matrix (a multiple of 64)
   int strip_end;  // work-groups [strip_end of the previous, strip_end) belong to this matrix
   int n_off;      // channels of the launch's matrices before this one (split-K sums)
-  int reserved;
+  int row_u4;     // STRIDED only: 16-byte items between two K-slice rows of a strip (one output group over all slices)
 };
 struct StripParams {
   const __half* act;
@@ -663,7 +663,7 @@ __device__ __forceinline__ StripSegment SelectSegment(const StripParams& p, int&
     asm volatile("" : : "s"(s1.weights), "s"(s2.weights), "s"(s1.scale), "s"(s2.scale), "s"(sg.weights), "s"(sg.scale));
 #define MLD_PICK(f) sg.f = third ? s2.f : (second ? s1.f : sg.f)
     MLD_PICK(weights); MLD_PICK(scale); MLD_PICK(zero_point); MLD_PICK(bias); MLD_PICK(dst);
-    MLD_PICK(n_pad); MLD_PICK(n_off);
+    MLD_PICK(n_pad); MLD_PICK(n_off); MLD_PICK(row_u4);
 #undef MLD_PICK
     strip -= third ? e1 : (second ? e0 : 0);
   }
@@ -679,10 +679,13 @@ __device__ __forceinline__ StripSegment SelectSegment(const StripParams& p, int&
 // the compiler is left to order loads and arithmetic (it defers the last weight loads behind the
 // first rows' arithmetic).  At a launch of a few microseconds every instruction in front of the
 // first load and behind the last one counts: 4 waves per SIMD issue them one after the other.
-template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false, bool ONE = false>
+// STRIDED (with ONE): the weights are packed in one output group over all slices (the reference's
+// own layout): the 128-byte rows of a strip lie a whole K-slice row of the matrix apart.
+template <int LPR, int WAVES, bool GROUPED, bool ZP, bool MULTI, bool BATCHED = false, bool ONE = false, bool STRIDED = false>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) {
   static_assert(!BATCHED || !MULTI, "a batched launch has one matrix list entry");
   static_assert(!ONE || (!BATCHED && !ZP), "the one-chunk form serves plain launches");
+  static_assert(!STRIDED || ONE, "strided strips are served by the one-chunk form");
   constexpr int ROWS = WAVES * 64 / LPR;  // chunks of 8 K-slices the work-group covers per pass
   constexpr int STRIP = LPR * 8;          // channels of a strip (one output group of the layout)
   __shared__ float red[WAVES][STRIP];
@@ -731,7 +734,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
   u32x4 zv = {0u, 0u, 0u, 0u};
   // row r of the strip: LPR uint4; chunk c: 8 rows
-  const u32x4* wstrip = weights + ((size_t)strip * nb + wb) * ks * LPR + (ONE ? 0 : col);
+  const u32x4* wstrip = STRIDED ? weights + (size_t)strip * LPR : weights + ((size_t)strip * nb + wb) * ks * LPR + (ONE ? 0 : col);
+  const uint32_t row_items = STRIDED ? (uint32_t)sg.row_u4 : (uint32_t)LPR;  // 16-byte items from one K-slice row to the next
   // Loads of one chunk, in the order the memory pipeline returns them (loads return in order): the
   // small ones that come from cache first (activations, group scales), then the eight weight loads
   // back to back.
@@ -740,7 +744,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   auto issue = [&](int c) {
     const u32x4* wp = wstrip + (size_t)c * (8 * LPR);
     if (ONE) {  // c = row: byte offsets of the lane in 32 bits, the strip's base is scalar
-      const uint32_t voff = ((uint32_t)row * (8 * LPR) + (uint32_t)col) * 16u;
+      const uint32_t voff = (__umul24((uint32_t)row * 8u, row_items) + (uint32_t)col) * 16u;
       wp = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wstrip) + voff);
       const u32x4* ap = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(p.act) + (uint32_t)row * 64u);
 #pragma unroll
@@ -759,7 +763,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
       if (ZP) zv = *reinterpret_cast<const u32x4*>(zero_point + so);
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + j * LPR);
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + (STRIDED ? (size_t)j * row_items : (size_t)j * LPR));
   };
   auto consume = [&]() {
     u32x2 a[8][1];
@@ -856,7 +860,7 @@ __global__ __launch_bounds__(64) void fc_w4_strip_reduce_kernel(StripParams p) {
 }
 
 template <int LPR, int WAVES>
-hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
+hipError_t LaunchStripW(const StripParams& p, bool grouped, bool strided, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
   const dim3 block(WAVES * 64);
   if (p.batch_ids != nullptr) {  // batched weights: strips of 64 channels only
@@ -872,13 +876,19 @@ hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream
   // every thread exactly one chunk, K inside the work-group: the one-chunk form (strips of 64 channels)
   if constexpr (LPR == 8) {
     if (!zp && p.ksplit == 1 && p.chunks == WAVES * 64 / LPR && GetTuning().gemv_one_chunk != 0) {
-#define MLD_STRIP_1(G, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, false, MU, false, true>), grid, block, 0, stream, p)
-      if (grouped) { if (multi) MLD_STRIP_1(true, true); else MLD_STRIP_1(true, false); }
-      else         { if (multi) MLD_STRIP_1(false, true); else MLD_STRIP_1(false, false); }
+#define MLD_STRIP_1(G, MU, ST) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, false, MU, false, true, ST>), grid, block, 0, stream, p)
+      if (strided) {
+        if (grouped) { if (multi) MLD_STRIP_1(true, true, true); else MLD_STRIP_1(true, false, true); }
+        else         { if (multi) MLD_STRIP_1(false, true, true); else MLD_STRIP_1(false, false, true); }
+      } else {
+        if (grouped) { if (multi) MLD_STRIP_1(true, true, false); else MLD_STRIP_1(true, false, false); }
+        else         { if (multi) MLD_STRIP_1(false, true, false); else MLD_STRIP_1(false, false, false); }
+      }
 #undef MLD_STRIP_1
       return hipGetLastError();
     }
   }
+  if (strided) return hipErrorInvalidValue;  // (the launcher offers strided strips to the one-chunk form only)
 #define MLD_STRIP(G, Z, MU) hipLaunchKernelGGL((fc_w4_strip_kernel<LPR, WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
     if (zp) { if (multi) MLD_STRIP(true, true, true); else MLD_STRIP(true, true, false); }
@@ -892,13 +902,13 @@ hipError_t LaunchStripW(const StripParams& p, bool grouped, dim3 grid, hipStream
 }
 
 template <int LPR>
-hipError_t LaunchStripL(const StripParams& p, int waves, bool grouped, dim3 grid, hipStream_t stream) {
+hipError_t LaunchStripL(const StripParams& p, int waves, bool grouped, bool strided, dim3 grid, hipStream_t stream) {
   switch (waves) {
-    case 1: return LaunchStripW<LPR, 1>(p, grouped, grid, stream);
-    case 2: return LaunchStripW<LPR, 2>(p, grouped, grid, stream);
-    case 4: return LaunchStripW<LPR, 4>(p, grouped, grid, stream);
-    case 8: return LaunchStripW<LPR, 8>(p, grouped, grid, stream);
-    default: return LaunchStripW<LPR, 16>(p, grouped, grid, stream);
+    case 1: return LaunchStripW<LPR, 1>(p, grouped, strided, grid, stream);
+    case 2: return LaunchStripW<LPR, 2>(p, grouped, strided, grid, stream);
+    case 4: return LaunchStripW<LPR, 4>(p, grouped, strided, grid, stream);
+    case 8: return LaunchStripW<LPR, 8>(p, grouped, strided, grid, stream);
+    default: return LaunchStripW<LPR, 16>(p, grouped, strided, grid, stream);
   }
 }
 
@@ -920,9 +930,33 @@ bool StripKernelServes(const FcArgs* args, int count) {
   return true;
 }
 
-hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grouped, hipStream_t stream) {
+// One output group over all slices (the reference's own layout) is served by the one-chunk form of
+// the strip kernel, with strided rows: one token, whole strips of 64 channels, every thread exactly
+// one chunk (K = 256 ... 4096 channels), no zero points, strips enough to keep K inside the
+// work-groups.
+bool StridedStripKernelServes(const FcArgs* args, int count) {
   const Tuning& tune = GetTuning();
-  const int group = EffectiveGroup(args[0].group, p.seg[0].ns);  // 16, 8 or 4 slices: 8, 4 or 2 lanes per row
+  if (tune.gemv_fast == 0 || tune.gemv_one_chunk == 0 || tune.gemv_ksplit > 0 || tune.gemv_waves > 0) return false;
+  if (args[0].params != nullptr || args[0].batch_ids != nullptr || args[0].m != 1) return false;
+  const int ks = DivUp(args[0].k, 4);
+  if (args[0].k % 32 != 0) return false;
+  const int chunks = ks / 8;
+  if (chunks < 8 || chunks > 128 || (chunks & (chunks - 1)) != 0) return false;
+  int strips = 0;
+  for (int i = 0; i < count; ++i) {
+    const int ns = DivUp(args[i].n, 4);
+    if (args[i].n % 64 != 0 || EffectiveGroup(args[i].group, ns) != ns || args[i].has_zero_point) return false;
+    if ((size_t)ks * ns * 8 >= ((size_t)1 << 32) || ns / 2 >= (1 << 24)) return false;  // 32-bit lane offsets
+    strips += ns / 16;
+  }
+  return strips >= 128;
+}
+
+hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grouped, hipStream_t stream,
+                       bool strided = false) {
+  const Tuning& tune = GetTuning();
+  // 16, 8 or 4 slices: 8, 4 or 2 lanes per row (strided: strips of 16 slices out of the one group)
+  const int group = strided ? kNativeGroup : EffectiveGroup(args[0].group, p.seg[0].ns);
   const int lpr = group / 2;
   int strips = 0;
   for (int i = 0; i < count; ++i) {
@@ -984,13 +1018,13 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   sp.magic_hi = p.magic_hi;
   for (int i = 0; i < kMaxSegments; ++i) {
     const StreamSegment& g = p.seg[i];
-    sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, g.strip_end, g.n_off, 0};
+    sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, g.strip_end, g.n_off, g.row_u4};
   }
   hipError_t e;
   switch (lpr) {
-    case 2: e = LaunchStripL<2>(sp, waves, grouped, grid, stream); break;
-    case 4: e = LaunchStripL<4>(sp, waves, grouped, grid, stream); break;
-    default: e = LaunchStripL<8>(sp, waves, grouped, grid, stream); break;
+    case 2: e = LaunchStripL<2>(sp, waves, grouped, strided, grid, stream); break;
+    case 4: e = LaunchStripL<4>(sp, waves, grouped, strided, grid, stream); break;
+    default: e = LaunchStripL<8>(sp, waves, grouped, strided, grid, stream); break;
   }
   if (e != hipSuccess || ksplit == 1) return e;
   if (grouped)
@@ -1321,6 +1355,10 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   if (StripKernelServes(args, count)) {
     if (kernel_name) *kernel_name = "fc_w4_strip_kernel";
     return LaunchStrip(p, args, count, grouped, stream);
+  }
+  if (StridedStripKernelServes(args, count)) {
+    if (kernel_name) *kernel_name = "fc_w4_strip_kernel";
+    return LaunchStrip(p, args, count, grouped, stream, true);
   }
 
   // Launch shape.  Aim: every thread owns one chunk (all loads in flight at once) and the

@@ -299,12 +299,48 @@ def test_int8_math_bit_exact(oracle, bits, m, k, n):
     assert np.array_equal(got, ref)
     # 1..4 tokens stream (uint4 rows with an odd number of slices keep the tiled kernel)
     streams = m <= 4 and (bits == 8 or ((n + 3) // 4) % 2 == 0)
-    assert op.kernel_name == ("fc_i8math_stream_kernel" if streams else "fc_int8_math_kernel"), op.kernel_name
+    # one token over at least 128 whole strips of 64 channels and whole chunks of K: the strip form
+    strips = bits == 4 and m == 1 and n % 64 == 0 and n // 64 >= 128 and k % 32 == 0
+    assert op.kernel_name == ("fc_i8math_strip_kernel" if strips else "fc_i8math_stream_kernel" if streams
+                              else "fc_int8_math_kernel"), op.kernel_name
     if m * k * n <= 1 << 24:  # the restatement reads the reference's layout
         ns = (n + 3) // 4
         packed_ref = (oracle.int8_as_uint4 if bits == 4 else oracle.int8_as_uint8)(w, oracle.LAYOUT_I4O4, ns)
         mimic = oracle.from_slices(oracle.fc_int8_kernel(oracle.to_slices(src), packed_ref, m, k, n, bits), n)
         assert np.array_equal(got, mimic)
+
+
+@pytest.mark.parametrize("reference_layout", [False, True])
+@pytest.mark.parametrize("k,n", [(4096, 14336), (1024, 8192), (2048, 8192), (3072, 8256), (8192, 8192), (32, 8192),
+                                 (544, 16384)])
+def test_int8_math_strip_kernel(oracle, k, n, reference_layout):
+    """One token of int8 activations over uint4 weights in whole strips of 64 channels: one chunk per
+    thread at K = 1024 / 2048 / 4096, the chunk loop otherwise (also with idle rows), output groups of
+    16 slices and the reference's one group; exact."""
+    torch = torch_cuda()
+    rng = np.random.default_rng(k + n)
+    w = rng.integers(-8, 8, size=(n, k), dtype=np.int8)
+    src = rng.integers(-128, 128, size=(1, k), dtype=np.int8)
+    desc = M.fc_int4_weights_desc(n, k, reference=reference_layout)
+    packed = M.rearrange_int8_as_uint4(w, desc)
+    act = torch.from_numpy(W.to_slices(src)).cuda()
+    wt = torch.from_numpy(packed).cuda()
+    out = torch.zeros((n // 4, 1, 4), dtype=torch.int32, device="cuda")
+    op = M.fc_create(M.PRECISION_F32, M.INT8, M.INT32, n, k, desc, max_tokens=1)
+    op.bind([act, wt], [out])
+    op.set_shape(1, 1, 1)
+    print("int8 math strips", k, n, reference_layout, desc.output_group_size, flush=True)
+    op.launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert op.kernel_name == "fc_i8math_strip_kernel", op.kernel_name
+    got = W.from_slices(out.cpu().numpy(), n)
+    assert np.array_equal(got, oracle.fc_reference_i8(src, w))
+    with M.tuning(gemv_one_chunk=0):
+        out.zero_()
+        op.launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert op.kernel_name == "fc_i8math_stream_kernel", op.kernel_name
+        assert np.array_equal(W.from_slices(out.cpu().numpy(), n), got)
 
 
 @pytest.mark.parametrize("m,k,n,groups,bias", [(1, 2048, 16384, 64, False), (2, 2048, 16384, 64, True),
@@ -494,6 +530,52 @@ def test_strip_kernel_group_sizes(oracle, group, k, n, groups, zp, bias):
         if k // 32 >= ksplit:
             with M.tuning(fc_group=group, gemv_ksplit=ksplit):
                 run_case(oracle, case, "fc_w4_strip_kernel", layouts=[False])
+
+
+@pytest.mark.parametrize("reference_layout", [False, True])
+@pytest.mark.parametrize("k,n,groups,bias", [(4096, 14336, 1, False), (2048, 16384, 64, True), (256, 8192, 1, True),
+                                             (1024, 8192, 8, False), (512, 24576, 1, False)])
+def test_strip_kernel_one_chunk_forms(oracle, k, n, groups, bias, reference_layout):
+    """One token over at least 128 strips of 64 channels with K = 256 ... 4096: every thread owns exactly one
+    chunk, and the strip kernel runs without a chunk loop, over contiguous strips (output groups of 16
+    slices) and over strided ones (the reference's one output group).  With the form switched off the
+    older kernels serve the same case; both are held to the oracle."""
+    case = W.make_fc_case(seed=k + n, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=bias)
+    got = run_case(oracle, case, "fc_w4_strip_kernel", layouts=[reference_layout])
+    other = run_case(oracle, case, "fc_w4_strip_kernel" if not reference_layout else "fc_w4_stream_kernel",
+                     tune=dict(gemv_one_chunk=0), layouts=[reference_layout])
+    rms = float(np.sqrt(np.mean(np.square(other.astype(np.float64)))))
+    assert np.abs(got.astype(np.float64) - other).max() <= 4e-3 * rms  # (another order of the K sum: fp16 ulps)
+
+
+@pytest.mark.parametrize("reference_layout", [False, True])
+def test_strip_kernel_fused_launch_one_chunk_forms(oracle, reference_layout):
+    """Two and three matrices that read one source tensor in one launch (one list of strips): the
+    one-chunk forms give the bytes of the single launches, in both layouts."""
+    torch = torch_cuda()
+    shapes = [(1024, 8192, 32, True), (1024, 8256, 32, False), (1024, 8192, 32, False)]
+    devs = []
+    for i, (k, n, groups, bias) in enumerate(shapes):
+        case = W.make_fc_case(seed=90 + i, m=1, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups, with_bias=bias)
+        devs.append(W.FcDevice(case, reference_layout=reference_layout))
+    for d in devs[1:]:  # the same source tensor for all
+        d.op.bind([devs[0].act, d.weights, d.scale] + ([d.bias] if d.case["bias"] is not None else []), [d.out])
+        d.case["act"] = devs[0].case["act"]
+    single = []
+    for d in devs:
+        d.run()
+        assert d.op.kernel_name == "fc_w4_strip_kernel", d.op.kernel_name
+        single.append(d.result())
+        check_fp(single[-1], textbook(d.case), d.case, "single launch")
+        d.out.zero_()
+    for count in (2, 3):
+        print("fused one-chunk launch of", count, "matrices, reference layout" if reference_layout else "", flush=True)
+        M.fc_launch_fused([d.op for d in devs[:count]], torch.cuda.current_stream().cuda_stream)
+        for d, want in zip(devs[:count], single):
+            assert d.op.kernel_name == "fc_w4_strip_kernel", d.op.kernel_name
+            assert np.array_equal(d.result(), want)
+            d.out.zero_()
 
 
 def test_split_k_launches_repeat_bit_for_bit(oracle):
