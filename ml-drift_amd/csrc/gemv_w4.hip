@@ -597,6 +597,21 @@ typedef uint32_t u32x2s __attribute__((ext_vector_type(2)));
 // of the 8 channel sums of every lane; the result of channel (lane % LPR) * 8 + (lane / 8) % 8 is
 // returned in this lane (lanes that differ only in the bits between LPR and 8 hold the same
 // sums).  All 64 lanes must be active.
+// v + the value of the lane that differs in one bit of the lane number, as data-parallel moves
+// inside the rows of 16 lanes (no trip through the LDS crossbar): bits 0 and 1 are quad
+// permutations, bit 2 a shift by 4 lanes in either direction, each for the banks it is valid in.
+__device__ __forceinline__ float AddLaneXor1(float v) {
+  return v + __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float AddLaneXor2(float v) {
+  return v + __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float AddLaneXor4(float v) {
+  const uint32_t up = __builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+  const uint32_t both = __builtin_amdgcn_update_dpp(up, __float_as_uint(v), 0x114 /* row_shr:4 */, 0xf, 0xA, false);
+  return v + __uint_as_float(both);
+}
+
 template <int LPR>
 __device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
   float s4[4], s2[2];
@@ -615,9 +630,9 @@ __device__ __forceinline__ float WaveStripSum(const float acc[8], int lane) {
     s2[i] += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s2[i]), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
   float v = (lane & 8) ? s2[1] : s2[0];
   // narrower rows: the lanes 4 (and 2) apart hold further rows of the same channels
-  if (LPR <= 4) v += __shfl_xor(v, 4, 64);
-  if (LPR <= 2) v += __shfl_xor(v, 2, 64);
-  if (LPR <= 1) v += __shfl_xor(v, 1, 64);
+  if (LPR <= 4) v = AddLaneXor4(v);
+  if (LPR <= 2) v = AddLaneXor2(v);
+  if (LPR <= 1) v = AddLaneXor1(v);
   return v;
 }
 
@@ -701,6 +716,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_kernel(StripParams p) 
   struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
   const u32x4* weights = sg.weights;
   const u32x4* astrip = reinterpret_cast<const u32x4*>(p.act);  // chunk c: 4 uint4 (8 slices x 4 halfs)
+  // (input-only operands: the pointers keep their address space, and their scalar loads join the
+  // first batch instead of being issued where the pointer is first used)
+  asm volatile("" : : "s"(p.act), "s"(sg.dst), "s"(sg.bias), "s"(sg.scale));
   int ks = p.ks, group_chunks = p.group_chunks, n_pad = sg.n_pad;
   asm volatile("" : "+s"(up.mask_lo), "+s"(up.mask_hi), "+s"(ks), "+s"(group_chunks), "+s"(n_pad));
   // BATCHED: this row's matrix (an id outside the batch is clamped into it) and its source row (one
@@ -1045,9 +1063,7 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
 // K reduction: the 8 channel sums of the 64 lanes by the register exchanges of the strip kernel
 // (all lanes hold rows of the same 8 channels), across waves through LDS in wave order.
 // ------------------------------------------------------------------------------------------
-// ONE: K is exactly 8 rows per thread (the shape the launcher sizes the work-group for): one pass
-// without bounds, the lane's byte offsets are 32-bit values over scalar bases.
-template <int WAVES, bool GROUPED, bool ZP, bool MULTI, bool ONE = false>
+template <int WAVES, bool GROUPED, bool ZP, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   constexpr int T = WAVES * 64;
   __shared__ float red[WAVES][8];
@@ -1061,6 +1077,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   if (strip < (int)(gridDim.x & ~63u)) strip = (strip & ~63) + ((strip & 7) << 3) + ((strip >> 3) & 7);
   const StripSegment sg = SelectSegment<MULTI>(p, strip);
   struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
+  asm volatile("" : : "s"(p.act), "s"(sg.dst), "s"(sg.bias), "s"(sg.scale));  // (fetched with the first batch of scalar loads)
   const u32x4* wstrip = sg.weights + (size_t)strip * p.ks;  // row r of the strip: K-slice r, 2 slices x 8 bytes
   const u32x2* act2 = reinterpret_cast<const u32x2*>(p.act);
   const __half* scale = sg.scale;
@@ -1074,30 +1091,11 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   for (int o = 0; o < 8; ++o) acc[o] = 0.0f;
   u32x4 zv_lin = {0u, 0u, 0u, 0u};
   if (ZP && !GROUPED) zv_lin = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * 8);
-
-  for (int r0 = tid; ONE ? r0 == tid : r0 < ks; r0 += 8 * T) {
+  for (int r0 = tid; r0 < ks; r0 += 8 * T) {
     u32x4 w[8], sv[8], zv[8];
     u32x2 a[8];
     // small loads that come from cache first, then the eight weight loads back to back
-    if (ONE) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        a[j] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const char*>(p.act) + (uint32_t)(tid + T * j) * 8u);
-      if (GROUPED) {
-        // a scale group has at most T K-slices (the launcher checks), so row tid + T * j lies
-        // (T * j) >> group_shift groups behind row tid: one lane offset over 8 scalar bases
-        const uint32_t so = (__umul24((uint32_t)tid >> group_shift, (uint32_t)n_pad) + (uint32_t)strip * 8u) * 2u;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const size_t sj = (size_t)((uint32_t)((T * j) >> group_shift) * (uint32_t)n_pad) * 2u;
-          sv[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(scale) + sj + so);
-          if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(zero_point) + sj + so);
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        w[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wstrip) + (uint32_t)(tid + T * j) * 16u));
-    } else {
+    {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int r = r0 + T * j;
@@ -1180,20 +1178,6 @@ template <int WAVES>
 hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
   const dim3 block(WAVES * 64);
-  // exactly 8 rows per thread, scale tensors within 32-bit byte offsets: the one-pass form
-  if (!zp && p.ks == 8 * WAVES * 64 && GetTuning().gemv_one_chunk != 0) {
-    bool fits = true;
-    for (int i = 0; i < p.segments; ++i)
-      fits = fits && (!grouped || ((size_t)(p.ks >> p.group_chunks) * p.seg[i].n_pad < ((size_t)1 << 24) &&
-                                   p.seg[i].n_pad < (1 << 24) && (1 << p.group_chunks) <= WAVES * 64));
-    if (fits) {
-#define MLD_ROWS_1(G, MU) hipLaunchKernelGGL((fc_w4_rows_kernel<WAVES, G, false, MU, true>), grid, block, 0, stream, p)
-      if (grouped) { if (multi) MLD_ROWS_1(true, true); else MLD_ROWS_1(true, false); }
-      else         { if (multi) MLD_ROWS_1(false, true); else MLD_ROWS_1(false, false); }
-#undef MLD_ROWS_1
-      return hipGetLastError();
-    }
-  }
 #define MLD_ROWS(G, Z, MU) hipLaunchKernelGGL((fc_w4_rows_kernel<WAVES, G, Z, MU>), grid, block, 0, stream, p)
   if (grouped) {
     if (zp) { if (multi) MLD_ROWS(true, true, true); else MLD_ROWS(true, true, false); }

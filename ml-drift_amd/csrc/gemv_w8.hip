@@ -339,15 +339,22 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_rows_kernel(W8Params p) {
   // Every lane holds sums of the same 4 channels.  Two exchange steps halve what a lane carries
   // (lanes 32.. keep channels 2 and 3, then lanes 16.. of each half the odd one), four more add
   // the 16 lanes that are left with the same channel: lane l ends with channel 2 * (l / 32) + (l / 16) % 2.
-  // (Named scalars and selects between them: an index into `acc` that depends on the lane would
-  // move the array out of registers.)
-  const float c0 = acc[0], c1 = acc[1], c2 = acc[2], c3 = acc[3];
-  const bool up32 = (lane & 32) != 0, up16 = (lane & 16) != 0;
-  const float x0 = (up32 ? c2 : c0) + __shfl_xor(up32 ? c0 : c2, 32, 64);
-  const float x1 = (up32 ? c3 : c1) + __shfl_xor(up32 ? c1 : c3, 32, 64);
-  float v = (up16 ? x1 : x0) + __shfl_xor(up16 ? x0 : x1, 16, 64);
-#pragma unroll
-  for (int off = 8; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  // (register exchanges and data-parallel moves: nothing goes through the LDS crossbar)
+  typedef unsigned u32x2s __attribute__((ext_vector_type(2)));
+  const u32x2s e0 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[0]), __float_as_uint(acc[2]), false, false);
+  const u32x2s e1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[1]), __float_as_uint(acc[3]), false, false);
+  const float x0 = __uint_as_float(e0[0]) + __uint_as_float(e0[1]);
+  const float x1 = __uint_as_float(e1[0]) + __uint_as_float(e1[1]);
+  const u32x2s e2 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x0), __float_as_uint(x1), false, false);
+  float v = __uint_as_float(e2[0]) + __uint_as_float(e2[1]);
+  v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+  {
+    const uint32_t up = __builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+    const uint32_t both = __builtin_amdgcn_update_dpp(up, __float_as_uint(v), 0x114 /* row_shr:4 */, 0xf, 0xA, false);
+    v += __uint_as_float(both);
+  }
+  v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, false));
+  v += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, false));
   const int ch = 2 * (lane >> 5) + ((lane >> 4) & 1);
   if (WAVES > 1) {
     if ((lane & 15) == 0) red[wave][ch] = v;
