@@ -54,6 +54,7 @@ struct W4Segment {
   int group;  // slices per output group of the packed weights (ns: one group, the rows span all of N)
   int tile_end;
   uint32_t a_bytes, s_bytes;
+  int group_shift;  // log2(group) when it is a power of two, else -1
 };
 
 struct GemmParams {
@@ -92,6 +93,13 @@ struct GemmParams {
   // pg_params[pg_offset + pg_groups + g] of the one source row.  pg_groups = 0: not set.
   const int32_t* pg_params;
   int pg_offset, pg_groups, pg_max;
+  // fp16 path: launch geometry worked out on the host, so that no work-group divides by a run-time
+  // number in front of its first load: token tiles of the launch, the XCD rectangle (token tiles x
+  // channel tiles), log2(xcd_m), ceil(2^32 / rect_m) (0 when rect_m = 1), and the 16-channel steps
+  // of one wave's share of K (a multiple of the prefetch depth).
+  int geo_tiles_m, geo_rect_m, geo_rect_n, geo_xm_shift;
+  uint32_t geo_rect_m_magic;
+  int geo_per_wave;
 };
 
 __device__ __forceinline__ half2_t AsHalf2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
@@ -569,6 +577,24 @@ __device__ __forceinline__ void SwapRegisters(u32x4& a, u32x4& b) {
 // activations, so every activation tile is fetched from L2 once for 256 channels, and there are
 // half as many work-groups and reduction rounds; for launches with many tiles.
 enum { kModePlain = 0, kModeGated = 1, kModeDual = 2 };
+// Entry `index` of the launch's matrix list, by value.  Every field of every entry sits at a fixed
+// offset of the kernel arguments, so all of them are fetched by one batch of scalar loads and
+// chosen with scalar selects; indexing the list with a run-time number makes the entry's loads
+// wait for the round trip that produces the number.
+template <bool DYNAMIC>
+__device__ __forceinline__ W4Segment PickSegment(const GemmParams& p, int index) {
+  W4Segment sg = p.seg[0];
+  if (DYNAMIC) {
+    const W4Segment s1 = p.seg[1], s2 = p.seg[2];
+#define MLD_PICK(f) sg.f = index == 2 ? s2.f : (index == 1 ? s1.f : sg.f)
+    MLD_PICK(w4); MLD_PICK(scale); MLD_PICK(zp); MLD_PICK(bias); MLD_PICK(dst); MLD_PICK(partial);
+    MLD_PICK(n); MLD_PICK(ns); MLD_PICK(group); MLD_PICK(tile_end); MLD_PICK(a_bytes); MLD_PICK(s_bytes);
+    MLD_PICK(group_shift);
+#undef MLD_PICK
+  }
+  return sg;
+}
+
 template <int WB, int FM, int U, int WAVES, bool ZP, bool PAIR, bool MULTI, int MODE = kModePlain>
 __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParams p) {
   constexpr bool GATED = MODE == kModeGated, DUAL = MODE == kModeDual;
@@ -584,6 +610,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   constexpr int RPH = WAVES == 4 ? 16 : 8;  // accumulator registers (x 4 MFMAs) per phase
   __shared__ float4 red[2][WAVES][RPH][64];
 
+  // One batch of scalar loads for what the prologue reads.  (Left alone, the compiler fetches
+  // every argument where it is first used: seven scalar round trips, one behind the other, in
+  // front of the first operand load.  Input-only operands keep the pointers' address spaces.)
+  asm volatile("" : : "s"(p.m), "s"(p.ks), "s"(p.ksplit), "s"(p.xcd_m), "s"(p.pg_groups), "s"(p.group_shift),
+               "s"(p.b_bytes), "s"(p.act), "s"(p.magic_lo), "s"(p.magic_hi), "s"(p.mask_lo), "s"(p.mask_hi), "s"(p.segments),
+               "s"(p.geo_tiles_m), "s"(p.geo_rect_m), "s"(p.geo_rect_n), "s"(p.geo_xm_shift), "s"(p.geo_rect_m_magic),
+               "s"(p.geo_per_wave));
+  asm volatile("" : : "s"(p.seg[0].w4), "s"(p.seg[0].scale), "s"(p.seg[0].ns), "s"(p.seg[0].group), "s"(p.seg[0].tile_end),
+               "s"(p.seg[0].a_bytes), "s"(p.seg[0].s_bytes), "s"(p.seg[0].dst), "s"(p.seg[0].bias), "s"(p.seg[0].partial));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -598,7 +633,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const int tiles_n = DUAL ? (tiles_n_all + 1) / 2 : tiles_n_all;        // channel tiles of the grid
   // Packed groups: this work-group's matrix and the run of tokens it multiplies (else: all tokens).
   int m_lo = 0, m_hi = p.m, pg_e = 0;
-  int tiles_m = (p.m + BM - 1) / BM;
+  const int tiles_m = p.geo_tiles_m;  // (packed groups: the tiles of the largest group)
   if (p.pg_groups > 0) {
     pg_e = blockIdx.z;
     const int size = min(p.pg_params[p.pg_offset + pg_e], p.pg_max);
@@ -606,13 +641,15 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
     if (off < 0) return;
     m_lo = off;
     m_hi = min(off + size, p.m);
-    tiles_m = (p.pg_max + BM - 1) / BM;
   }
   const int xcd = blockIdx.x % 8, local = blockIdx.x / 8;
-  const int xm = p.xcd_m, xn = 8 / xm;
-  const int rect_m = (tiles_m + xm - 1) / xm, rect_n = (tiles_n + xn - 1) / xn;
-  const int tm = (xcd % xm) * rect_m + local % rect_m;
-  const int tn_grid = (xcd / xm) * rect_n + local / rect_m;
+  const int xm = p.xcd_m;
+  const int rect_m = p.geo_rect_m, rect_n = p.geo_rect_n;
+  // local / rect_m by the host's reciprocal (exact: local and rect_m are below 2^16)
+  const int local_n = rect_m == 1 ? local : (int)__umulhi((uint32_t)local, p.geo_rect_m_magic);
+  const int local_m = local - local_n * rect_m;
+  const int tm = (xcd & (xm - 1)) * rect_m + local_m;
+  const int tn_grid = (xcd >> p.geo_xm_shift) * rect_n + local_n;
   if (tm >= tiles_m || tn_grid >= tiles_n) return;
   // channel tile of the launch -> matrix of the launch (return value) and tile inside it
   auto locate = [&](int& tile) {
@@ -629,7 +666,7 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   const bool tile_ok = !DUAL || tn < tiles_n_all;  // the last pair of an odd count has one tile
   if (!tile_ok) tn = 0;
   const int si = locate(tn);
-  const W4Segment& sg = p.seg[GATED ? half : (MULTI ? si : 0)];
+  const W4Segment sg = PickSegment<GATED || MULTI>(p, GATED ? half : (MULTI ? si : 0));
   const int slice0 = tn * (BN / 4);  // first output slice of the tile
   const int m0 = m_lo + tm * BM;
   if (m0 >= m_hi) return;  // (packed groups: a tile beyond the group's size; the whole work-group leaves)
@@ -640,9 +677,9 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // activations end where the wave's share of K ends, so the prefetches that run past it (and
   // past K itself) read zeros without a test in the loop; a lane without an output slice or
   // a token gets an offset beyond every buffer.
-  const int steps_total = (p.k + 15) / 16;
-  const int shares = KW * p.ksplit;  // blockIdx.y selects the work-group's part of K
-  const int per_wave = ((steps_total + shares - 1) / shares + U - 1) / U * U;  // multiple of U
+  // (blockIdx.y selects the work-group's part of K; per_wave: the steps of one of the KW * ksplit
+  // shares, a multiple of U)
+  const int per_wave = p.geo_per_wave;
   const int t_begin = __builtin_amdgcn_readfirstlane(((int)blockIdx.y * KW + wave % KW) * per_wave);
   // Weights with output groups: the K-slice rows of a group lie one after the other (row = the
   // group's slices), the groups one after the other.  With one group the buffer ends, for this
@@ -688,10 +725,12 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   // Only the per-lane offset takes part in the range check of a buffer load, so the whole
   // address lives there.
   const uint32_t step_w = 4u * row_w, step_x = 4u * row_x;
+  // (the slice's output group and its place inside it: a shift where the group size allows)
+  const uint32_t nsi_group = sg.group_shift >= 0 ? (uint32_t)nsi >> sg.group_shift : (uint32_t)(nsi / sg.group);
+  const uint32_t nsi_in_group = (uint32_t)nsi - nsi_group * (uint32_t)sg.group;
   const uint32_t col_w = one_group ? (uint32_t)nsi * kBlk
-                                   : (((uint32_t)(nsi / sg.group) * (uint32_t)max(p.pg_groups, 1) + (uint32_t)pg_e) * (uint32_t)p.ks *
-                                          (uint32_t)sg.group +
-                                      (uint32_t)(nsi % sg.group)) * kBlk;
+                                   : ((nsi_group * (uint32_t)max(p.pg_groups, 1) + (uint32_t)pg_e) * (uint32_t)p.ks * (uint32_t)sg.group +
+                                      nsi_in_group) * kBlk;
   uint32_t vw0 = n_ok ? ((uint32_t)t_begin * 4u + (uint32_t)g2 * 2u) * row_w + col_w : kOob;
   const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
   // token of this lane in MFMA token block fm
@@ -963,8 +1002,8 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_mfma_direct_kernel(GemmParam
   if (!tile_b_ok) tile_b = 0;
   int tile_a = DUAL ? 2 * tn_grid : tn;
   const int seg_a = DUAL ? locate(tile_a) : si, seg_b = DUAL ? locate(tile_b) : 0;
-  const W4Segment& sga = p.seg[GATED ? 0 : (MULTI ? seg_a : 0)];
-  const W4Segment& sgb = p.seg[GATED ? 1 : (MULTI ? seg_b : 0)];
+  const W4Segment sga = PickSegment<!GATED && MULTI>(p, GATED ? 0 : (MULTI ? seg_a : 0));
+  const W4Segment sgb = PickSegment<GATED || MULTI>(p, GATED ? 1 : (MULTI ? seg_b : 0));
   const int slice0_a = DUAL ? tile_a * (BN / 4) : slice0, slice0_b = tile_b * (BN / 4);
   // one slice of four channels of one token: the K-split partial sums, or the fp16 result
   auto store = [&](const W4Segment& sgx, int slice, int mi, const float4& sum) {
@@ -1251,6 +1290,9 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     sg.group = EffectiveGroup(args[i].group, sg.ns);
     if (sg.ns % sg.group != 0) return hipErrorInvalidValue;  // whole groups only
     if (args[i].weight_bits != a.weight_bits) return hipErrorInvalidValue;
+    sg.group_shift = -1;
+    for (int sh = 0; sh < 30; ++sh)
+      if ((1 << sh) == sg.group) sg.group_shift = sh;
     sg.a_bytes = (uint32_t)((size_t)p.ks * sg.ns * (a.weight_bits == 8 ? 16 : 8));
     sg.s_bytes = (uint32_t)((size_t)p.groups * sg.ns * 8 * (packed ? a.weights_batch : 1));
     if (gated) {
@@ -1268,6 +1310,19 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     *kernel_name = gated ? (a.weight_bits == 8 ? "fc_w8_gated_mfma_gemm_kernel" : "fc_w4_gated_mfma_gemm_kernel")
                          : (a.weight_bits == 8 ? "fc_w8_mfma_gemm_kernel" : "fc_w4_mfma_gemm_kernel");
   const Tuning& tune = GetTuning();
+  // the geometry the work-groups would otherwise divide out: waves = waves of the work-group that
+  // share one tile's K (all of them, or half in the gated and two-tile modes)
+  auto set_geometry = [&p](int tiles_m, int tiles_n_grid, int fm, bool halves) {
+    const int xn = 8 / p.xcd_m;
+    p.geo_tiles_m = tiles_m;
+    p.geo_rect_m = DivUp(tiles_m, p.xcd_m);
+    p.geo_rect_n = DivUp(tiles_n_grid, xn);
+    p.geo_xm_shift = p.xcd_m == 8 ? 3 : (p.xcd_m == 4 ? 2 : (p.xcd_m == 2 ? 1 : 0));
+    p.geo_rect_m_magic = p.geo_rect_m > 1 ? (uint32_t)((((uint64_t)1 << 32) + p.geo_rect_m - 1) / p.geo_rect_m) : 0u;
+    const int waves = fm == 4 ? 4 : 8, kw = halves ? waves / 2 : waves, prefetch = 4;
+    const int shares = kw * p.ksplit, steps_total = DivUp(p.k, 16);
+    p.geo_per_wave = DivUp(DivUp(steps_total, shares), prefetch) * prefetch;
+  };
   if (packed) {
     p.pg_params = a.params;
     p.pg_offset = a.packed_params_offset;
@@ -1282,6 +1337,8 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     p.xcd_m = 1;  // few token tiles per matrix: the XCDs share the channel tiles
     if (tune.gemm_xcd_m == 1 || tune.gemm_xcd_m == 2 || tune.gemm_xcd_m == 4 || tune.gemm_xcd_m == 8) p.xcd_m = tune.gemm_xcd_m;
     const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), 1, a.weights_batch);
+    if (grid.x / 8 >= (1u << 16)) return hipErrorInvalidValue;  // (the reciprocal of rect_m is exact below 2^16)
+    set_geometry(tiles_m, tiles_n, fm, false);
     const bool zp = p.seg[0].zp != nullptr;
     if (fm == 4)
       LaunchDirect<4, 4, 4, false, false>(a.weight_bits, zp, grid, stream, p);
@@ -1317,6 +1374,8 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
   if (tune.gemm_xcd_m > 0) p.xcd_m = tune.gemm_xcd_m;
   if (p.xcd_m != 1 && p.xcd_m != 2 && p.xcd_m != 4 && p.xcd_m != 8) p.xcd_m = 8;
   const dim3 grid(8 * DivUp(tiles_m, p.xcd_m) * DivUp(tiles_n, 8 / p.xcd_m), p.ksplit);
+  if (grid.x / 8 >= (1u << 16)) return hipErrorInvalidValue;  // (the reciprocal of rect_m is exact below 2^16)
+  set_geometry(tiles_m, tiles_n, fm, gated || p.dual);
   const bool zp = p.seg[0].zp != nullptr;
   if (fm == 4)
     LaunchDirect<4, 4, 4, true, true>(a.weight_bits, zp, grid, stream, p);
