@@ -231,6 +231,9 @@ __global__ __launch_bounds__(kI8Threads) void conv_int8_mfma_kernel(GemmParams p
   const LdsPtr lds = (LdsPtr)smem;
   const uint32_t lds_base = (uint32_t)(size_t)lds;
 
+  // (one batch of scalar loads for the arguments, those of the epilogue included)
+  asm volatile("" : : "s"(p.m), "s"(p.n), "s"(p.k), "s"(p.ns), "s"(p.k16), "s"(p.a_bytes), "s"(p.b_bytes), "s"(p.wi8), "s"(p.codes),
+               "s"(p.dst), "s"(p.bias), "s"(p.params), "s"(p.wsum), "s"(p.wscale), "s"(p.wzp));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1128,35 +1131,51 @@ void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
 // the bias.  One thread per (slice, token).
 __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) {
-  // items of all matrices of the launch, matrix after matrix
-  size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  // items of all matrices of the launch, matrix after matrix (the list entries by value: fixed
+  // argument offsets, one batch of scalar loads)
+  uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t m = (uint32_t)p.m;
+  const uint32_t items0 = (uint32_t)p.seg[0].ns * m, items1 = (uint32_t)p.seg[1].ns * m;
   int si = 0;
-  while (si < p.segments && idx >= (size_t)p.seg[si].ns * p.m) {
-    idx -= (size_t)p.seg[si].ns * p.m;
-    ++si;
+  if (p.segments > 1 && idx >= items0) {
+    idx -= items0;
+    si = 1;
+    if (p.segments > 2 && idx >= items1) {
+      idx -= items1;
+      si = 2;
+    }
   }
-  if (si >= p.segments) return;
-  const W4Segment& sg = p.seg[si];
-  const size_t items = (size_t)sg.ns * p.m;
-  const float4* part = reinterpret_cast<const float4*>(sg.partial);
-  float4 sum = part[idx];
-  for (int s = 1; s < p.ksplit; ++s) {
-    const float4 o = part[(size_t)s * items + idx];
-    sum.x += o.x;
-    sum.y += o.y;
-    sum.z += o.z;
-    sum.w += o.w;
+  const W4Segment sg = PickSegment<true>(p, si);
+  const uint32_t items = (uint32_t)sg.ns * m;
+  if (idx >= items) return;
+  const float4* part = reinterpret_cast<const float4*>(sg.partial) + idx;
+  // the shares are added in their order, four loads in flight at a time
+  float4 sum = part[0];
+  const int ksplit = p.ksplit;
+  for (int s0 = 1; s0 < ksplit; s0 += 4) {
+    float4 o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = part[(size_t)min(s0 + j, ksplit - 1) * items];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (s0 + j < ksplit) {
+        sum.x += o[j].x;
+        sum.y += o[j].y;
+        sum.z += o[j].z;
+        sum.w += o[j].w;
+      }
+    }
   }
   __half h[4] = {__float2half_rn(sum.x), __float2half_rn(sum.y), __float2half_rn(sum.z), __float2half_rn(sum.w)};
   if (sg.bias) {
-    const __half* bias = sg.bias + (idx / p.m) * 4;
+    const __half* bias = sg.bias + (idx / m) * 4;
 #pragma unroll
     for (int c = 0; c < 4; ++c) h[c] = __hadd(h[c], bias[c]);
   }
-  u32x2 o;
-  o[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
-  o[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
-  reinterpret_cast<u32x2*>(sg.dst)[idx] = o;
+  u32x2 o2;
+  o2[0] = (uint32_t)__half_as_ushort(h[0]) | ((uint32_t)__half_as_ushort(h[1]) << 16);
+  o2[1] = (uint32_t)__half_as_ushort(h[2]) | ((uint32_t)__half_as_ushort(h[3]) << 16);
+  reinterpret_cast<u32x2*>(sg.dst)[idx] = o2;
 }
 
 // Token tile of the int4 GEMM in blocks of 32 tokens.  64 tokens when that still yields a
