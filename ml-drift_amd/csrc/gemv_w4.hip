@@ -1174,6 +1174,168 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_kernel(StripParams p) {
   sg.dst[n_out] = h;
 }
 
+
+// The same kernel for 2..4 tokens (MT = 2 or 4 token slots, `m` of them live): a K-slice row of the
+// activations holds the tokens one after the other, every unpacked weight pair feeds MT dot
+// products, the MT x 8 sums of a lane are reduced token by token.  Up to 8 waves (the 1024-thread
+// shape would spill its MT x 8 accumulators and MT x 8 activation pairs).
+template <int WAVES, int MT, bool GROUPED, bool ZP, bool MULTI>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_rows_tokens_kernel(StripParams p, int m) {
+  constexpr int T = WAVES * 64;
+  __shared__ float red[WAVES][MT][8];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  int strip = blockIdx.x;
+  if (strip < (int)(gridDim.x & ~63u)) strip = (strip & ~63) + ((strip & 7) << 3) + ((strip >> 3) & 7);
+  const StripSegment sg = SelectSegment<MULTI>(p, strip);
+  struct { uint32_t mask_lo, mask_hi, magic_lo, magic_hi; } up = {p.mask_lo, p.mask_hi, p.magic_lo, p.magic_hi};
+  asm volatile("" : : "s"(p.act), "s"(sg.dst), "s"(sg.bias), "s"(sg.scale));  // (fetched with the first batch of scalar loads)
+  const u32x4* wstrip = sg.weights + (size_t)strip * p.ks;
+  const u32x2* act2 = reinterpret_cast<const u32x2*>(p.act);
+  const __half* scale = sg.scale;
+  const __half* zero_point = sg.zero_point;
+  const int ks = p.ks, n_pad = sg.n_pad;
+  const int group_shift = p.group_chunks;
+  const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+
+  float acc[MT][8], asum_all[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    asum_all[t] = 0.0f;
+#pragma unroll
+    for (int o = 0; o < 8; ++o) acc[t][o] = 0.0f;
+  }
+  u32x4 zv_lin = {0u, 0u, 0u, 0u};
+  if (ZP && !GROUPED) zv_lin = *reinterpret_cast<const u32x4*>(zero_point + (size_t)strip * 8);
+  for (int r0 = tid; r0 < ks; r0 += 8 * T) {
+    u32x4 w[8], sv[8], zv[8];
+    u32x2 a[8][MT];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int r = r0 + T * j;
+      const size_t base = (size_t)min(r, ks - 1) * m;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const u32x2 v = act2[base + min(t, m - 1)];
+        const bool live = r < ks && t < m;
+        a[j][t] = u32x2{live ? v[0] : 0u, live ? v[1] : 0u};
+      }
+    }
+    if (GROUPED) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const size_t so = (size_t)(min(r0 + T * j, ks - 1) >> group_shift) * n_pad + (size_t)strip * 8;
+        sv[j] = *reinterpret_cast<const u32x4*>(scale + so);
+        if (ZP) zv[j] = *reinterpret_cast<const u32x4*>(zero_point + so);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = __builtin_nontemporal_load(wstrip + min(r0 + T * j, ks - 1));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // the 8 outputs' pairs for inputs (0, 1) and for inputs (2, 3), unpacked once for all tokens
+      half2_t qa[8], qb[8];
+#pragma unroll
+      for (int h = 0; h < 4; h += 2) {
+        const uint32_t lo0 = w[j][h], hi0 = lo0 >> 8, lo1 = w[j][h + 1], hi1 = lo1 >> 8;
+        const int ob = 4 * (h >> 1);
+        qa[ob + 0] = AsHalf2(AndOr(lo0, up.mask_lo, up.magic_lo));
+        qa[ob + 1] = AsHalf2(AndOr(lo0, up.mask_hi, up.magic_hi));
+        qa[ob + 2] = AsHalf2(AndOr(hi0, up.mask_lo, up.magic_lo));
+        qa[ob + 3] = AsHalf2(AndOr(hi0, up.mask_hi, up.magic_hi));
+        qb[ob + 0] = AsHalf2(AndOr(lo1, up.mask_lo, up.magic_lo));
+        qb[ob + 1] = AsHalf2(AndOr(lo1, up.mask_hi, up.magic_hi));
+        qb[ob + 2] = AsHalf2(AndOr(hi1, up.mask_lo, up.magic_lo));
+        qb[ob + 3] = AsHalf2(AndOr(hi1, up.mask_hi, up.magic_hi));
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const half2_t a01 = AsHalf2(a[j][t][0]), a23 = AsHalf2(a[j][t][1]);
+        float asum = __builtin_amdgcn_fdot2(a01, ones, 0.0f, false);
+        asum = __builtin_amdgcn_fdot2(a23, ones, asum, false);
+        float tt[8];
+#pragma unroll
+        for (int o = 0; o < 8; ++o) {
+          tt[o] = __builtin_amdgcn_fdot2(qa[o], a01, 0.0f, false);
+          tt[o] = __builtin_amdgcn_fdot2(qb[o], a23, tt[o], false);
+        }
+        if (GROUPED) {
+#pragma unroll
+          for (int o = 0; o < 8; ++o) {
+            float centre = (o & 1) ? -72.0f : -1032.0f;
+            if (ZP) centre -= (float)AsHalf2(zv[j][o >> 1])[o & 1];
+            acc[t][o] = fmaf((float)AsHalf2(sv[j][o >> 1])[o & 1], fmaf(centre, asum, tt[o]), acc[t][o]);
+          }
+        } else {
+          asum_all[t] += asum;
+#pragma unroll
+          for (int o = 0; o < 8; ++o) acc[t][o] += tt[o];
+        }
+      }
+    }
+  }
+  const int ch = (lane >> 3) & 7;
+  float v[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (!GROUPED) {
+#pragma unroll
+      for (int o = 0; o < 8; ++o) {
+        float centre = (o & 1) ? -72.0f : -1032.0f;
+        if (ZP) centre -= (float)AsHalf2(zv_lin[o >> 1])[o & 1];
+        acc[t][o] = fmaf(centre, asum_all[t], acc[t][o]);
+      }
+    }
+    v[t] = WaveStripSum<1>(acc[t], lane);
+  }
+  if (WAVES > 1) {
+    if ((lane & 7) == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) red[wave][t][ch] = v[t];
+    }
+    __syncthreads();
+    if (tid >= 64) return;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      v[t] = 0.0f;
+#pragma unroll
+      for (int q = 0; q < WAVES; ++q) v[t] += red[q][t][ch];
+    }
+  }
+  if ((lane & 7) != 0) return;
+  const int n_out = strip * 8 + ch;
+  const float out_scale = GROUPED ? 1.0f : __half2float(scale[n_out]);
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (t >= m) break;
+    __half h = __float2half_rn(GROUPED ? v[t] : v[t] * out_scale);
+    if (sg.bias) h = __hadd(h, sg.bias[n_out]);
+    sg.dst[((size_t)(n_out >> 2) * m + t) * 4 + (n_out & 3)] = h;
+  }
+}
+
+template <int WAVES, int MT>
+hipError_t LaunchRowsTokensW(const StripParams& p, int m, bool grouped, dim3 grid, hipStream_t stream) {
+  const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
+  const dim3 block(WAVES * 64);
+#define MLD_ROWS_T(G, Z, MU) hipLaunchKernelGGL((fc_w4_rows_tokens_kernel<WAVES, MT, G, Z, MU>), grid, block, 0, stream, p, m)
+  if (grouped) {
+    if (zp) { if (multi) MLD_ROWS_T(true, true, true); else MLD_ROWS_T(true, true, false); }
+    else    { if (multi) MLD_ROWS_T(true, false, true); else MLD_ROWS_T(true, false, false); }
+  } else {
+    if (zp) { if (multi) MLD_ROWS_T(false, true, true); else MLD_ROWS_T(false, true, false); }
+    else    { if (multi) MLD_ROWS_T(false, false, true); else MLD_ROWS_T(false, false, false); }
+  }
+#undef MLD_ROWS_T
+  return hipGetLastError();
+}
+template <int WAVES>
+hipError_t LaunchRowsTokens(const StripParams& p, int m, bool grouped, dim3 grid, hipStream_t stream) {
+  return m <= 2 ? LaunchRowsTokensW<WAVES, 2>(p, m, grouped, grid, stream) : LaunchRowsTokensW<WAVES, 4>(p, m, grouped, grid, stream);
+}
+
 template <int WAVES>
 hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_t stream) {
   const bool zp = p.seg[0].zero_point != nullptr, multi = p.segments > 1;
@@ -1190,12 +1352,12 @@ hipError_t LaunchRowsW(const StripParams& p, bool grouped, dim3 grid, hipStream_
   return hipGetLastError();
 }
 
-// The row-interleaved kernel serves: one token, every matrix of the launch packed in output groups
+// The row-interleaved kernels serve: 1..4 tokens, every matrix of the launch packed in output groups
 // of 2 slices, scale groups of a power-of-two number of K-slices.
 bool RowsKernelServes(const FcArgs* args, int count) {
   if (GetTuning().gemv_fast == 0) return false;
   if (args[0].params != nullptr) return false;  // runtime channel bounds: the streaming kernel
-  if (args[0].m != 1 || args[0].batch_ids != nullptr || args[0].k % 4 != 0) return false;
+  if (args[0].m < 1 || args[0].m > kGemvMaxTokens || args[0].batch_ids != nullptr || args[0].k % 4 != 0) return false;
   for (int i = 0; i < count; ++i) {
     const int ns = DivUp(args[i].n, 4);
     if (args[i].n % 8 != 0 || EffectiveGroup(args[i].group, ns) != 2) return false;
@@ -1237,6 +1399,14 @@ hipError_t LaunchRows(const StreamParams& p, const FcArgs* args, int count, bool
   while (waves < 16 && waves * 64 * rpt < p.ks) waves *= 2;
   if (GetTuning().gemv_waves > 0) waves = GetTuning().gemv_waves;
   const dim3 grid(strips);
+  if (p.m > 1) {  // 2..4 tokens: the token form, up to 8 waves
+    switch (std::min(waves, 8)) {
+      case 1: return LaunchRowsTokens<1>(sp, p.m, grouped, grid, stream);
+      case 2: return LaunchRowsTokens<2>(sp, p.m, grouped, grid, stream);
+      case 4: return LaunchRowsTokens<4>(sp, p.m, grouped, grid, stream);
+      default: return LaunchRowsTokens<8>(sp, p.m, grouped, grid, stream);
+    }
+  }
   switch (waves) {
     case 1: return LaunchRowsW<1>(sp, grouped, grid, stream);
     case 2: return LaunchRowsW<2>(sp, grouped, grid, stream);

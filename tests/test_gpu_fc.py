@@ -676,6 +676,43 @@ def test_rows_kernel(oracle, k, n, groups, zp, bias):
             check_fp(dev.result(), ref, case, "waves %d" % waves)
 
 
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 64, False, False), (2048, 2560, 1, True, True),
+                                               (16384, 2048, 512, False, True), (172, 536, 1, False, False),
+                                               (40000, 64, 1, True, False), (4096, 1536, 32, True, True)])
+def test_rows_kernel_tokens(oracle, m, k, n, groups, zp, bias):
+    """2..4 tokens over weights packed in output groups of 2 slices: the token form of the row-interleaved
+    kernel (a slot of 2 or 4 tokens, 3 tokens in a slot of 4), K that needs several passes and K that is no
+    multiple of the rows per pass; every work-group size the launcher can pick."""
+    case = W.make_fc_case(seed=k + n + m, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    print("rows kernel", m, "tokens", k, n, groups, zp, bias, flush=True)
+    dev = W.FcDevice(case, output_group=2)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_rows_kernel", dev.op.kernel_name
+    dev.out.zero_()
+    dev.run()
+    assert np.array_equal(got, dev.result())
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    if m * k * n <= 1 << 27:
+        rest = oracle_fc(oracle, case).astype(np.float64)
+        check_fp(got, rest, case, "kernel restatement")
+        check_as_accurate_as(got, rest, ref, case, "fc_w4_rows_kernel")
+    for waves in (1, 2, 8):
+        with M.tuning(gemv_waves=waves):
+            dev.out.zero_()
+            dev.run()
+            check_fp(dev.result(), ref, case, "waves %d" % waves)
+    # the streaming kernel that served these launches before agrees within the bar
+    with M.tuning(gemv_fast=0):
+        dev.out.zero_()
+        dev.run()
+        assert dev.op.kernel_name == "fc_w4_stream_kernel", dev.op.kernel_name
+        check_fp(dev.result(), ref, case, "streaming kernel")
+
+
 @pytest.mark.parametrize("td", [np.float32, np.float16])
 @pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 1, False, False), (2048, 2048, 64, True, True),
                                                (171, 536, 1, True, True), (16384, 256, 512, False, False),
