@@ -820,7 +820,9 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       } else
       // 2..16 tokens on wide per-channel layers: the matrix-core GEMV (one token streams faster
       // on the vector-ALU kernel; the tuning knob gemv_mfma = 1 forces the matrix-core one there too)
-      if (!force_generic && (a.m >= 2 || GetTuning().gemv_mfma > 0 || !FcW4StreamSupported(a)) &&
+      if (!force_generic && a.m >= 2 && a.m <= 4 && FcW4StripTokensSupported(a)) {
+        e = LaunchFcW4Stream(a, stream, &op->last_kernel);  // (2..4 tokens in whole strips: the token form of the strip kernel)
+      } else if (!force_generic && (a.m >= 2 || GetTuning().gemv_mfma > 0 || !FcW4StreamSupported(a)) &&
           FcW4MfmaStreamSupported(a)) {
         e = LaunchFcW4MfmaStream(a, stream, &op->last_kernel);
       } else if (!force_generic && FcW4StreamSupported(a)) {

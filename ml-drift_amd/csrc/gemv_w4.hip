@@ -1052,6 +1052,207 @@ hipError_t LaunchStrip(StreamParams& p, const FcArgs* args, int count, bool grou
   return hipGetLastError();
 }
 
+
+// ------------------------------------------------------------------------------------------
+// 2..4 tokens over strips of 64 channels, one chunk per thread (the launch shapes of the one-chunk
+// form above), with the multiply-accumulate on the matrix cores: v_mfma_f32_4x4x4_16B_f16 works on
+// 16 independent blocks of 4 lanes.  Lane i of a block supplies row i of A = the 4 K-values of
+// one of its 8 outputs (two unpacked words: exactly what the nibble trick yields), lane j supplies
+// column j of B = the 4 K-values of token j, and D[i][j] arrives in lane j, register i.  The 4
+// lanes of a block are 4 neighbouring 16-byte columns of one K-slice row, so they share the
+// K-slice and differ in the channels: one MFMA per output index multiplies the block's 32 channels
+// with up to 4 tokens, at the price of one token on the vector ALU.  Lane (row, col) then holds,
+// for token col % 4, the sums of the 32 channels of its block (value 8 * i + o = lane i, output o),
+// which meet across the 8 rows of a wave by the register exchanges of the one-token kernels (32 ->
+// 16 -> 8 -> 4 values per lane) and across waves through LDS.
+// The constant offsets of the unpacked codes (1024 + 8, 64 + 8) are removed per chunk with the
+// lane's own sum of its token's activations.
+// ------------------------------------------------------------------------------------------
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4v_t __attribute__((ext_vector_type(4)));
+
+template <int WAVES, bool GROUPED, bool MULTI, bool STRIDED>
+__global__ __launch_bounds__(WAVES * 64) void fc_w4_strip_tokens_kernel(StripParams p, int m) {
+  constexpr int LPR = 8, STRIP = 64, MT = 4;
+  __shared__ float red[WAVES][MT][STRIP];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane & 7;
+  const int row = tid >> 3;  // the thread's chunk
+  const int jt = col & 3;    // token slot of this lane
+  const int half = col >> 2; // which 32 channels of the strip its block holds
+  int strip = blockIdx.x;
+  const StripSegment sg = SelectSegment<MULTI>(p, strip);
+  const uint32_t mask_lo = p.mask_lo, mask_hi = p.mask_hi;
+  uint32_t magic_lo = p.magic_lo, magic_hi = p.magic_hi;
+  asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));  // (x & mask) | magic selects to one v_and_or_b32 that the compiler can see
+  asm volatile("" : : "s"(p.act), "s"(sg.dst), "s"(sg.bias), "s"(sg.scale));
+  const int ks = p.ks, n_pad = sg.n_pad;
+  const u32x4* wstrip = STRIDED ? sg.weights + (size_t)strip * LPR : sg.weights + (size_t)strip * ks * LPR;
+  const uint32_t row_items = STRIDED ? (uint32_t)sg.row_u4 : (uint32_t)LPR;
+  const uint32_t voff = (__umul24((uint32_t)row * 8u, row_items) + (uint32_t)col) * 16u;
+  const u32x4* wp = reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(wstrip) + voff);
+  // this lane's token (slots beyond the launch's tokens repeat the last one; their sums are dropped)
+  const u32x2* ap = reinterpret_cast<const u32x2*>(p.act) + ((size_t)row * 8 * m + min(jt, m - 1));
+  u32x4 w[8];
+  u32x2 a[8];
+  u32x4 sv[4];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) w[j] = __builtin_nontemporal_load(wp + (size_t)j * row_items);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) a[j] = ap[(size_t)j * m];
+  if (GROUPED) {
+    const int g = row / p.group_chunks;
+    const __half* sp = sg.scale + (size_t)g * n_pad + (size_t)strip * STRIP + half * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sv[i] = *reinterpret_cast<const u32x4*>(sp + i * 8);
+  }
+#pragma unroll
+  for (int j = 2; j < 8; ++j) w[j] = __builtin_nontemporal_load(wp + (size_t)j * row_items);
+
+  float4v_t acc[8];
+#pragma unroll
+  for (int o = 0; o < 8; ++o) acc[o] = float4v_t{0.0f, 0.0f, 0.0f, 0.0f};
+  float asum = 0.0f;
+  const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const half4_t b = __builtin_bit_cast(half4_t, a[j]);
+    asum = __builtin_amdgcn_fdot2(AsHalf2(a[j][0]), ones, asum, false);
+    asum = __builtin_amdgcn_fdot2(AsHalf2(a[j][1]), ones, asum, false);
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {  // outputs 4 * hh .. + 3: words 2 * hh (inputs 0, 1) and 2 * hh + 1 (inputs 2, 3)
+      const uint32_t l0 = w[j][2 * hh], l1 = w[j][2 * hh + 1];
+      const uint32_t h0 = l0 >> 8, h1 = l1 >> 8;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t s0 = (t & 2) ? h0 : l0, s1 = (t & 2) ? h1 : l1;
+        u32x2 q;
+        q[0] = (t & 1) ? ((s0 & mask_hi) | magic_hi) : ((s0 & mask_lo) | magic_lo);
+        q[1] = (t & 1) ? ((s1 & mask_hi) | magic_hi) : ((s1 & mask_lo) | magic_lo);
+        acc[4 * hh + t] = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, q), b, acc[4 * hh + t], 0, 0, 0);
+      }
+    }
+  }
+  // value 8 * i + o: channel 32 * half + 8 * i + o of the strip (lane i of the block, its output o)
+  float r[32];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+      const float centered = fmaf((o & 1) ? -72.0f : -1032.0f, asum, acc[o][i]);
+      r[8 * i + o] = GROUPED ? (float)AsHalf2(sv[i][o >> 1])[o & 1] * centered : centered;
+    }
+  }
+  float s16[16], s8[8];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const u32x2s x = __builtin_amdgcn_permlane32_swap(__float_as_uint(r[q]), __float_as_uint(r[q + 16]), false, false);
+    s16[q] = __uint_as_float(x[0]) + __uint_as_float(x[1]);
+  }
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const u32x2s x = __builtin_amdgcn_permlane16_swap(__float_as_uint(s16[q]), __float_as_uint(s16[q + 8]), false, false);
+    s8[q] = __uint_as_float(x[0]) + __uint_as_float(x[1]);
+  }
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+    s8[q] += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s8[q]), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+  const bool up8 = (lane & 8) != 0;
+  const float4 mine = make_float4(up8 ? s8[4] : s8[0], up8 ? s8[5] : s8[1], up8 ? s8[6] : s8[2], up8 ? s8[7] : s8[3]);
+  // lanes 32.. kept values 16.., lanes 16.. of each half values 8.., lanes 8.. of each 16 values 4..
+  const int first = 32 * half + ((lane >> 5) & 1) * 16 + ((lane >> 4) & 1) * 8 + ((lane >> 3) & 1) * 4;
+  *reinterpret_cast<float4*>(&red[wave][jt][first]) = mine;
+  __syncthreads();
+  for (int idx = tid; idx < STRIP * m; idx += WAVES * 64) {
+    const int t = idx >> 6, ch = idx & 63;
+    float v = 0.0f;
+#pragma unroll
+    for (int q = 0; q < WAVES; ++q) v += red[q][t][ch];
+    const int n_out = strip * STRIP + ch;
+    if (!GROUPED) v *= __half2float(sg.scale[n_out]);
+    __half h = __float2half_rn(v);
+    if (sg.bias) h = __hadd(h, sg.bias[n_out]);
+    sg.dst[((size_t)(n_out >> 2) * m + t) * 4 + (n_out & 3)] = h;
+  }
+}
+
+template <int WAVES>
+hipError_t LaunchStripTokensW(const StripParams& p, int m, bool grouped, bool strided, dim3 grid, hipStream_t stream) {
+  const bool multi = p.segments > 1;
+  const dim3 block(WAVES * 64);
+#define MLD_STRIP_T(G, MU, ST) hipLaunchKernelGGL((fc_w4_strip_tokens_kernel<WAVES, G, MU, ST>), grid, block, 0, stream, p, m)
+  if (strided) {
+    if (grouped) { if (multi) MLD_STRIP_T(true, true, true); else MLD_STRIP_T(true, false, true); }
+    else         { if (multi) MLD_STRIP_T(false, true, true); else MLD_STRIP_T(false, false, true); }
+  } else {
+    if (grouped) { if (multi) MLD_STRIP_T(true, true, false); else MLD_STRIP_T(true, false, false); }
+    else         { if (multi) MLD_STRIP_T(false, true, false); else MLD_STRIP_T(false, false, false); }
+  }
+#undef MLD_STRIP_T
+  return hipGetLastError();
+}
+
+// The token form serves: 2..4 tokens, no zero points, no batched weights or runtime bounds, every
+// matrix in whole strips of 64 channels packed in output groups of 16 slices (or all in the
+// reference's one group: strided rows), K = 256 ... 4096 input channels in powers of two (every
+// thread exactly one chunk), strips enough to keep K inside the work-groups.
+bool StripTokensServes(const FcArgs* args, int count, bool* strided) {
+  const Tuning& tune = GetTuning();
+  if (tune.gemv_fast == 0 || tune.gemv_one_chunk == 0 || tune.gemv_ksplit > 0 || tune.gemv_waves > 0 || tune.gemv_mfma == 0) return false;
+  if (args[0].params != nullptr || args[0].batch_ids != nullptr || args[0].m < 2 || args[0].m > 4) return false;
+  if (args[0].k % 32 != 0) return false;
+  const int ks = args[0].k / 4, chunks = ks / 8;
+  if (chunks < 8 || chunks > 128 || (chunks & (chunks - 1)) != 0) return false;
+  int strips = 0, native = 0, one = 0;
+  for (int i = 0; i < count; ++i) {
+    const int ns = DivUp(args[i].n, 4);
+    if (args[i].n % 64 != 0 || args[i].has_zero_point) return false;
+    const int group = EffectiveGroup(args[i].group, ns);
+    if (group == kNativeGroup) ++native; else if (group == ns) ++one; else return false;
+    if ((size_t)ks * ns * 8 >= ((size_t)1 << 32) || ns / 2 >= (1 << 24)) return false;  // 32-bit lane offsets
+    strips += ns / 16;
+  }
+  if (native != count && one != count) return false;
+  *strided = one == count && native != count;
+  return strips >= 128;
+}
+
+hipError_t LaunchStripTokens(StreamParams& p, const FcArgs* args, int count, bool grouped, bool strided, hipStream_t stream) {
+  int strips = 0;
+  for (int i = 0; i < count; ++i) {
+    strips += p.seg[i].ns / kNativeGroup;
+    p.seg[i].strip_end = strips;
+  }
+  StripParams sp = {};
+  sp.act = p.act;
+  sp.partial = nullptr;
+  sp.ks = p.ks;
+  sp.chunks = p.chunks;
+  sp.chunks_per_split = p.chunks;
+  sp.ksplit = 1;
+  sp.group_chunks = p.group_chunks;
+  sp.n_total = p.n_total;
+  sp.segments = p.segments;
+  sp.mask_lo = p.mask_lo;
+  sp.mask_hi = p.mask_hi;
+  sp.magic_lo = p.magic_lo;
+  sp.magic_hi = p.magic_hi;
+  for (int i = 0; i < kMaxSegments; ++i) {
+    const StreamSegment& g = p.seg[i];
+    sp.seg[i] = StripSegment{g.weights, g.scale, g.zero_point, g.bias, g.dst, g.n_pad, g.strip_end, g.n_off, g.row_u4};
+  }
+  const dim3 grid(strips);
+  switch (p.chunks / 8) {
+    case 1: return LaunchStripTokensW<1>(sp, p.m, grouped, strided, grid, stream);
+    case 2: return LaunchStripTokensW<2>(sp, p.m, grouped, strided, grid, stream);
+    case 4: return LaunchStripTokensW<4>(sp, p.m, grouped, strided, grid, stream);
+    case 8: return LaunchStripTokensW<8>(sp, p.m, grouped, strided, grid, stream);
+    default: return LaunchStripTokensW<16>(sp, p.m, grouped, strided, grid, stream);
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // One token over weights packed in output groups of 2 slices (8 channels): the whole K of a strip
 // of 8 channels is one contiguous run of 16-byte rows, so layers of a few thousand channels, which
@@ -1418,6 +1619,11 @@ hipError_t LaunchRows(const StreamParams& p, const FcArgs* args, int count, bool
 
 }  // namespace
 
+bool FcW4StripTokensSupported(const FcArgs& a) {
+  bool strided = false;
+  return FcW4StreamSupported(a) && StripTokensServes(&a, 1, &strided);
+}
+
 bool FcW4StreamSupported(const FcArgs& a) {
   if (a.weight_bits != 4 || !a.act_f16 || !a.dst_f16) return false;
   if (a.params != nullptr && (a.packed_params_offset >= 0 || a.ring_i_index >= 0 || a.ring_o_index >= 0)) return false;
@@ -1505,6 +1711,11 @@ hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stre
   if (RowsKernelServes(args, count)) {
     if (kernel_name) *kernel_name = "fc_w4_rows_kernel";
     return LaunchRows(p, args, count, grouped, stream);
+  }
+  bool tokens_strided = false;
+  if (StripTokensServes(args, count, &tokens_strided)) {
+    if (kernel_name) *kernel_name = "fc_w4_strip_tokens_kernel";
+    return LaunchStripTokens(p, args, count, grouped, tokens_strided, stream);
   }
   if (StripKernelServes(args, count)) {
     if (kernel_name) *kernel_name = "fc_w4_strip_kernel";

@@ -105,6 +105,8 @@ constexpr int kGemvMaxKSplit = 32;
 
 hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 bool FcW4StreamSupported(const FcArgs& a);
+// 2..4 tokens over wide layers in whole strips, one chunk per thread: the matrix-core token form of the strip kernel.
+bool FcW4StripTokensSupported(const FcArgs& a);
 hipError_t LaunchFcW4Stream(const FcArgs& a, hipStream_t stream, const char** kernel_name);
 // Up to 3 FCs that read the same activations (same m, k, scale grouping) as one launch.
 hipError_t LaunchFcW4StreamFused(const FcArgs* args, int count, hipStream_t stream, const char** kernel_name);

@@ -53,12 +53,13 @@ def test_no_alloc_decode_layout():
 
 
 def test_no_alloc_where_op_launch_takes_another_kernel(oracle):
-    """2 and 4 tokens on a per-channel layer of 8192 channels: mldhip_op_launch runs the matrix-core
+    """2 and 4 tokens on a per-channel layer of 8192 channels and 1056 input channels: mldhip_op_launch runs the matrix-core
     GEMV there, this entry point the streaming one, so the result is held to the oracle, not to the op."""
     import torch
     from test_gpu_fc import check_as_accurate_as, check_fp, oracle_fc, textbook
     for m in (2, 4):
-        case = W.make_fc_case(seed=76 + m, m=m, k=1024, n=8192, weight_bits=4, tensor_dtype=np.float16, groups=1, with_bias=True)
+        # (K = 1056: 33 chunks, so the one-chunk token form of the strip kernel does not serve the launch either)
+        case = W.make_fc_case(seed=76 + m, m=m, k=1056, n=8192, weight_bits=4, tensor_dtype=np.float16, groups=1, with_bias=True)
         dev = W.FcDevice(case)
         dev.run()
         assert dev.op.kernel_name == "fc_w4_mfma_stream_kernel", dev.op.kernel_name
