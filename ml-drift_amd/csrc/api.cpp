@@ -355,7 +355,7 @@ int mldhip_fc_is_recommended(int precision, int tokens) {
   return tokens <= kGemvMaxTokens ? 1 : 0;
 }
 
-static int AllocWorkspace(mldhip_op* op, int n) {
+static int AllocWorkspace(mldhip_op* op, int n, bool ring_i = false) {
   if (op->partial) return MLDHIP_OK;
   // A host without a GPU can still create and inspect ops (object lists, validation); they cannot
   // be launched there, so they need no workspace.
@@ -367,6 +367,8 @@ static int AllocWorkspace(mldhip_op* op, int n) {
   const int n_pad = DivUp(n, 4) * 4;
   op->partial_floats = std::max((size_t)kGemvMaxKSplit * kGemvMaxTokens * n_pad,
                                 FcW4MfmaWorkspaceFloats(op->fc.max_tokens, op->fc.i, op->fc.o));
+  // (the ring over the input channels: partial sums of the parts of its window)
+  if (ring_i) op->partial_floats = FcW8RingWorkspaceFloats(op->fc.max_tokens, op->fc.o);
   hipError_t e = hipMalloc(reinterpret_cast<void**>(&op->partial), op->partial_floats * sizeof(float));
   if (e != hipSuccess) return HipFail(e, "hipMalloc(workspace)");
   return MLDHIP_OK;
@@ -503,8 +505,8 @@ static int CreateFc(const mldhip_fc_desc* d, bool batch_ids, int weights_batch, 
   op->AddDst("dst_tensor");
   // split-K workspace of the fp16 streaming and matrix-core kernels: allocated here, so that no
   // launch allocates (a first launch may be under stream capture)
-  if (!int8_math && d->src_type == MLDHIP_FLOAT16) {
-    if (int rc = AllocWorkspace(op, d->o)) {
+  if (!int8_math && (d->src_type == MLDHIP_FLOAT16 || ring_i)) {
+    if (int rc = AllocWorkspace(op, d->o, ring_i)) {
       delete op;
       return rc;
     }
@@ -805,6 +807,10 @@ int mldhip_op_launch(mldhip_op* op, void* stream_ptr) {
       const bool bounded_stream = bounded && a.packed_params_offset < 0 && a.ring_i_index < 0 && a.ring_o_index < 0 &&
                                   (FcW4StreamSupported(a) || FcW8StreamSupported(a));
       const bool force_generic = GetTuning().force_generic > 0 || (bounded && !bounded_stream);
+      // ringed weights over the input channels at a few tokens: the kernel that walks the ring's rows
+      if (GetTuning().force_generic <= 0 && FcW8RingSupported(a)) {
+        e = LaunchFcW8Ring(a, stream, &op->last_kernel);
+      } else
       // packed groups: the matrix-core GEMM with one launch plane per matrix where it serves the shape
       if (GetTuning().force_generic <= 0 && FcW4MfmaPackedSupported(a)) {
         e = LaunchFcW4Mfma(a, stream, &op->last_kernel);

@@ -104,6 +104,11 @@ constexpr int kGemvMaxTokens = 4;
 constexpr int kGemvMaxKSplit = 32;
 
 hipError_t LaunchFcGeneric(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+// Ringed uint8 weights with the ring over the input channels, 1..4 tokens per row, up to 16 tokens per
+// launch: walks the ring's own K-slice rows (aligned 16-byte blocks) and shifts the activations.
+bool FcW8RingSupported(const FcArgs& a);
+hipError_t LaunchFcW8Ring(const FcArgs& a, hipStream_t stream, const char** kernel_name);
+size_t FcW8RingWorkspaceFloats(int max_tokens, int o);
 bool FcW4StreamSupported(const FcArgs& a);
 // 2..4 tokens over wide layers in whole strips, one chunk per thread: the matrix-core token form of the strip kernel.
 bool FcW4StripTokensSupported(const FcArgs& a);

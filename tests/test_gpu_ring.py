@@ -65,14 +65,20 @@ def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=
     op.bind(srcs, [out])
     op.set_shape(1, batch, tokens) if batch > 1 else op.set_shape(1, 1, tokens)
     conv = (lambda a: o.f32_to_f16_bits(np.asarray(a, np.float32))) if f16 else (lambda a: np.asarray(a, np.float32))
-    for off in offsets:
+    # a ring over the input channels, a multiple of 4 long, with the window inside one turn, at up to 4
+    # tokens per row and 16 per launch, runs on the kernel that walks the ring's rows; every case also
+    # runs on the unspecialised kernel
+    fast = axis == "i" and ring % 4 == 0 and src_c <= ring and tokens <= 4 and batch * tokens <= 16
+    for forced, off in [(f, x) for f in (False, True) for x in offsets]:
         params[0] = off
         d_params.copy_(torch.from_numpy(params))
         out.fill_(7.0)
-        print("ring", axis, src_c, dst_c, ring, "batch", batch, "tokens", tokens, "offset", off, "f16", f16, "src_end", src_end_ch, flush=True)
-        op.launch(torch.cuda.current_stream().cuda_stream)
+        print("ring", axis, src_c, dst_c, ring, "batch", batch, "tokens", tokens, "offset", off, "f16", f16, "src_end", src_end_ch,
+              "unspecialised" if forced else "", flush=True)
+        with M.tuning(**(dict(force_generic=1) if forced else {})):
+            op.launch(torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
-        assert op.kernel_name == "fc_generic_kernel", op.kernel_name
+        assert op.kernel_name == ("fc_w8_ring_i_kernel" if fast and not forced else "fc_generic_kernel"), op.kernel_name
         got = W.from_slices(out.cpu().numpy().astype(np.float32), dst_c)
         active = None if src_end_ch is None else (min(src_end_ch, src_c) + 3) // 4 * 4
         for b in range(batch):
@@ -112,6 +118,18 @@ def test_ringed_i_with_src_end_ch(oracle, src_end_ch):
     """ring_i_offset_index beside src_end_ch_index, as the reference's ringed test binds them
     (params = {ring_offset, src_end_ch})."""
     run_ring(oracle, "i", 20, 72, 56, 1, [17, 49], False, seed=21, src_end_ch=src_end_ch)
+
+
+@pytest.mark.parametrize("f16", [False, True])
+def test_ring_i_window_shapes(oracle, f16):
+    """The ring-walking kernel: windows that fill the ring (the window wraps onto its first row), windows of one
+    and of a few channels, every offset modulo 4, dst widths below and above 64 slices, 2 and 4 tokens per
+    row, rows with batched weights, a source bound inside the window."""
+    run_ring(oracle, "i", 1024, 64, 1024, 1, [0, 1, 2, 3, 1021, 517], f16, seed=41)
+    run_ring(oracle, "i", 1, 256, 64, 1, [0, 3, 62, 63], f16, seed=42)
+    run_ring(oracle, "i", 6, 520, 128, 1, [0, 125, 127], f16, seed=43, tokens=2)
+    run_ring(oracle, "i", 2048, 128, 2048, 4, [5, 2047], f16, seed=44, tokens=4)
+    run_ring(oracle, "i", 4096, 256, 8192, 1, [0, 4095, 6001], f16, seed=45, src_end_ch=1001)
 
 
 def test_larger_rings_and_odd_offsets(oracle):
