@@ -99,6 +99,41 @@ struct Quantizer {
 // codes in the C16 layout); the first CACHE groups of a thread stay in registers between the
 // min/max pass and the encoding pass, so a row of up to 16 * CACHE * lanes channels is read
 // from memory once.
+// The value of the lane whose number differs in bit OFF (8, 16 or 32), paired with the lane's own:
+// {own or partner, partner or own} in some order, which is all a symmetric reduction (max, min, sum)
+// needs.  Register exchanges and a data-parallel move instead of a trip through the LDS crossbar.
+typedef uint32_t u32x2q __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ __forceinline__ u32x2q PairAcross(uint32_t v) {
+  if constexpr (OFF == 32) {
+    return __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  } else if constexpr (OFF == 16) {
+    return __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  } else if constexpr (OFF == 8) {
+    return u32x2q{v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128 /* row_ror:8 */, 0xf, 0xf, false)};
+  } else {
+    return u32x2q{v, (uint32_t)__shfl_xor((int)v, OFF)};
+  }
+}
+template <int FROM, typename Op>
+__device__ __forceinline__ float ReduceAcross(float v, Op op) {
+  if constexpr (FROM < 64) {
+    const u32x2q r = PairAcross<FROM>(__float_as_uint(v));
+    return ReduceAcross<FROM * 2>(op(__uint_as_float(r[0]), __uint_as_float(r[1])), op);
+  } else {
+    return v;
+  }
+}
+template <int FROM>
+__device__ __forceinline__ int SumAcross(int v) {
+  if constexpr (FROM < 64) {
+    const u32x2q r = PairAcross<FROM>((uint32_t)v);
+    return SumAcross<FROM * 2>((int)r[0] + (int)r[1]);
+  } else {
+    return v;
+  }
+}
+
 template <typename SrcT, int TT, bool SYM, int CACHE, bool RNE = false>
 __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
   using RawT = typename Raw<SrcT>::type;
@@ -171,14 +206,11 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
     }
   }
   // lanes of a wave that share a token, then the waves of the work-group
-#pragma unroll
-  for (int off = TT; off < 64; off *= 2) {
-    if (SYM) {
-      r0 = fmaxf(r0, __shfl_xor(r0, off));
-    } else {
-      r0 = fminf(r0, __shfl_xor(r0, off));
-      r1 = fmaxf(r1, __shfl_xor(r1, off));
-    }
+  if (SYM) {
+    r0 = ReduceAcross<TT>(r0, [](float a, float b) { return fmaxf(a, b); });
+  } else {
+    r0 = ReduceAcross<TT>(r0, [](float a, float b) { return fminf(a, b); });
+    r1 = ReduceAcross<TT>(r1, [](float a, float b) { return fmaxf(a, b); });
   }
   if (threadIdx.x % 64 < TT) {
     s_a[wave][lt] = r0;
@@ -306,8 +338,7 @@ __global__ __launch_bounds__(1024) void quantize_kernel(QuantParams p) {
   }
   if (p.calculate_sum) {
     int total = (int)sum;
-#pragma unroll
-    for (int off = TT; off < 64; off *= 2) total += __shfl_xor(total, off);
+    total = SumAcross<TT>(total);
     if (threadIdx.x % 64 < TT) s_sum[wave][lt] = total;
     __syncthreads();
     total = 0;
