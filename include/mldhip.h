@@ -101,10 +101,13 @@ const char* mldhip_version(void);
 /* Overrides a launch heuristic of this library for the whole process (tests and tuning runs;
  * the reference keeps its counterpart, the work-group size argument of
  * CreateFullyConnectedExternalWeights, common/kernels/fully_connected.h:155-161, per call).
- * value -1 restores the heuristic.  Knobs: force_generic, gemv_mfma, gemv_fast, gemv_lpr,
- * gemv_waves, gemv_ksplit, gemv_narrow_max_mb, gemm_fm, gemm_ksplit, gemm_no_pair, gemm_dual,
- * gemm_xcd_m, gemm_i8_fm.  MLDHIP_NOT_FOUND for an unknown name.  Not thread-safe against
- * concurrent launches. */
+ * value -1 restores the heuristic.  Knobs: force_generic, gemv_mfma, gemv_fast, gemv_one_chunk,
+ * fc_group, gemv_lpr, gemv_waves, gemv_ksplit, gemv_rows_rpt, gemv_narrow_max_mb, gemm_fm,
+ * gemm_ksplit, gemm_no_pair, gemm_dual, gemm_xcd_m, gemm_i8_fm.  MLDHIP_NOT_FOUND for an unknown
+ * name.  A test and tuning aid, not part of the op contract: the state is one set of plain
+ * integers per process, read without synchronisation at every launch (and by
+ * mldhip_fc_int4_weights_desc for fc_group), so it must not be changed while another thread
+ * creates or launches ops; a product build never calls it. */
 int mldhip_set_tuning(const char* name, int value);
 
 /* ------------------------------------------------------------------------------------ */
