@@ -17,7 +17,7 @@ from test_oracle_ring import make, rolled_product
 OFFSETS = [0, 17, 20, 33, 49]
 
 
-def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=None, tokens=1):
+def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=None, tokens=1, dst_end_ch=None):
     """One op, its ring offset rewritten on the device between launches.  batch > 1: the batch-ids op with
     one dst row per matrix (the reference's test puts matrix y on row y)."""
     import torch
@@ -37,7 +37,7 @@ def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=
     ks, ns = (src_c + 3) // 4, (dst_c + 3) // 4
     pad = lambda v: np.pad(v, (0, ns * 4 - dst_c)).astype(np.float32)
     tens = lambda v: torch.from_numpy(M.scale_to_tensor(v, mt).view(td) if f16 else M.scale_to_tensor(v, mt)).cuda()
-    params = np.array([0, -1 if src_end_ch is None else src_end_ch], np.int32)
+    params = np.array([0, -1 if src_end_ch is None else src_end_ch, -1 if dst_end_ch is None else dst_end_ch], np.int32)
     kw = dict(ring_size=ring, has_bias=True, has_zero_point_tensor=True, scale_shape=(dst_c, 1), max_tokens=batch * tokens)
     kw["ring_i_offset_index" if axis == "i" else "ring_o_offset_index"] = 0
     if axis == "i":
@@ -46,6 +46,8 @@ def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=
         kw["dst_channels"] = dst_c
     if src_end_ch is not None:
         kw["src_end_ch_index"] = 1
+    if dst_end_ch is not None:
+        kw["dst_end_ch_index"] = 2
     if batch > 1:
         kw["weights_batch"] = batch
     op = M.fc_create(M.PRECISION_F32_F16 if f16 else M.PRECISION_F32, mt, mt, w_o, w_i, desc, **kw)
@@ -80,6 +82,10 @@ def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=
         torch.cuda.synchronize()
         assert op.kernel_name == ("fc_w8_ring_i_kernel" if fast and not forced else "fc_generic_kernel"), op.kernel_name
         got = W.from_slices(out.cpu().numpy().astype(np.float32), dst_c)
+        # dst slices from the bound (rounded up to 32 channels) on are not written
+        n_written = dst_c if dst_end_ch is None else min((dst_end_ch + 31) // 32 * 32, ns * 4)
+        if n_written < dst_c:
+            assert np.all(got[:, n_written:] == 7.0), "dst slices beyond the bound were written"
         active = None if src_end_ch is None else (min(src_end_ch, src_c) + 3) // 4 * 4
         for b in range(batch):
             rows = slice(b * tokens, (b + 1) * tokens)
@@ -90,9 +96,10 @@ def run_ring(o, axis, src_c, dst_c, ring, batch, offsets, f16, seed, src_end_ch=
             rest = o.from_slices(o.f16_bits_to_f32(rest) if f16 else rest, dst_c)
             for t in range(tokens):
                 exact = rolled_product(q, a_rows[t], scale, zp, bias, axis, ring, off, b, src_c, dst_c, active=active)
+                exact = exact[:n_written]
                 rms = np.sqrt(np.mean(exact ** 2))
-                err = np.abs(got[rows][t] - exact).max()
-                err_rest = np.abs(rest[t] - exact).max()
+                err = np.abs(got[rows][t][:n_written] - exact).max()
+                err_rest = np.abs(rest[t][:n_written] - exact).max()
                 if f16:
                     assert err <= 2e-2 * rms, (b, off, err, rms)
                 else:
@@ -130,6 +137,7 @@ def test_ring_i_window_shapes(oracle, f16):
     run_ring(oracle, "i", 6, 520, 128, 1, [0, 125, 127], f16, seed=43, tokens=2)
     run_ring(oracle, "i", 2048, 128, 2048, 4, [5, 2047], f16, seed=44, tokens=4)
     run_ring(oracle, "i", 4096, 256, 8192, 1, [0, 4095, 6001], f16, seed=45, src_end_ch=1001)
+    run_ring(oracle, "i", 512, 320, 512, 2, [0, 258], f16, seed=46, dst_end_ch=70, tokens=2)
 
 
 def test_larger_rings_and_odd_offsets(oracle):
