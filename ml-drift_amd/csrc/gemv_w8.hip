@@ -369,6 +369,171 @@ __global__ __launch_bounds__(WAVES * 64) void fc_w8_rows_kernel(W8Params p) {
   Store1(static_cast<T*>(p.dst), n, v, static_cast<const T*>(p.bias), n);
 }
 
+// ------------------------------------------------------------------------------------------
+// The same walk for 2..4 tokens: every weight row is converted once and used for MT token slots
+// (tensors are [slice][token][4], so the MT activation vectors of a K-slice are neighbours in
+// memory).  3 tokens run in 4 slots: the last slot re-reads token 2 and is not stored.  Fewer rows
+// are in flight per lane as the slots grow (8 at 2 slots, 4 at 4), which keeps the kernel clear of
+// register spills.
+// ------------------------------------------------------------------------------------------
+template <typename T, int WAVES, int MT, bool GROUPED>
+__global__ __launch_bounds__(WAVES * 64) void fc_w8_rows_tokens_kernel(W8Params p) {
+  constexpr int TH = WAVES * 64;
+  constexpr int U = MT == 2 ? 8 : 4;
+  __shared__ float red[WAVES][MT][4];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  int slice = blockIdx.x;
+  if (slice < (int)(gridDim.x & ~63u)) slice = (slice & ~63) + ((slice & 7) << 3) + ((slice >> 3) & 7);
+  const int ks = p.ks;
+  const int m = p.m;
+  const u32x4* wrow = p.weights + (size_t)slice * ks;
+  const T* act = static_cast<const T*>(p.act);
+  const T* scale = static_cast<const T*>(p.scale);
+  const T* zero_point = static_cast<const T*>(p.zero_point);
+  const size_t group_stride = (size_t)p.ns * 4;
+  const int group_shift = p.group_chunks;
+
+  float acc[MT][4], asum_all[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    asum_all[t] = 0.0f;
+#pragma unroll
+    for (int o = 0; o < 4; ++o) acc[t][o] = 0.0f;
+  }
+  float s_lin[4] = {1.0f, 1.0f, 1.0f, 1.0f}, z_lin[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (!GROUPED) {
+    Load4(scale, (size_t)slice * 4, s_lin);
+    if (zero_point) Load4(zero_point, (size_t)slice * 4, z_lin);
+  }
+  const bool has_zp = zero_point != nullptr;
+  const T* zsrc = has_zp ? zero_point : scale;
+  for (int r0 = tid; r0 < ks; r0 += U * TH) {
+    u32x4 w[U];
+    decltype(LoadRaw4(act, 0)) araw[U][MT], sraw[U], zraw[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        araw[j][t] = LoadRaw4(act, ((size_t)min(r0 + TH * j, ks - 1) * m + min(t, m - 1)) * 4);
+    if (GROUPED) {
+#pragma unroll
+      for (int j = 0; j < U; ++j) {
+        const size_t so = (size_t)(min(r0 + TH * j, ks - 1) >> group_shift) * group_stride + (size_t)slice * 4;
+        sraw[j] = LoadRaw4(scale, so);
+        zraw[j] = LoadRaw4(zsrc, so);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) w[j] = __builtin_nontemporal_load(wrow + min(r0 + TH * j, ks - 1));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      const bool live = r0 + TH * j < ks;
+      float u[4][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t word = w[j][i];
+        u[i][0] = (float)(word & 0xFFu);
+        u[i][1] = (float)((word >> 8) & 0xFFu);
+        u[i][2] = (float)((word >> 16) & 0xFFu);
+        u[i][3] = (float)(word >> 24);
+      }
+      float sc[4], zp[4];
+      if (GROUPED) {
+        Cvt4(sraw[j], sc);
+        Cvt4(zraw[j], zp);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        float a[4], tt[4] = {0.0f, 0.0f, 0.0f, 0.0f}, asum = 0.0f;
+        Cvt4(araw[j][t], a);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float av = live ? a[i] : 0.0f;
+          asum += av;
+#pragma unroll
+          for (int o = 0; o < 4; ++o) tt[o] = fmaf(av, u[i][o], tt[o]);
+        }
+        if (GROUPED) {
+#pragma unroll
+          for (int o = 0; o < 4; ++o)
+            acc[t][o] = fmaf(sc[o], fmaf(-(128.0f + (has_zp ? zp[o] : 0.0f)), asum, tt[o]), acc[t][o]);
+        } else {
+          asum_all[t] += asum;
+#pragma unroll
+          for (int o = 0; o < 4; ++o) acc[t][o] += tt[o];
+        }
+      }
+    }
+  }
+  // per token the reduction of the one-token kernel: lane l ends with channel 2 * (l / 32) + (l / 16) % 2
+  typedef unsigned u32x2s __attribute__((ext_vector_type(2)));
+  float v[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (!GROUPED) {
+#pragma unroll
+      for (int o = 0; o < 4; ++o) acc[t][o] = s_lin[o] * fmaf(-(128.0f + z_lin[o]), asum_all[t], acc[t][o]);
+    }
+    const u32x2s e0 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[t][0]), __float_as_uint(acc[t][2]), false, false);
+    const u32x2s e1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[t][1]), __float_as_uint(acc[t][3]), false, false);
+    const float x0 = __uint_as_float(e0[0]) + __uint_as_float(e0[1]);
+    const float x1 = __uint_as_float(e1[0]) + __uint_as_float(e1[1]);
+    const u32x2s e2 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x0), __float_as_uint(x1), false, false);
+    float x = __uint_as_float(e2[0]) + __uint_as_float(e2[1]);
+    x += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x128 /* row_ror:8 */, 0xf, 0xf, false));
+    {
+      const uint32_t up = __builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x104 /* row_shl:4 */, 0xf, 0x5, false);
+      const uint32_t both = __builtin_amdgcn_update_dpp(up, __float_as_uint(x), 0x114 /* row_shr:4 */, 0xf, 0xA, false);
+      x += __uint_as_float(both);
+    }
+    x += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x4E /* quad_perm:[2,3,0,1] */, 0xf, 0xf, false));
+    x += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0xB1 /* quad_perm:[1,0,3,2] */, 0xf, 0xf, false));
+    v[t] = x;
+  }
+  const int ch = 2 * (lane >> 5) + ((lane >> 4) & 1);
+  if (WAVES > 1) {
+    if ((lane & 15) == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) red[wave][t][ch] = v[t];
+    }
+    __syncthreads();
+    if (tid >= 64) return;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      v[t] = 0.0f;
+#pragma unroll
+      for (int q = 0; q < WAVES; ++q) v[t] += red[q][t][ch];
+    }
+  }
+  if ((lane & 15) != 0) return;
+  const size_t n = (size_t)slice * 4 + ch;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+    if (t < m) Store1(static_cast<T*>(p.dst), ((size_t)slice * m + t) * 4 + ch, v[t], static_cast<const T*>(p.bias), n);
+}
+
+template <typename T, int WAVES, int MT>
+hipError_t LaunchRowsTokensG(const W8Params& p, dim3 grid, hipStream_t stream) {
+  if (p.grouped)
+    hipLaunchKernelGGL((fc_w8_rows_tokens_kernel<T, WAVES, MT, true>), grid, dim3(WAVES * 64), 0, stream, p);
+  else
+    hipLaunchKernelGGL((fc_w8_rows_tokens_kernel<T, WAVES, MT, false>), grid, dim3(WAVES * 64), 0, stream, p);
+  return hipGetLastError();
+}
+template <typename T, int MT>
+hipError_t LaunchRowsTokensT(const W8Params& p, int waves, hipStream_t stream) {
+  const dim3 grid(p.ns);
+  switch (waves) {
+    case 1: return LaunchRowsTokensG<T, 1, MT>(p, grid, stream);
+    case 2: return LaunchRowsTokensG<T, 2, MT>(p, grid, stream);
+    case 4: return LaunchRowsTokensG<T, 4, MT>(p, grid, stream);
+    default: return LaunchRowsTokensG<T, 8, MT>(p, grid, stream);
+  }
+}
+
 template <typename T, int WAVES>
 hipError_t LaunchRowsG(const W8Params& p, dim3 grid, hipStream_t stream) {
   if (p.grouped)
@@ -391,12 +556,19 @@ hipError_t LaunchRowsT(const W8Params& p, int waves, hipStream_t stream) {
 template <typename T, int LPR, int WAVES, bool BATCHED>
 hipError_t LaunchMB(const W8Params& p, dim3 grid, hipStream_t stream) {
   const dim3 block(WAVES * 64);
-  switch (p.m) {
-    case 1: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1, BATCHED>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 2, BATCHED>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 3, BATCHED>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 4, BATCHED>), grid, block, 0, stream, p); break;
-    default: return hipErrorInvalidValue;
+  // 16 waves leave a lane 128 registers, which only the one-token form fits without spills; more
+  // tokens run with 8 waves at most (256 registers)
+  if constexpr (WAVES == 16) {
+    if (p.m != 1) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1, BATCHED>), grid, block, 0, stream, p);
+  } else {
+    switch (p.m) {
+      case 1: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 1, BATCHED>), grid, block, 0, stream, p); break;
+      case 2: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 2, BATCHED>), grid, block, 0, stream, p); break;
+      case 3: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 3, BATCHED>), grid, block, 0, stream, p); break;
+      case 4: hipLaunchKernelGGL((fc_w8_stream_kernel<T, LPR, WAVES, 4, BATCHED>), grid, block, 0, stream, p); break;
+      default: return hipErrorInvalidValue;
+    }
   }
   return hipGetLastError();
 }
@@ -408,8 +580,11 @@ hipError_t LaunchM(const W8Params& p, dim3 grid, hipStream_t stream) {
 template <typename T>
 hipError_t LaunchT(const W8Params& p, int lpr, int waves, hipStream_t stream) {
   const dim3 grid(DivUp(p.ns, lpr), 1, p.batch_ids ? p.rows : 1);
-  if (lpr == 4) return waves == 4 ? LaunchM<T, 4, 4>(p, grid, stream) : LaunchM<T, 4, 16>(p, grid, stream);
-  return waves == 4 ? LaunchM<T, 8, 4>(p, grid, stream) : LaunchM<T, 8, 16>(p, grid, stream);
+  if (lpr == 4)
+    return waves == 4 ? LaunchM<T, 4, 4>(p, grid, stream)
+         : waves == 8 ? LaunchM<T, 4, 8>(p, grid, stream) : LaunchM<T, 4, 16>(p, grid, stream);
+  return waves == 4 ? LaunchM<T, 8, 4>(p, grid, stream)
+       : waves == 8 ? LaunchM<T, 8, 8>(p, grid, stream) : LaunchM<T, 8, 16>(p, grid, stream);
 }
 
 }  // namespace
@@ -429,10 +604,10 @@ bool FcW8StreamSupported(const FcArgs& a) {
   return true;
 }
 
-// The row-interleaved kernel serves: one token, output groups of one slice, scale groups of a
+// The row-interleaved kernels serve: 1..4 tokens, output groups of one slice, scale groups of a
 // power-of-two number of K-slices.
 bool FcW8RowsSupported(const FcArgs& a) {
-  if (a.weight_bits != 8 || a.act_f16 != a.dst_f16 || a.m != 1 || a.batch_ids != nullptr) return false;
+  if (a.weight_bits != 8 || a.act_f16 != a.dst_f16 || a.m < 1 || a.m > 4 || a.batch_ids != nullptr) return false;
   if (a.params != nullptr) return false;  // runtime channel bounds: the streaming kernel
   const int ns = DivUp(a.n, 4), ks = DivUp(a.k, 4);
   if (ns < 2 || EffectiveGroup(a.group, ns) != 1) return false;
@@ -454,7 +629,7 @@ hipError_t LaunchFcW8Rows(const FcArgs& a, hipStream_t stream, const char** kern
   p.zero_point = a.has_zero_point ? a.zero_point : nullptr;
   p.bias = a.bias;
   p.dst = a.dst;
-  p.m = 1;
+  p.m = a.m;
   p.ks = DivUp(a.k, 4);
   p.ns = DivUp(a.n, 4);
   p.chunks = DivUp(p.ks, 8);
@@ -472,6 +647,17 @@ hipError_t LaunchFcW8Rows(const FcArgs& a, hipStream_t stream, const char** kern
   int waves = 1;
   while (waves < 8 && waves * 64 * 8 < p.ks) waves *= 2;
   if (GetTuning().gemv_waves > 0) waves = GetTuning().gemv_waves;
+  if (a.m > 1) {
+    // rows in flight per lane: 8 at 2 token slots, 4 at 4
+    const int per_lane = a.m == 2 ? 8 : 4;
+    waves = 1;
+    while (waves < 8 && waves * 64 * per_lane < p.ks) waves *= 2;
+    if (GetTuning().gemv_waves > 0) waves = GetTuning().gemv_waves;
+    if (kernel_name) *kernel_name = "fc_w8_rows_tokens_kernel";
+    if (a.m == 2)
+      return a.act_f16 ? LaunchRowsTokensT<__half, 2>(p, waves, stream) : LaunchRowsTokensT<float, 2>(p, waves, stream);
+    return a.act_f16 ? LaunchRowsTokensT<__half, 4>(p, waves, stream) : LaunchRowsTokensT<float, 4>(p, waves, stream);
+  }
   if (kernel_name) *kernel_name = "fc_w8_rows_kernel";
   return a.act_f16 ? LaunchRowsT<__half>(p, waves, stream) : LaunchRowsT<float>(p, waves, stream);
 }
@@ -502,7 +688,7 @@ hipError_t LaunchFcW8Stream(const FcArgs& a, hipStream_t stream, const char** ke
   // 128-byte row segments (8 slices) when that still gives a work-group to half the CUs, else
   // 64-byte ones; small work-groups when K is covered by 64 / 128 rows of chunks
   const int lpr = (long)DivUp(p.ns, 8) * (a.batch_ids ? a.rows : 1) >= 128 ? 8 : 4;
-  const int waves = p.chunks <= 4 * 64 / lpr ? 4 : 16;
+  const int waves = p.chunks <= 4 * 64 / lpr ? 4 : p.m > 1 ? 8 : 16;
   if (kernel_name) *kernel_name = "fc_w8_stream_kernel";
   return a.act_f16 ? LaunchT<__half>(p, lpr, waves, stream) : LaunchT<float>(p, lpr, waves, stream);
 }

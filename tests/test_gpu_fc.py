@@ -790,6 +790,55 @@ def test_w8_rows_kernel(oracle, td, k, n, groups, zp, bias):
             check_fp(dev.result(), ref, case, "waves %d" % waves)
 
 
+@pytest.mark.parametrize("td", [np.float32, np.float16])
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("k,n,groups,zp,bias", [(2048, 2048, 1, False, False), (2048, 2048, 64, True, True),
+                                               (171, 536, 1, True, True), (16384, 256, 512, False, False),
+                                               (4096, 1536, 1, False, True), (40, 8, 1, False, False),
+                                               (10000, 64, 1, True, False)])
+def test_w8_rows_kernel_tokens(oracle, td, m, k, n, groups, zp, bias):
+    """2..4 tokens over uint8 weights packed in output groups of one slice: the token form of the
+    row-interleaved kernel (slots of 2 or 4 tokens, 3 tokens in a slot of 4), both tensor types, every
+    work-group size, ragged K and K that needs several passes."""
+    case = W.make_fc_case(seed=k + n + m, m=m, k=k, n=n, weight_bits=8, tensor_dtype=td, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    print("w8 rows kernel", m, "tokens", td.__name__, k, n, groups, zp, bias, flush=True)
+    dev = W.FcDevice(case, decode_layout=True)
+    assert dev.desc.output_group_size == 1
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w8_rows_tokens_kernel", dev.op.kernel_name
+    dev.out.zero_()
+    dev.run()
+    assert np.array_equal(got, dev.result())
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    if m * k * n <= 1 << 25:
+        rest = oracle_fc(oracle, case).astype(np.float64)
+        check_fp(got, rest, case, "kernel restatement")
+    for waves in (1, 2, 8):
+        with M.tuning(gemv_waves=waves):
+            dev.out.zero_()
+            dev.run()
+            check_fp(dev.result(), ref, case, "waves %d" % waves)
+    # the unspecialised kernel agrees within the bar
+    with M.tuning(force_generic=1):
+        dev.out.zero_()
+        dev.run()
+        assert dev.op.kernel_name == "fc_generic_kernel", dev.op.kernel_name
+        check_fp(dev.result(), ref, case, "unspecialised kernel")
+
+
+@pytest.mark.parametrize("m", [2, 3, 4])
+@pytest.mark.parametrize("groups", [1, 32])
+def test_w8_stream_kernel_tokens_long_k(oracle, m, groups):
+    """2..4 tokens over uint8 weights in the library layout with a K long enough for the large
+    work-group of the streaming kernel (8 waves at these token counts)."""
+    case = W.make_fc_case(seed=61 + m, m=m, k=4096, n=2048, weight_bits=8, tensor_dtype=np.float16,
+                          groups=groups, with_bias=True, with_zero_point=groups > 1)
+    run_case(oracle, case, "fc_w8_stream_kernel")
+
+
 def test_config1_decode_layout(oracle):
     """c1 over the layout mldhip_fc_int8_weights_desc_decode asks for, as the bench runs it."""
     case = W.make_fc_case(**W.CONFIGS["c1"])
