@@ -41,6 +41,8 @@ def parse():
     p.add_argument("--tokens", type=int, default=128,
                    help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
                         "kernels away from the launch-bound regime)")
+    p.add_argument("--shape", default="", help="c3: another GEMM shape as M,K,N,GROUP (tokens, input channels, output "
+                   "channels, input channels per scale group), e.g. 8192,4096,14336,32 for a large prefill chunk")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
     p.add_argument("--layout", default="default", choices=["default", "library", "reference", "decode"],
                    help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
@@ -228,15 +230,20 @@ def run_other(args, torch, M, W):
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
     elif args.workload == "c3":
-        case = W.make_fc_case(**W.CONFIGS["c3"])
+        cfg = dict(W.CONFIGS["c3"])
+        label = "c3: FullyConnected prefill GEMM M=512 K=4096 N=4096 int4 group-32, fp16 act/out"
+        if args.shape:
+            sm, sk, sn, sg = [int(v) for v in args.shape.split(",")]
+            cfg.update(m=sm, k=sk, n=sn, groups=sk // sg)
+            label = "c3 at another shape: FullyConnected prefill GEMM M=%d K=%d N=%d int4 group-%d, fp16 act/out" % (sm, sk, sn, sg)
+        case = W.make_fc_case(**cfg)
         dev = W.FcDevice(case)
         wall, us, reg = time_graph(torch, stream, lambda s, i: dev.op.launch(s), args.steps, args.warmup)
         flops = 2.0 * case["m"] * case["k"] * case["n"]
         out = dict(base, metric="int4_prefill_gemm_throughput", value=round(flops / wall / 1e12, 1),
                    unit="TFLOP/s", ms_per_step=round(wall * 1e3, 6),
                    dtype="u4 weights x f16 activations, f32 accumulate (fp16 MFMA)",
-                   config=dict({"workload": "c3: FullyConnected prefill GEMM M=512 K=4096 N=4096 int4 group-32, fp16 act/out",
-                                "flops_per_step": flops}, **reg),
+                   config=dict({"workload": label, "flops_per_step": flops}, **reg),
                    roofline={"bound": "mfma", "kernel": dev.op.kernel_name, "achieved": round(flops / us / 1e6, 1),
                              "peak": 2500.0, "unit": "TFLOP/s", "frac": round(flops / us / 1e6 / 2500.0, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})

@@ -103,7 +103,7 @@ const char* mldhip_version(void);
  * CreateFullyConnectedExternalWeights, common/kernels/fully_connected.h:155-161, per call).
  * value -1 restores the heuristic.  Knobs: force_generic, gemv_mfma, gemv_fast, gemv_one_chunk,
  * fc_group, gemv_lpr, gemv_waves, gemv_ksplit, gemv_rows_rpt, gemv_narrow_max_mb, gemm_fm,
- * gemm_ksplit, gemm_no_pair, gemm_dual, gemm_xcd_m, gemm_i8_fm.  MLDHIP_NOT_FOUND for an unknown
+ * gemm_ksplit, gemm_no_pair, gemm_dual, gemm_xcd_m, gemm_i8_fm, gemm_tiled.  MLDHIP_NOT_FOUND for an unknown
  * name.  A test and tuning aid, not part of the op contract: the state is one set of plain
  * integers per process, read without synchronisation at every launch (and by
  * mldhip_fc_int4_weights_desc for fc_group), so it must not be changed while another thread

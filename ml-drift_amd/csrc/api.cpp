@@ -186,7 +186,7 @@ int mldhip_set_tuning(const char* name, int value) {
       {"gemv_lpr", &t.gemv_lpr}, {"gemv_waves", &t.gemv_waves}, {"gemv_ksplit", &t.gemv_ksplit},
       {"gemv_narrow_max_mb", &t.gemv_narrow_max_mb}, {"gemm_fm", &t.gemm_fm}, {"gemm_ksplit", &t.gemm_ksplit},
       {"gemm_no_pair", &t.gemm_no_pair}, {"gemm_dual", &t.gemm_dual}, {"gemm_xcd_m", &t.gemm_xcd_m},
-      {"gemm_i8_fm", &t.gemm_i8_fm}};
+      {"gemm_i8_fm", &t.gemm_i8_fm}, {"gemm_tiled", &t.gemm_tiled}};
   for (const auto& k : knobs)
     if (std::strcmp(name, k.name) == 0) {
       *k.field = value;

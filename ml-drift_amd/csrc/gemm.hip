@@ -1128,6 +1128,318 @@ void LaunchDirect(int weight_bits, bool zp, dim3 grid, hipStream_t stream, const
     LaunchDirectW<4, FM, U, WAVES, PAIR, kModePlain>(zp, grid, stream, p);
 }
 
+// ------------------------------------------------------------------------------------------
+// int4-weight GEMM for many tokens with both operands shared through LDS.
+//
+// Work-group = 4 waves (2 x 2) on 256 channels x 256 tokens, each wave 128 x 128 (its 256
+// accumulators in the AGPR half of the register file), K in stages of 32 input channels (two MFMA
+// steps).  Per stage and work-group:
+//  - weights: 64 slices x 8 K-slice rows of 8-byte blocks.  Thread (slice = lane, K-slice pair = wave)
+//    loads its two blocks four stages ahead, dequantizes them once for the whole work-group (the
+//    direct kernel dequantizes every weight once per 128-token tile) into the four A operands of
+//    MFMAs t = 0..3 (rows = channels 4 * slice + t) and writes them to LDS as
+//    [MFMA step][K half][t][slice][16 bytes]: a lane's operand read is one aligned 16-byte item and a
+//    wave's read covers consecutive items.  Two slots: the stage being multiplied and the next one.
+//  - activations: 8 K-slice rows x 256 tokens x 8 bytes, copied global -> LDS by loads that write
+//    LDS directly, in the tensor's own order ([row][token][4 halfs], 2 KB per row).  A lane's B
+//    operand (8 consecutive input channels of one token) is the two 8-byte items of rows 2q, 2q + 1:
+//    one ds_read2st64_b64.  Four slots, three stages of copies in flight.
+// One barrier per stage, between its two MFMA steps: step 0 runs next to the reads of step 1, the
+// copies and loads of later stages and the dequantization of the next stage, step 1 next to the
+// operand reads of the next stage's step 0.  The LDS side is inline asm: the compiler does not know
+// what the LDS-writing loads touch and would wait for all of them in front of any LDS access it sees.
+// ------------------------------------------------------------------------------------------
+constexpr int kTlThreads = 256;
+constexpr int kTlASlot = 16384, kTlBSlot = 16384;  // bytes of one stage of either tile
+constexpr int kTlBBase = 2 * kTlASlot;            // the activation slots follow the two weight slots
+
+template <int OFF>
+__device__ __forceinline__ void DsWrite128(uint32_t addr, const u32x4& v) {
+  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(v), "n"(OFF) : "memory");
+}
+// two 8-byte items, 512 * O0 and 512 * O1 bytes behind addr
+template <int O0, int O1>
+__device__ __forceinline__ void DsRead2x64(u32x4& dst, uint32_t addr) {
+  asm volatile("ds_read2st64_b64 %0, %1 offset0:%2 offset1:%3" : "=v"(dst) : "v"(addr), "n"(O0), "n"(O1));
+}
+
+template <bool ZP>
+__global__ __launch_bounds__(kTlThreads) void fc_w4_mfma_tiled_kernel(GemmParams p) {
+  __shared__ u32x4 smem[(2 * kTlASlot + 4 * kTlBSlot) / 16];
+  const LdsPtr lds = (LdsPtr)smem;
+  const uint32_t lds_base = (uint32_t)(size_t)lds;
+  asm volatile("" : : "s"(p.m), "s"(p.ks), "s"(p.group_shift), "s"(p.b_bytes), "s"(p.act), "s"(p.magic_lo), "s"(p.magic_hi),
+               "s"(p.mask_lo), "s"(p.mask_hi));
+  asm volatile("" : : "s"(p.seg[0].w4), "s"(p.seg[0].scale), "s"(p.seg[0].ns), "s"(p.seg[0].group), "s"(p.seg[0].a_bytes),
+               "s"(p.seg[0].s_bytes), "s"(p.seg[0].dst), "s"(p.seg[0].bias), "s"(p.seg[0].group_shift));
+  const W4Segment sg = p.seg[0];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wm = wave >> 1;
+  const int r32 = lane & 31, g2 = lane >> 5;
+
+  // Tile order: XCD x (work-groups go round-robin to the 8 XCDs) takes a contiguous range of a
+  // numbering that walks blocks of 8 channel tiles token tile by token tile, so that the tiles
+  // which share an L2 form a compact rectangle.
+  const int tiles_n = (sg.ns + 63) / 64;
+  const int tiles_m = (p.m + 255) / 256;
+  const int per_xcd = (tiles_n * tiles_m + 7) / 8;
+  const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (tile >= tiles_n * tiles_m) return;
+  int tn, tm;
+  {
+    const int full = tiles_n / 8;
+    if (tile < full * 8 * tiles_m) {
+      const int sc = tile / (8 * tiles_m), within = tile % (8 * tiles_m);
+      tn = sc * 8 + within % 8;
+      tm = within / 8;
+    } else {
+      const int rest = tile - full * 8 * tiles_m, width = tiles_n - full * 8;
+      tn = full * 8 + rest % width;
+      tm = rest / width;
+    }
+  }
+  const int slice0 = tn * 64;
+  const int m0 = tm * 256;
+
+  constexpr uint32_t kOob = 0x7FFFFFF0u;
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(sg.w4), 0, sg.a_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(p.act), 0, p.b_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_s = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(sg.scale), 0, sg.s_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_z =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<__half*>(ZP ? sg.zp : sg.scale), 0, sg.s_bytes, 0x00020000);
+
+  // Weight duty: slice `lane` of the tile, K-slice rows 2 * wave and 2 * wave + 1 of every stage.
+  // (Rows past K are beyond the buffer with one output group and read zeros; with several they are
+  // rows of other groups, finite values that meet the zeros the activations' descriptor returns.)
+  const int nsi = slice0 + lane;
+  const bool n_ok = nsi < sg.ns;
+  const bool one_group = sg.group >= sg.ns;
+  const uint32_t row_w = (uint32_t)sg.group * 8u;
+  const uint32_t nsi_group = sg.group_shift >= 0 ? (uint32_t)nsi >> sg.group_shift : (uint32_t)(nsi / sg.group);
+  const uint32_t nsi_in_group = (uint32_t)nsi - nsi_group * (uint32_t)sg.group;
+  const uint32_t col_w = one_group ? (uint32_t)nsi * 8u : (nsi_group * (uint32_t)p.ks * (uint32_t)sg.group + nsi_in_group) * 8u;
+  uint32_t vw = n_ok ? (uint32_t)(2 * wave) * row_w + col_w : kOob;
+  const uint32_t step_w = 8u * row_w;
+  const uint32_t vs = n_ok ? (uint32_t)nsi * 8u : kOob;
+  const uint32_t group_bytes = (uint32_t)sg.ns * 8u;
+  const uint32_t addr_w = lds_base + (uint32_t)((wave * 4) * 64 + lane) * 16u;
+
+  // Copy duty: rows 2 * wave, 2 * wave + 1 of every stage, two halves of 128 tokens (a lane moves a
+  // pair of tokens; the token count is even, so a pair is inside the row or past it).
+  const uint32_t row_x = (uint32_t)p.m * 8u, step_x = 8u * row_x;
+  uint32_t vb[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int tok = m0 + (c & 1) * 128 + 2 * lane;
+    vb[c] = tok < p.m ? (uint32_t)(2 * wave + (c >> 1)) * row_x + (uint32_t)tok * 8u : kOob;
+  }
+  auto copy_one = [&](int slot, int c) {
+    CopyToLds(rsrc_x, lds + kTlBBase + slot * kTlBSlot + ((2 * wave + (c >> 1)) * 256 + (c & 1) * 128) * 8, vb[c]);
+    vb[c] += step_x;
+  };
+
+  // operand addresses (slot, MFMA step and operand number go into the instructions' offsets)
+  const uint32_t addr_a = lds_base + (uint32_t)((g2 * 4) * 64 + wn * 32 + r32) * 16u;
+  const uint32_t addr_b0 = lds_base + (uint32_t)kTlBBase + (uint32_t)((2 * g2) * 256 + wm * 128 + r32) * 8u;
+  const uint32_t addr_b1 = addr_b0 + 256u;  // token blocks 1 and 3
+
+  // the registers of four stages of weights in flight
+  u32x2 wq[4][2], wsc[4], wzp[4];
+  auto load_w = [&](int set, int t) {
+    const uint32_t so = vs + (uint32_t)((2 * t) >> p.group_shift) * group_bytes;
+    wsc[set] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_s, so, 0, 0);
+    if (ZP) wzp[set] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_z, so, 0, 0);
+    wq[set][0] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw, 0, 0);
+    wq[set][1] = __builtin_amdgcn_raw_buffer_load_b64(rsrc_w, vw + row_w, 0, 0);
+    vw += step_w;
+  };
+  constexpr int kLw = ZP ? 4 : 3;  // loads of one stage of weights
+
+  uint32_t magic_lo = p.magic_lo, magic_hi = p.magic_hi;
+  asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
+  const half2_t off_lo = {(_Float16)-1032.0f, (_Float16)-1032.0f};
+  const half2_t off_hi = {(_Float16)-72.0f, (_Float16)-72.0f};
+  // word wd (input channels 2 wd, 2 wd + 1 of the 8) of the operand of MFMA t4, from register set `set`
+  auto dequant_word = [&](int set, int t4, int wd) -> uint32_t {
+    const uint32_t sp = (t4 & 2) ? wsc[set][1] : wsc[set][0];
+    const half2_t sph = AsHalf2(sp);
+    const half2_t s2 = (t4 & 1) ? __builtin_shufflevector(sph, sph, 1, 1) : __builtin_shufflevector(sph, sph, 0, 0);
+    half2_t mzs = {(_Float16)0.0f, (_Float16)0.0f};
+    if (ZP) {
+      const half2_t zq = AsHalf2((t4 & 2) ? wzp[set][1] : wzp[set][0]);
+      mzs = -(((t4 & 1) ? __builtin_shufflevector(zq, zq, 1, 1) : __builtin_shufflevector(zq, zq, 0, 0)) * s2);
+    }
+    const uint32_t raw = wq[set][wd >> 1][wd & 1];
+    const uint32_t x = (t4 & 2) ? raw >> 8 : raw;
+    const uint32_t bits = (t4 & 1) ? ((x & p.mask_hi) | magic_hi) : ((x & p.mask_lo) | magic_lo);
+    const half2_t centred = AsHalf2(bits) + ((t4 & 1) ? off_hi : off_lo);  // exact: u - 8
+    return AsU32(ZP ? __builtin_elementwise_fma(centred, s2, mzs) : centred * s2);
+  };
+
+  float16_t acc[4][4];
+#pragma unroll
+  for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+    for (int fm = 0; fm < 4; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[t4][fm][v] = 0.0f;
+
+  // Waits until the activation copies of the next stage have landed (the loads issued behind them
+  // stay in flight: two more stages of copies and three of weights) and this wave's LDS writes are
+  // done, then meets the other waves.
+  auto stage_barrier = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(8 + 3 * kLw) : "memory");
+  };
+
+  // Prologue, in the order the loop continues: weights 0, then (copies s, weights s + 1) for s = 0, 1, 2.
+  const int stages = (p.ks + 7) / 8;
+  load_w(0, 0);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s0 = 0; s0 < 3; ++s0) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) copy_one(s0, c);
+    __builtin_amdgcn_sched_barrier(0);
+    load_w(s0 + 1, s0 + 1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int t4 = 0; t4 < 4; ++t4) {
+    u32x4 aop;
+#pragma unroll
+    for (int wd = 0; wd < 4; ++wd) aop[wd] = dequant_word(0, t4, wd);
+    switch (t4) {
+      case 0: DsWrite128<0 * 1024>(addr_w, aop); break;
+      case 1: DsWrite128<1 * 1024>(addr_w, aop); break;
+      case 2: DsWrite128<2 * 1024>(addr_w, aop); break;
+      default: DsWrite128<3 * 1024>(addr_w, aop); break;
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  stage_barrier();
+  u32x4 fa[2][4], fb[2][4];
+  DsRead128<0 * 1024>(fa[0][0], addr_a);
+  DsRead128<1 * 1024>(fa[0][1], addr_a);
+  DsRead128<2 * 1024>(fa[0][2], addr_a);
+  DsRead128<3 * 1024>(fa[0][3], addr_a);
+  DsRead2x64<0, 4>(fb[0][0], addr_b0);
+  DsRead2x64<0, 4>(fb[0][1], addr_b1);
+  DsRead2x64<1, 5>(fb[0][2], addr_b0);
+  DsRead2x64<1, 5>(fb[0][3], addr_b1);
+
+  // Stage t, t % 4 = S known at compile time: every slot, register set and offset is a constant.
+  auto stage = [&](auto tag, int t) {
+    constexpr int S = decltype(tag)::value;
+    constexpr int SA = S & 1, SB = S;                  // slots of this stage
+    constexpr int NA = (S + 1) & 1, NB = (S + 1) & 3;  // slots of the next stage
+    constexpr int RB = (S + 3) & 3;                    // activation slot that takes stage t + 3
+    constexpr int NW = (S + 1) & 3;                    // register set of the next stage's weights
+    LdsWait(fa[0]);
+    LdsWait(fb[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 aop = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      const int t4 = idx / 4, fm = idx % 4;
+      acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fa[0][t4]),
+                                                           __builtin_bit_cast(half8_t, fb[0][fm]), acc[t4][fm], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // the operands of step 1, the copies of stage t + 3, the weights of stage t + 4
+      switch (idx) {
+        case 0: DsRead128<SA * kTlASlot + 8192 + 0 * 1024>(fa[1][0], addr_a); break;
+        case 1: DsRead128<SA * kTlASlot + 8192 + 1 * 1024>(fa[1][1], addr_a); break;
+        case 2: DsRead128<SA * kTlASlot + 8192 + 2 * 1024>(fa[1][2], addr_a); break;
+        case 3: DsRead128<SA * kTlASlot + 8192 + 3 * 1024>(fa[1][3], addr_a); break;
+        case 4: DsRead2x64<SB * 32 + 16 + 0, SB * 32 + 16 + 4>(fb[1][0], addr_b0); break;
+        case 5: DsRead2x64<SB * 32 + 16 + 0, SB * 32 + 16 + 4>(fb[1][1], addr_b1); break;
+        case 6: DsRead2x64<SB * 32 + 16 + 1, SB * 32 + 16 + 5>(fb[1][2], addr_b0); break;
+        case 7: DsRead2x64<SB * 32 + 16 + 1, SB * 32 + 16 + 5>(fb[1][3], addr_b1); break;
+        case 8: copy_one(RB, 0); break;
+        case 9: copy_one(RB, 1); break;
+        case 10: copy_one(RB, 2); break;
+        case 11: copy_one(RB, 3); break;
+        case 12: load_w(S, t + 4); break;
+        default: break;
+      }
+      // one word of the next stage's weights; every fourth completes an operand
+      aop[idx % 4] = dequant_word(NW, idx / 4, idx % 4);
+      if (idx % 4 == 3) {
+        switch (idx / 4) {
+          case 0: DsWrite128<NA * kTlASlot + 0 * 1024>(addr_w, aop); break;
+          case 1: DsWrite128<NA * kTlASlot + 1 * 1024>(addr_w, aop); break;
+          case 2: DsWrite128<NA * kTlASlot + 2 * 1024>(addr_w, aop); break;
+          default: DsWrite128<NA * kTlASlot + 3 * 1024>(addr_w, aop); break;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    LdsWait(fa[1]);
+    LdsWait(fb[1]);
+    stage_barrier();  // stage t + 1 is complete in LDS for every wave
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int idx = 0; idx < 16; ++idx) {
+      const int t4 = idx / 4, fm = idx % 4;
+      acc[t4][fm] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fa[1][t4]),
+                                                           __builtin_bit_cast(half8_t, fb[1][fm]), acc[t4][fm], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      switch (idx) {  // step 0 of the next stage
+        case 0: DsRead128<NA * kTlASlot + 0 * 1024>(fa[0][0], addr_a); break;
+        case 1: DsRead128<NA * kTlASlot + 1 * 1024>(fa[0][1], addr_a); break;
+        case 2: DsRead128<NA * kTlASlot + 2 * 1024>(fa[0][2], addr_a); break;
+        case 3: DsRead128<NA * kTlASlot + 3 * 1024>(fa[0][3], addr_a); break;
+        case 4: DsRead2x64<NB * 32 + 0, NB * 32 + 4>(fb[0][0], addr_b0); break;
+        case 5: DsRead2x64<NB * 32 + 0, NB * 32 + 4>(fb[0][1], addr_b1); break;
+        case 6: DsRead2x64<NB * 32 + 1, NB * 32 + 5>(fb[0][2], addr_b0); break;
+        case 7: DsRead2x64<NB * 32 + 1, NB * 32 + 5>(fb[0][3], addr_b1); break;
+        default: break;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // (stages past K, up to the next multiple of four, multiply zeros)
+  for (int t = 0; t < stages; t += 4) {
+    stage(std::integral_constant<int, 0>{}, t);
+    stage(std::integral_constant<int, 1>{}, t + 1);
+    stage(std::integral_constant<int, 2>{}, t + 2);
+    stage(std::integral_constant<int, 3>{}, t + 3);
+  }
+  // the copies and reads that ran ahead land before the work-group's LDS is released
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+  // Register v of lane (g2, r32) belongs to slice 8 * (v / 4) + 4 * g2 + v % 4 of the wave's 32 and to
+  // token r32 of the block; the four MFMAs hold the slice's four channels: one 8-byte store.
+  // (the bias of the lane's 16 slices is requested before any of it is used: one memory latency)
+  u32x2 bias_all[16];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) bias_all[v] = u32x2{0x80008000u, 0x80008000u};  // -0.0: adding it changes nothing
+  if (sg.bias) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int slice = min(slice0 + wn * 32 + 8 * (v >> 2) + 4 * g2 + (v & 3), sg.ns - 1);
+      bias_all[v] = *reinterpret_cast<const u32x2*>(sg.bias + (size_t)slice * 4);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int slice = slice0 + wn * 32 + 8 * (v >> 2) + 4 * g2 + (v & 3);
+    if (slice >= sg.ns) continue;
+    const u32x2 bias2 = bias_all[v];
+#pragma unroll
+    for (int fm = 0; fm < 4; ++fm) {
+      const int mi = m0 + wm * 128 + fm * 32 + r32;
+      if (mi >= p.m) continue;
+      u32x2 o;
+      o[0] = AsU32(__builtin_convertvector(float2v_t{acc[0][fm][v], acc[1][fm][v]}, half2_t) + AsHalf2(bias2[0]));
+      o[1] = AsU32(__builtin_convertvector(float2v_t{acc[2][fm][v], acc[3][fm][v]}, half2_t) + AsHalf2(bias2[1]));
+      *reinterpret_cast<u32x2*>(sg.dst + ((size_t)slice * p.m + mi) * 4) = o;
+    }
+  }
+}
+
 // Second pass of a K split across work-groups: adds the parts in a fixed order, converts, adds
 // the bias.  One thread per (slice, token).
 __global__ __launch_bounds__(256) void fc_w4_splitk_reduce_kernel(GemmParams p) {
@@ -1342,6 +1654,27 @@ hipError_t LaunchDirectGemm(const FcArgs* args, int count, int gate_activation, 
     const int shares = kw * p.ksplit, steps_total = DivUp(p.k, 16);
     p.geo_per_wave = DivUp(DivUp(steps_total, shares), prefetch) * prefetch;
   };
+  // Many tokens over one uint4 matrix: both operands shared through LDS, 256 x 256 tiles.  Both
+  // kernels run into the same limit on large launches (the chip lowers its clock under dense MFMA
+  // work on random data) and finish within a few percent of each other, so the tile counts decide:
+  // the large tiles are taken where they fill one round of the 256 CUs and the 128 x 128 tiles of
+  // the direct kernel would leave its last round half empty (1024 x 4096 x 14336: 131 against 155 us).
+  {
+    const bool tiled_ok = !gated && !packed && count == 1 && a.weight_bits == 4 && a.m % 2 == 0 && p.group_size % 32 == 0;
+    const long tiles = (long)DivUp(a.n, 256) * DivUp(a.m, 256);
+    const long small_tiles_last = ((long)DivUp(a.n, 128) * DivUp(a.m, 128)) % 256;
+    bool tiled = tiled_ok && a.m >= 1024 && tiles >= 208 && tiles <= 256 && small_tiles_last >= 1 && small_tiles_last <= 160;
+    if (tune.gemm_tiled >= 0) tiled = tiled_ok && tune.gemm_tiled != 0;
+    if (tiled) {
+      if (kernel_name) *kernel_name = "fc_w4_mfma_tiled_kernel";
+      const dim3 grid((unsigned)DivUp(tiles, 8L) * 8u), block(kTlThreads);
+      if (p.seg[0].zp != nullptr)
+        hipLaunchKernelGGL((fc_w4_mfma_tiled_kernel<true>), grid, block, 0, stream, p);
+      else
+        hipLaunchKernelGGL((fc_w4_mfma_tiled_kernel<false>), grid, block, 0, stream, p);
+      return hipGetLastError();
+    }
+  }
   if (packed) {
     p.pg_params = a.params;
     p.pg_offset = a.packed_params_offset;

@@ -174,6 +174,7 @@ struct Tuning {
   int gemv_one_chunk = -1;      // 0: never take the one-chunk form of the contiguous-strip GEMV
   int gemm_fm = -1, gemm_ksplit = -1, gemm_no_pair = -1, gemm_dual = -1, gemm_xcd_m = -1;
   int gemm_i8_fm = -1;
+  int gemm_tiled = -1;          // 1 / 0: always / never take the LDS-tiled int4 GEMM where it can run
 };
 Tuning& GetTuning();
 

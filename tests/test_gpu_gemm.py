@@ -118,6 +118,67 @@ def test_gemm_fractional_zero_points(oracle, bits, m, k, n, groups):
     check_restatement(oracle, got[:small], sub, "kernel restatement")
 
 
+@pytest.mark.parametrize("m,k,n,groups,zp,bias", [(256, 64, 256, 1, False, False),     # one tile, two stages
+                                                  (300, 352, 1000, 11, True, True),    # ragged edges, 11 stages of one group each
+                                                  (1026, 96, 260, 1, False, True),     # 5 token tiles, the last of 2 tokens
+                                                  (512, 4096, 512, 128, False, False),
+                                                  (2048, 64, 4096, 2, True, True),
+                                                  (130, 1024, 640, 8, False, True),
+                                                  (258, 160, 516, 1, True, False)])
+def test_w4_gemm_tiled_kernel(oracle, m, k, n, groups, zp, bias):
+    """The LDS-tiled int4 GEMM (256 x 256 tiles, weights dequantized once per work-group), forced on
+    shapes of test size: ragged token and channel edges, stage counts that are no multiple of the
+    four the loop is unrolled by, group-wise scales down to one stage per group, zero points, bias,
+    both weight layouts (which must agree bit for bit)."""
+    case = W.make_fc_case(seed=m + n + k, m=m, k=k, n=n, weight_bits=4, tensor_dtype=np.float16, groups=groups,
+                          with_bias=bias, with_zero_point=zp)
+    print("tiled gemm", m, k, n, groups, zp, bias, flush=True)
+    from test_gpu_fc import native_layout_differs
+    results = []
+    with M.tuning(gemm_tiled=1):
+        for ref_layout in ([False, True] if native_layout_differs(case) else [True]):
+            dev = W.FcDevice(case, reference_layout=ref_layout)
+            dev.run()
+            got = dev.result()
+            assert dev.op.kernel_name == "fc_w4_mfma_tiled_kernel", dev.op.kernel_name
+            dev.out.zero_()
+            dev.run()
+            assert np.array_equal(got, dev.result())
+            results.append(got)
+    if len(results) == 2:
+        assert np.array_equal(results[0], results[1]), "the two weight layouts give different sums"
+    got = results[0]
+    check_fp(got, textbook(case), case, "textbook")
+    small = min(m, 64)
+    sub = dict(case, m=small, act=case["act"][:small])
+    if restatement_affordable(sub):
+        check_restatement(oracle, got[:small], sub, "kernel restatement")
+    # the last tokens too (the ragged token tile)
+    tail = dict(case, m=min(m, 32), act=case["act"][-min(m, 32):])
+    if restatement_affordable(tail):
+        check_restatement(oracle, got[-min(m, 32):], tail, "kernel restatement (last tokens)")
+
+
+def test_w4_gemm_tiled_kernel_chosen_for_one_round_of_large_tiles(oracle):
+    """1024 tokens x 14336 channels are 224 tiles of 256 x 256 (one round of the 256 CUs) and 896 of
+    128 x 128 (three and a half): the launcher takes the LDS-tiled kernel by itself; a forced direct
+    launch agrees within the bar."""
+    case = W.make_fc_case(seed=77, m=1024, k=256, n=14336, weight_bits=4, tensor_dtype=np.float16, groups=8, with_bias=True)
+    dev = W.FcDevice(case)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_mfma_tiled_kernel", dev.op.kernel_name
+    ref = textbook(case)
+    check_fp(got, ref, case, "textbook")
+    with M.tuning(gemm_tiled=0):
+        dev.out.zero_()
+        dev.run()
+        assert dev.op.kernel_name == "fc_w4_mfma_gemm_kernel", dev.op.kernel_name
+        check_fp(dev.result(), ref, case, "direct kernel")
+    sub = dict(case, m=64, act=case["act"][:64])
+    check_restatement(oracle, got[:64], sub, "kernel restatement (first 64 tokens)")
+
+
 @pytest.mark.parametrize("bits,m,k,n,groups,zp", [(4, 64, 512, 384, 4, False),    # 3 channel tiles: the last pair holds one
                                                   (4, 130, 352, 1000, 11, True),   # ragged channels and tokens, 64-token tile
                                                   (4, 256, 96, 260, 1, False),
