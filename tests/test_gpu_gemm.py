@@ -179,6 +179,21 @@ def test_w4_gemm_tiled_kernel_chosen_for_one_round_of_large_tiles(oracle):
     check_restatement(oracle, got[:64], sub, "kernel restatement (first 64 tokens)")
 
 
+def test_w4_gemm_tiled_kernel_full_size(oracle):
+    """The LDS-tiled kernel at the size its launcher picks it for (1024 tokens x 4096 x 14336, scale groups of
+    32 channels: 128 stages per tile): every output against the textbook reference, the first and the last 32
+    tokens against the restatement of the reference's kernel."""
+    case = W.make_fc_case(seed=5, m=1024, k=4096, n=14336, weight_bits=4, tensor_dtype=np.float16, groups=128)
+    dev = W.FcDevice(case)
+    dev.run()
+    got = dev.result()
+    assert dev.op.kernel_name == "fc_w4_mfma_tiled_kernel", dev.op.kernel_name
+    check_fp(got, textbook(case), case, "textbook")
+    for name, rows in (("first", slice(0, 32)), ("last", slice(-32, None))):
+        sub = dict(case, m=32, act=case["act"][rows])
+        check_restatement(oracle, got[rows], sub, "kernel restatement (%s 32 tokens)" % name)
+
+
 @pytest.mark.parametrize("bits,m,k,n,groups,zp", [(4, 64, 512, 384, 4, False),    # 3 channel tiles: the last pair holds one
                                                   (4, 130, 352, 1000, 11, True),   # ragged channels and tokens, 64-token tile
                                                   (4, 256, 96, 260, 1, False),
