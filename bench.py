@@ -35,14 +35,16 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=None, help="default 4000 (c2, c1, f2), 2000 (moe), 200 (c3, c4), 20 (c5-*)")
     p.add_argument("--warmup", type=int, default=None, help="default steps / 10")
-    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe"],
+    p.add_argument("--workload", default="c2", choices=["c2", "c1", "c3", "c4", "c5-decode", "c5-prefill", "f2", "moe", "gemv"],
                    help="c2 (default) is the headline line; the others time the remaining configurations "
                         "the same way (one JSON line each, no CPU baseline)")
     p.add_argument("--tokens", type=int, default=128,
                    help="c5-prefill: tokens per step (the configuration is quoted at 128; larger chunks show the "
                         "kernels away from the launch-bound regime)")
     p.add_argument("--shape", default="", help="c3: another GEMM shape as M,K,N,GROUP (tokens, input channels, output "
-                   "channels, input channels per scale group), e.g. 8192,4096,14336,32 for a large prefill chunk")
+                   "channels, input channels per scale group), e.g. 8192,4096,14336,32 for a large prefill chunk; "
+                   "gemv: the shape of the few-token FullyConnected to time (GROUP = K: per-channel scales)")
+    p.add_argument("--bits", type=int, default=4, choices=[4, 8], help="gemv: weight bits")
     p.add_argument("--ring", type=int, default=16, help="distinct weight copies (16 x 29.4 MB > 256 MB)")
     p.add_argument("--layout", default="default", choices=["default", "library", "reference", "decode"],
                    help="c2: int4 weights in the layout mldhip_fc_int4_weights_desc asks for (output groups of 16 "
@@ -59,7 +61,7 @@ def parse():
                         "reference dispatch) followed by 64 launches over the weight ring, then exit")
     a = p.parse_args()
     if a.steps is None:
-        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "moe": 2000, "c3": 200, "c4": 200}.get(a.workload, 20)
+        a.steps = {"c2": 4000, "c1": 4000, "f2": 4000, "moe": 2000, "gemv": 2000, "c3": 200, "c4": 200}.get(a.workload, 20)
     if a.warmup is None:
         a.warmup = max(1, a.steps // 10)
     return a
@@ -188,6 +190,39 @@ def run_other(args, torch, M, W):
         out = dict(base, metric=metric, value=round(nbytes / wall / 1e9, 1), unit="GB/s",
                    ms_per_step=round(wall * 1e3, 6), dtype=dtype,
                    config=dict({"workload": label, "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes}, **reg),
+                   roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                             "traffic": None, "avg_launch_us": round(us, 3)})
+    elif args.workload == "gemv":
+        # a FullyConnected of 1..16 tokens at a shape of the caller's choice (fp16 tensors, symmetric weights), over a
+        # ring of weight copies larger than the 256 MB cache: the few-token figures quoted beside the configurations
+        if not args.shape:
+            print("--workload gemv needs --shape M,K,N,GROUP", file=sys.stderr)
+            sys.exit(2)
+        sm, sk, sn, sg = [int(v) for v in args.shape.split(",")]
+        groups = 1 if sg >= sk else sk // sg
+        case = W.make_fc_case(seed=0, m=sm, k=sk, n=sn, weight_bits=args.bits, tensor_dtype=np.float16, groups=groups)
+        dev0 = W.FcDevice(case, reference_layout=args.layout == "reference", decode_layout=args.layout == "decode")
+        wbytes = dev0.weights.numel()
+        ring = max(2, min(100, -(-(300 << 20) // wbytes)))
+        gen = torch.Generator(device="cuda").manual_seed(1)
+        ops, keep = [dev0.op], [dev0]
+        for r in range(1, ring):
+            wt = torch.randint(0, 256, dev0.weights.shape, dtype=torch.uint8, device="cuda", generator=gen)
+            op = M.fc_create(M.PRECISION_F32_F16, M.FLOAT16, M.FLOAT16, sn, sk, dev0.desc, scale_shape=(sn, groups), max_tokens=sm)
+            op.bind([dev0.act, wt, dev0.scale], [dev0.out])
+            op.set_shape(1, 1, sm)
+            ops.append(op)
+            keep.append(wt)
+        nbytes, _ = ops[0].cost()
+        wall, us, reg = time_graph(torch, stream, lambda s, i: ops[i % len(ops)].launch(s), args.steps, args.warmup,
+                                   ring=len(ops))
+        out = dict(base, metric="decode_gemv_hbm_bandwidth", value=round(nbytes / wall / 1e9, 1), unit="GB/s",
+                   ms_per_step=round(wall * 1e3, 6), dtype="u%d weights x f16 activations, f32 accumulate" % args.bits,
+                   config=dict({"workload": "gemv: FullyConnected M=%d K=%d N=%d int%d, %s, fp16 act/out" % (
+                                    sm, sk, sn, args.bits, "per-channel" if groups == 1 else "group-%d" % sg),
+                                "weights_layout": "kOSpatialIOGroupI4O4, output_group_size %d" % dev0.desc.output_group_size,
+                                "weight_ring": len(ops), "algorithmic_bytes_per_step": nbytes}, **reg),
                    roofline={"bound": "hbm", "kernel": ops[0].kernel_name, "achieved": round(nbytes / us / 1e3, 1),
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                              "traffic": None, "avg_launch_us": round(us, 3)})
